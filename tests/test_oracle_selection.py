@@ -1,0 +1,135 @@
+"""Pins oracle.selection against the reference selector's own outputs (golden),
+torch.mean/std, and brute-force loops.  CPU only."""
+from __future__ import annotations
+
+import pytest
+import torch
+
+from conftest import load_golden
+from oracle import scoring as osc
+from oracle import selection as osel
+
+
+def _golden_raw(gold, aggregation="mean"):
+    layers, hkv, t, d = gold["keys"].shape
+    hq = gold["q_mean_complex"].shape[1]
+    g = hq // hkv
+    offs = osc.geometric_offsets(65536)
+    raw = []
+    for l in range(layers):
+        keys = gold["keys"][l].float().repeat_interleave(g, dim=0)      # selector_hf.py:308-312
+        raw.append(osc.raw_scores(keys, gold["q_mean_complex"][l], gold["q_abs_mean"][l], gold["omega"],
+                                  offs, torch.ones(hq, d // 2), int(gold["round_start"]), aggregation))
+    return raw, hkv
+
+
+CASES = {
+    "default": dict(),
+    "chunk64_prefill": dict(chunk_tokens=64, protect_prefill=True),
+    "nonorm": dict(normalize=False),
+    "aggmax": dict(),
+}
+
+
+def _sets_equal_off_ties(keep, want, fin, k):
+    """Rows must be equal as sets; where they differ, every differing index must sit
+    exactly at the k-th largest score (a tie the reference resolves arbitrarily)."""
+    for h in range(keep.shape[0]):
+        a, b = set(keep[h].tolist()), set(want[h].tolist())
+        if a == b:
+            continue
+        thr = torch.sort(fin[h], descending=True).values[k - 1]
+        for idx in a ^ b:
+            assert fin[h, idx] == thr, (h, idx, float(fin[h, idx]), float(thr))
+
+
+@pytest.mark.parametrize("tag", list(CASES))
+def test_group_selection_matches_reference(tag):
+    gold = load_golden("selector_group.pt")
+    raw, hkv = _golden_raw(gold, "max" if tag == "aggmax" else "mean")
+    kw = dict(window_size=int(gold["window"]), prefill_len=int(gold["prefill_len"]))
+    kw.update(CASES[tag])
+    keep, fin = osel.group_keep_per_head(raw, hkv, int(gold["budget"]), **kw)
+    want = gold[f"group_{tag}_keep"]
+    assert keep.shape == want.shape and keep.dtype == torch.long
+    assert bool((keep[:, 1:] > keep[:, :-1]).all())
+    _sets_equal_off_ties(keep, want, fin, int(gold["budget"]))
+    assert torch.equal(keep, want)          # no ties at the threshold in this fixture
+
+
+@pytest.mark.parametrize("tag", list(CASES))
+def test_layer_selection_matches_reference(tag):
+    gold = load_golden("selector_group.pt")
+    raw, hkv = _golden_raw(gold, "max" if tag == "aggmax" else "mean")
+    kw = dict(window_size=int(gold["window"]), prefill_len=int(gold["prefill_len"]))
+    kw.update(CASES[tag])
+    fin = osel.layer_final_scores(raw[1], hkv, **kw)
+    keep = osel.topk_ascending(fin, int(gold["budget"]))
+    want = gold[f"layer1_{tag}_keep"]
+    _sets_equal_off_ties(keep, want, fin, int(gold["budget"]))
+    assert torch.equal(keep, want)
+
+
+def test_streaming_stats_match_torch():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(6, 1000, generator=g) * 3 + 5
+    for chunk in (1000, 256, 17):
+        mean, std = osel.znorm_stats_streaming(x, chunk)
+        assert torch.allclose(mean, x.mean(-1), rtol=1e-5)
+        assert torch.allclose(std, x.std(-1), rtol=1e-4)
+    z = osel.znorm_two_pass(x)
+    assert torch.allclose(z.mean(-1), torch.zeros(6), atol=1e-5)
+    assert torch.allclose(z.std(-1), torch.ones(6), atol=1e-5)
+    const = torch.full((2, 50), 3.0)
+    assert torch.equal(osel.znorm_two_pass(const), torch.zeros(2, 50))         # std<eps -> 1
+    m, s = osel.znorm_stats_streaming(const, 50)
+    assert torch.equal(s, torch.ones(2))
+
+
+def test_guards_and_bruteforce_aggregation():
+    g = torch.Generator().manual_seed(4)
+    layers, hq, hkv, t, k = 3, 6, 2, 64, 20
+    raw = [torch.randn(hq, t, generator=g) for _ in range(layers)]
+    keep, fin = osel.group_keep_per_head(raw, hkv, k, window_size=5, prefill_len=4, protect_prefill=True)
+    must = set(range(4)) | set(range(t - 5, t))
+    for h in range(hkv):
+        assert must <= set(keep[h].tolist())
+    # brute force: python loops
+    gsz = hq // hkv
+    want = torch.zeros(hkv, t)
+    for h in range(hkv):
+        for n in range(t):
+            acc = 0.0
+            for l in range(layers):
+                best = -float("inf")
+                for a in range(h * gsz, (h + 1) * gsz):
+                    row = raw[l][a]
+                    z = (row[n] - row.mean()) / row.std()
+                    if n < 4 or n >= t - 5:
+                        z = float("inf")
+                    best = max(best, float(z))
+                acc += best
+            want[h, n] = acc / layers
+    assert torch.allclose(fin, want, rtol=1e-4, atol=1e-5)
+    # max over layers variant
+    fin_max = osel.group_final_scores(raw, hkv, window_size=0, layer_agg="max")
+    zs = torch.stack([osel.reduce_group(osel.znorm_two_pass(r), hkv) for r in raw])
+    assert torch.allclose(fin_max, zs.max(0).values, atol=1e-5)
+
+
+def test_topk_tie_rule_and_early_out():
+    s = torch.tensor([[1.0, 3.0, 3.0, 2.0, 3.0, 0.0]])
+    assert osel.topk_ascending(s, 2).tolist() == [[1, 2]]
+    assert osel.topk_ascending(s, 4).tolist() == [[1, 2, 3, 4]]
+    x = torch.randn(4, 33)
+    k = 7
+    want = torch.sort(torch.sort(x, descending=True).indices[:, :k]).values
+    assert torch.equal(osel.topk_ascending(x, k), want)
+    keep, fin = osel.group_keep_per_head([torch.randn(4, 10)], 2, 16)
+    assert fin is None and keep.tolist() == [list(range(10))] * 2
+
+
+def test_chunk_size_rule():
+    assert osel.score_chunk_tokens(16, 300, 4096) == 300
+    assert osel.score_chunk_tokens(16, 5000, 4096) == 4096
+    assert osel.score_chunk_tokens(16, 8, 4096) == 16
