@@ -1,0 +1,173 @@
+/*
+ * triattention_hip.h -- C ABI of the MI355X (gfx950) KV scoring / selection /
+ * compaction library (libtriattention_hip.so).
+ *
+ * Every entry point is stream ordered: it enqueues kernels on `stream`
+ * (a hipStream_t passed as void*, NULL = the null stream), never synchronises the
+ * device and never allocates.  All pointers are DEVICE pointers unless a comment
+ * says "host".  Return value: TRI_OK or a negative tri_status; a message for the
+ * last failure on the calling thread is available from tri_last_error().
+ * Nothing is thrown and no torch type crosses this boundary.
+ *
+ * Reference citations are paths inside the TriAttention checkout
+ * (triattention/vllm/...).
+ */
+#ifndef TRIATTENTION_HIP_H
+#define TRIATTENTION_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRI_ABI_VERSION 1
+
+typedef enum tri_status {
+  TRI_OK = 0,
+  TRI_ERR_INVALID_ARGUMENT = -1, /* shape / flag / null-pointer check failed on the host */
+  TRI_ERR_UNSUPPORTED = -2,      /* valid request this build has no kernel for */
+  TRI_ERR_WORKSPACE = -3,        /* workspace too small */
+  TRI_ERR_LAUNCH = -4            /* hipLaunchKernel reported an error */
+} tri_status;
+
+typedef enum tri_kv_dtype { TRI_KV_BF16 = 0, TRI_KV_FP16 = 1, TRI_KV_FP8_E4M3 = 2 } tri_kv_dtype;
+typedef enum tri_rope_style { TRI_ROPE_HALF = 0, TRI_ROPE_INTERLEAVED = 1 } tri_rope_style;
+typedef enum tri_reduce { TRI_REDUCE_MEAN = 0, TRI_REDUCE_MAX = 1 } tri_reduce;
+
+/* Paged (or dense) key/value storage of every layer of one KV-cache group.
+ * Element (layer l, physical block p, in-block token o, head h, dim d) of K lives at
+ *   k_layers[l] + p*stride_block + o*stride_token + h*stride_head + d   (in elements)
+ * which covers both vLLM layouts, [2, nb, bs, H, D] and [nb, 2, bs, H, D]
+ * (runtime/kv_compaction.py:38-53,94-117), by passing separate K and V bases.
+ * A dense [B, H, T, D] tensor (core/scoring.py:93) is the same thing with
+ * block_size = T, one block per sequence and an identity block table. */
+typedef struct tri_kv_layout {
+  int32_t num_layers;
+  int32_t num_kv_heads;
+  int32_t head_dim;           /* 64, 128 or 256 */
+  int32_t block_size;         /* tokens per block */
+  int32_t kv_dtype;           /* tri_kv_dtype */
+  int32_t rope_style;         /* tri_rope_style */
+  int64_t stride_block;
+  int64_t stride_token;
+  int64_t stride_head;
+  const void* const* k_layers; /* device array [num_layers] of device pointers */
+  const void* const* v_layers; /* device array [num_layers]; may be NULL for score-only calls */
+  /* fp8 only: per-(token, head) fp32 dequantisation scales, element
+   * (l, p, o, h) at k_scale_layers[l] + (p*block_size + o)*num_kv_heads + h. */
+  const float* const* k_scale_layers;
+  const float* const* v_scale_layers;
+} tri_kv_layout;
+
+/* The sequences of one compression step (the reference handles one request per
+ * call, runtime/runner_compression_actions.py:24; a batch is a loop of those). */
+typedef struct tri_batch {
+  int32_t num_seqs;
+  int32_t max_seq_len;          /* host copy of max(seq_lens): sizes grids and scratch rows */
+  int32_t max_budget;           /* host copy of max(budgets) */
+  int32_t block_table_pitch;    /* int32 elements between rows of block_table */
+  const int32_t* block_table;   /* [num_seqs][pitch] physical block ids (runtime/kv_compaction.py:139-157) */
+  const int32_t* seq_lens;      /* [num_seqs] cached tokens T (group_total_tokens, runtime/hook_group_pipeline.py:72-73) */
+  const int32_t* round_start;   /* [num_seqs] num_computed_tokens (runtime/hook_group_pipeline.py:78) */
+  const int32_t* prefill_lens;  /* [num_seqs] or NULL (=0) */
+  const int32_t* budgets;       /* [num_seqs] k = min(budget_total, T) (runtime/selector_hf.py:823) */
+} tri_batch;
+
+/* Scoring statistics, already resolved per runtime layer (layer index modulo the
+ * available stats layers, runtime/selector_hf.py:132-143) and folded by
+ * tri_fold_stats. */
+typedef struct tri_score_params {
+  int32_t num_score_heads;      /* heads scored per layer: Hq when stats are per query head, else Hkv */
+  int32_t num_offsets;          /* <= 32 */
+  int32_t aggregation;          /* tri_reduce over offsets (core/scoring.py:336-341) */
+  const float* folded;          /* [L][num_score_heads][3][F] from tri_fold_stats */
+  const float* omega;           /* [F] rotary inv_freq (core/compressor.py:192-194) */
+  const float* offsets;         /* [num_offsets] (core/compressor.py:222-242) */
+} tri_score_params;
+
+/* Selection semantics (runtime/selector_hf.py:813-1033 and :473-677). */
+typedef struct tri_select_params {
+  int32_t normalize;            /* sparse_normalize_scores */
+  int32_t window_size;          /* recent tokens forced to +inf (runtime/selector_hf.py:121-130) */
+  int32_t protect_prefill;      /* tokens < prefill_len forced to +inf */
+  int32_t group_reduce;         /* tri_reduce over the query heads of a KV head (runtime/selector_hf.py:277-297) */
+  int32_t layer_reduce;         /* tri_reduce over layers; -1 = none (one keep set per layer) */
+  int32_t shared;               /* 1: max over KV heads, one index list per (seq[, layer]) (runtime/selector_hf.py:636-637) */
+} tri_select_params;
+
+int tri_abi_version(void);
+const char* tri_last_error(void);
+
+/* Replaces the per-call stat preparation of core/scoring.py:259-271,346-351:
+ * folded[l][a][0][f] = s*q_r, [1] = s*q_i, [2] = s*(q_abs - sqrt(q_r^2+q_i^2+1e-8))
+ * (s*q_abs when disable_mlr; [0]=[1]=0 when disable_trig).  Inputs [L][A][F] fp32. */
+int tri_fold_stats(const float* q_mean_real, const float* q_mean_imag, const float* q_abs_mean,
+                   const float* freq_scale_sq, int32_t num_layers, int32_t num_score_heads,
+                   int32_t num_pairs, int32_t disable_mlr, int32_t disable_trig, float* folded,
+                   void* stream);
+
+/* Bytes of device scratch the calls below need for (layout, batch, score params);
+ * 0 on invalid input.  Host-only, launches nothing. */
+uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
+                             const tri_score_params* sp);
+
+/* Raw scores of every cached key of every sequence and layer, straight from the
+ * paged blocks; replaces gather_request_k_dense_range + repeat_interleave +
+ * compute_scores_triton per (layer, chunk) (runtime/selector_hf.py:860-894,
+ * runtime/kv_compaction.py:322-352, core/scoring.py:79-204; math of
+ * core/scoring.py:207-362).  raw[(b*L + l)*raw_stride_layer + n*raw_stride_token
+ * + a*raw_stride_head], fp32.  Also leaves per-(seq, layer, head) sum / sum of
+ * squares partials in the workspace for tri_select. */
+int tri_score_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                    float* raw, int64_t raw_stride_layer, int64_t raw_stride_token,
+                    int64_t raw_stride_head, void* workspace, uint64_t workspace_bytes,
+                    void* stream);
+
+/* z-normalise, guard, reduce over the GQA group and over layers, then keep the
+ * top budget per row, ascending; replaces runtime/selector_hf.py:896-1025 (group
+ * mode) and :538-677 (per-layer modes).  `raw` and the workspace come from
+ * tri_score_paged on the same stream.  final_scores (may be NULL) receives the
+ * selection scores [rows][max_seq_len]; keep receives int32
+ * [rows][max_budget], rows = B * (layer_reduce<0 ? L : 1) * (shared ? 1 : Hkv).
+ * Ties at the threshold keep the lowest token index. */
+int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+               const tri_select_params* sel, const float* raw, int64_t raw_stride_layer,
+               int64_t raw_stride_token, int64_t raw_stride_head, float* final_scores,
+               int32_t* keep, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* Top-k of arbitrary fp32 rows (core/compressor.py:388-409): keep[r][0..k_r) =
+ * ascending indices of the k_r largest of scores[r][0..len_r). */
+int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,
+                  const int32_t* row_ks, int32_t rows_per_entry, int32_t max_len, int32_t* keep,
+                  int32_t keep_pitch, void* stream);
+
+/* In-place, order-preserving compaction of K and V of every layer: slot j of
+ * (seq b, head h) receives the row of token keep[...][j], for j < budget_b;
+ * replaces compact_request_kv_in_place(_per_head) per layer
+ * (runtime/kv_compaction.py:355-599, runtime/layout_engine.py:112-138) for the
+ * slots that survive truncate_tail_reclaim_group (runtime/layout_engine.py:209-227).
+ * keep rows must be strictly ascending.  keep_per_layer: keep is
+ * [B][L][rows][max_budget] instead of [B][rows][max_budget]; shared: rows = 1. */
+int tri_compact_paged(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep,
+                      int32_t keep_per_layer, int32_t shared, void* stream);
+
+/* The reference's full permutation [kept..., dropped...] over all T slots
+ * (runtime/kv_compaction.py:512-546), through a caller-provided staging buffer of
+ * tri_compact_full_staging_bytes(). */
+uint64_t tri_compact_full_staging_bytes(const tri_kv_layout* kv, const tri_batch* batch);
+int tri_compact_paged_full(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep,
+                           int32_t keep_per_layer, int32_t shared, void* staging,
+                           uint64_t staging_bytes, void* stream);
+
+/* score + select + compact for every layer of every sequence in one call: the
+ * device side of run_group_compaction_pipeline (runtime/hook_group_pipeline.py:42-155)
+ * in the default per_head / hf_aligned_global_per_head mode. */
+int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                      const tri_select_params* sel, int32_t* keep, void* workspace,
+                      uint64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIATTENTION_HIP_H */

@@ -1,0 +1,68 @@
+"""Test helpers: run the oracle end to end on a synthetic workload (CPU) and push the
+same inputs through the HIP path."""
+from __future__ import annotations
+
+import torch
+
+from oracle import compaction as ocp
+from oracle import scoring as osc
+from oracle import selection as osel
+from triattention_amd import ops, synth
+
+
+def build_inputs(w: synth.Workload, kv_axis: int = 0):
+    """CPU-generated, seeded inputs of a workload."""
+    tables = synth.make_block_tables(w)
+    caches = synth.make_kv_pool(w, tables, "cpu", kv_axis)
+    qc, qa = synth.make_stats(w, "cpu")
+    omega = synth.rope_inv_freq(w)
+    offsets = synth.geometric_offsets()
+    fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2)
+    return dict(tables=tables, caches=caches, qc=qc, qa=qa, omega=omega, offsets=offsets, fs=fs, kv_axis=kv_axis)
+
+
+def oracle_raw(w, inp, b, round_start, aggregation="mean", disable_mlr=False, disable_trig=False):
+    """Raw scores [L][Hq, T_b] of sequence b from the oracle."""
+    g = w.num_q_heads // w.num_kv_heads
+    out = []
+    for l in range(w.num_layers):
+        kc, _ = ocp.split_kv(inp["caches"][l], inp["kv_axis"])
+        keys = ocp.gather_dense(kc, inp["tables"][b], w.block_size, 0, w.seq_lens[b])[0]      # [Hkv, T, D]
+        keys = keys.float().repeat_interleave(g, dim=0)
+        out.append(osc.raw_scores(keys, inp["qc"][l], inp["qa"][l], inp["omega"], inp["offsets"], inp["fs"][l],
+                                  round_start, aggregation, w.rope_style, disable_mlr, disable_trig))
+    return out
+
+
+def device_objects(w, inp, device, round_start=None, budgets=None, prefill_lens=None, aggregation="mean",
+                   disable_mlr=False, disable_trig=False):
+    caches = [c.to(device) for c in inp["caches"]]
+    kv = ops.PagedKV.from_kv_caches(caches, w.rope_style, kv_axis=inp["kv_axis"])
+    batch = ops.StepBatch(device, w.seq_lens, round_start=round_start,
+                          budgets=budgets if budgets is not None else w.budget,
+                          block_tables=inp["tables"], prefill_lens=prefill_lens)
+    folded = ops.fold_stats(inp["qc"].to(device), inp["qa"].to(device), inp["fs"].to(device),
+                            disable_mlr, disable_trig)
+    sc = ops.ScoreConfig(folded, inp["omega"].to(device), inp["offsets"].to(device), aggregation)
+    return caches, kv, batch, sc
+
+
+def score_tolerance(ref: torch.Tensor):
+    """1e-3 relative, taken against the per-head RMS of the score (raw scores cross zero)."""
+    return 1e-3 * ref.pow(2).mean(dim=-1, keepdim=True).sqrt()
+
+
+def assert_keep_matches(keep: torch.Tensor, want: torch.Tensor, fin: torch.Tensor, k: int, tie_tol: float):
+    """Kept sets equal, except indices whose oracle score is within tie_tol of the
+    k-th largest oracle score (fp32 rounding of a different summation order can swap
+    those).  Returns the number of swapped indices."""
+    swapped = 0
+    for h in range(want.shape[0]):
+        a, b = set(keep[h].tolist()), set(want[h].tolist())
+        if a == b:
+            continue
+        thr = torch.sort(fin[h], descending=True).values[k - 1]
+        for idx in a ^ b:
+            assert abs(float(fin[h, idx]) - float(thr)) <= tie_tol, (h, idx, float(fin[h, idx]), float(thr))
+            swapped += 1
+    return swapped

@@ -1,0 +1,380 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle and with the
+reference's own outputs (golden fixtures).  All tests need an MI355X."""
+from __future__ import annotations
+
+import pytest
+import torch
+
+from conftest import load_golden
+from helpers import assert_keep_matches, build_inputs, device_objects, oracle_raw, score_tolerance
+from oracle import compaction as ocp
+from oracle import scoring as osc
+from oracle import selection as osel
+from triattention_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def small(**kw):
+    base = dict(name="t", num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128, seq_lens=(300,),
+                budget=96, block_size=16, window_size=12, rope_theta=1e6, index=7)
+    base.update(kw)
+    return synth.Workload(**base)
+
+
+def run_scores(w, inp, aggregation="mean", round_start=None, **flags):
+    caches, kv, batch, sc = device_objects(w, inp, DEV, round_start=round_start, aggregation=aggregation, **flags)
+    raw, ws = ops.score_paged(kv, batch, sc)
+    torch.cuda.synchronize()
+    return raw.cpu(), (caches, kv, batch, sc, ws)
+
+
+SCORE_CASES = {
+    "c0": dict(w=synth.config(0)),
+    "gqa4_two_layers": dict(w=small()),
+    "ragged_batch": dict(w=small(seq_lens=(300, 17, 1000, 256, 513), num_layers=3)),
+    "hkv8": dict(w=small(num_q_heads=32, num_kv_heads=8, seq_lens=(700, 90))),
+    "hkv4_g7": dict(w=small(num_q_heads=28, num_kv_heads=4, seq_lens=(333,))),
+    "g8": dict(w=small(num_q_heads=64, num_kv_heads=8, seq_lens=(260,))),
+    "g1": dict(w=small(num_q_heads=2, num_kv_heads=2, seq_lens=(129,))),
+    "hkv1": dict(w=small(num_q_heads=4, num_kv_heads=1, seq_lens=(200,))),
+    "hkv16": dict(w=small(num_q_heads=16, num_kv_heads=16, seq_lens=(150,))),
+    "d64": dict(w=small(head_dim=64, num_q_heads=16, num_kv_heads=8, seq_lens=(270,))),
+    "d256": dict(w=small(head_dim=256, seq_lens=(140,))),
+    "interleaved": dict(w=small(rope_style="interleaved")),
+    "fp16": dict(w=small(kv_dtype="fp16")),
+    "block32": dict(w=small(block_size=32, seq_lens=(500, 31))),
+    "block_not_pow2": dict(w=small(block_size=24, seq_lens=(301,))),
+    "kv_axis1": dict(w=small(seq_lens=(290, 64)), kv_axis=1),
+    "llama3": dict(w=small(rope_theta=5e5, rope_scaling="llama3")),
+    "max_agg": dict(w=small(seq_lens=(300, 40)), aggregation="max"),
+    "max_agg_d64": dict(w=small(head_dim=64, seq_lens=(100,)), aggregation="max"),
+    "no_mlr": dict(w=small(), disable_mlr=True),
+    "no_trig": dict(w=small(), disable_trig=True),
+    "no_trig_max": dict(w=small(), disable_trig=True, aggregation="max"),
+    "late_round": dict(w=small(), round_start=[70000]),
+}
+
+
+@pytest.mark.parametrize("name", list(SCORE_CASES))
+def test_raw_scores_match_oracle(name):
+    case = dict(SCORE_CASES[name])
+    w = case.pop("w")
+    kv_axis = case.pop("kv_axis", 0)
+    agg = case.pop("aggregation", "mean")
+    rs = case.pop("round_start", None)
+    inp = build_inputs(w, kv_axis)
+    print(f"case={name} workload={w}", flush=True)
+    raw, _ = run_scores(w, inp, agg, rs, **case)
+    for b, t in enumerate(w.seq_lens):
+        rstart = rs[b] if rs is not None else t
+        want = oracle_raw(w, inp, b, rstart, agg, **case)
+        for l in range(w.num_layers):
+            got = raw[b, l, :t].transpose(0, 1)                  # [A, T]
+            err = (got - want[l]).abs()
+            tol = score_tolerance(want[l])                        # 1e-3 relative to per-head RMS
+            assert bool((err <= tol).all()), (name, b, l, float(err.max()), float(tol.min()))
+
+
+def test_head_major_output_layout():
+    w = small(seq_lens=(200, 77))
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    a, ws = ops.score_paged(kv, batch, sc)
+    b, _ = ops.score_paged(kv, batch, sc, ws, head_major=True)
+    torch.cuda.synchronize()
+    for i, t in enumerate(w.seq_lens):
+        assert torch.equal(a[i, :, :t].transpose(1, 2), b[i, :, :, :t])
+
+
+def test_dense_keys_entry():
+    """[B, H, T, D] keys without a block table (core/scoring.py:79-204 call shape)."""
+    g = torch.Generator().manual_seed(3)
+    b, h, t, d = 2, 4, 150, 128
+    keys = torch.randn(b, h, t, d, generator=g).to(torch.bfloat16)
+    qc = torch.randn(1, h, d // 2, 2, generator=g)
+    qa = qc.pow(2).sum(-1).sqrt() + torch.rand(1, h, d // 2, generator=g)
+    fs = 0.5 + torch.rand(1, h, d // 2, generator=g)
+    omega = synth.rope_inv_freq(small())
+    offs = synth.geometric_offsets()
+    kd = keys.to(DEV)
+    kv = ops.PagedKV.from_dense_keys(kd)
+    batch = ops.StepBatch(DEV, [t, t], round_start=[500, 500])
+    sc = ops.ScoreConfig(ops.fold_stats(qc.to(DEV), qa.to(DEV), fs.to(DEV)), omega.to(DEV), offs.to(DEV))
+    raw, _ = ops.score_paged(kv, batch, sc, head_major=True)
+    torch.cuda.synchronize()
+    want = osc.raw_scores(keys, qc[0], qa[0], omega, offs, fs[0], 500)
+    got = raw[:, 0].cpu()
+    assert bool(((got - want).abs() <= score_tolerance(want)).all())
+
+
+SELECT_CASES = {
+    "default": dict(w=small(seq_lens=(300, 1000, 97))),
+    "c0": dict(w=synth.config(0)),
+    "prefill": dict(w=small(seq_lens=(400, 222)), prefill=[30, 5], protect_prefill=True),
+    "nonorm": dict(w=small(seq_lens=(300,)), normalize=False),
+    "layer_max": dict(w=small(seq_lens=(300,), num_layers=3), layer_reduce="max"),
+    "under_budget": dict(w=small(seq_lens=(50, 96, 97))),
+    "no_window": dict(w=small(seq_lens=(300,), window_size=0)),
+    "hkv8": dict(w=small(num_q_heads=32, num_kv_heads=8, seq_lens=(700,), budget=256)),
+    "g7": dict(w=small(num_q_heads=28, num_kv_heads=4, seq_lens=(333,))),
+}
+
+
+@pytest.mark.parametrize("name", list(SELECT_CASES))
+def test_group_selection_matches_oracle(name):
+    case = dict(SELECT_CASES[name])
+    w = case.pop("w")
+    prefill = case.pop("prefill", None)
+    protect = case.pop("protect_prefill", False)
+    normalize = case.pop("normalize", True)
+    layer_reduce = case.pop("layer_reduce", "mean")
+    inp = build_inputs(w)
+    print(f"case={name} workload={w}", flush=True)
+    caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=prefill)
+    raw, ws = ops.score_paged(kv, batch, sc)
+    sel = ops.SelectConfig(normalize=normalize, window_size=w.window_size, protect_prefill=protect,
+                           layer_reduce=layer_reduce)
+    keep, fin = ops.select(kv, batch, sc, sel, raw, ws, want_scores=True)
+    torch.cuda.synchronize()
+    keep, fin = keep.cpu(), fin.cpu()
+    h = w.num_kv_heads
+    total_swapped = 0
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        oraw = oracle_raw(w, inp, b, t)
+        want, ofin = osel.group_keep_per_head(
+            oraw, h, w.budget, normalize=normalize, window_size=w.window_size,
+            prefill_len=prefill[b] if prefill else 0, protect_prefill=protect,
+            chunk_tokens=osel.score_chunk_tokens(w.block_size, t), layer_agg=layer_reduce)
+        got = keep[b * h:(b + 1) * h, :k].long()
+        assert bool((got[:, 1:] > got[:, :-1]).all())            # strictly ascending
+        if ofin is None:
+            assert torch.equal(got, want)
+            continue
+        dfin = fin[b * h:(b + 1) * h, :t]
+        finite = torch.isfinite(ofin)
+        assert torch.equal(torch.isfinite(dfin), finite)
+        scale = ofin[finite].abs().max()
+        assert float((dfin[finite] - ofin[finite]).abs().max()) <= 2e-3 * float(scale)
+        total_swapped += assert_keep_matches(got, want, ofin, k, tie_tol=2e-3 * float(scale))
+    print("swapped near-tie indices:", total_swapped, flush=True)
+
+
+@pytest.mark.parametrize("tag,kw", [
+    ("default", dict()),
+    ("chunk64_prefill", dict(protect_prefill=True)),
+    ("nonorm", dict(normalize=False)),
+    ("aggmax", dict(aggregation="max")),
+])
+def test_group_selection_matches_reference_golden(tag, kw):
+    """Keep sets written by the reference's own selector (paged group branch)."""
+    gold = load_golden("selector_group.pt")
+    layers, hkv, t, d = gold["keys"].shape
+    hq = gold["q_mean_complex"].shape[1]
+    bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])
+    ids = gold["block_ids"].tolist()
+    caches = []
+    for l in range(layers):
+        kvc = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
+        tok = torch.arange(t)
+        blk = torch.tensor(ids)[tok // bs]
+        kvc[0, blk, tok % bs] = gold["keys"][l].transpose(0, 1)
+        kvc[1, blk, tok % bs] = gold["values"][l].transpose(0, 1)
+        caches.append(kvc.to(DEV))
+    kv = ops.PagedKV.from_kv_caches(caches)
+    budget = int(gold["budget"])
+    batch = ops.StepBatch(DEV, [t], round_start=[int(gold["round_start"])], budgets=budget,
+                          block_tables=[ids], prefill_lens=[int(gold["prefill_len"])])
+    folded = ops.fold_stats(gold["q_mean_complex"].to(DEV), gold["q_abs_mean"].to(DEV),
+                            torch.ones(layers, hq, d // 2, device=DEV))
+    sc = ops.ScoreConfig(folded, gold["omega"].to(DEV), synth.geometric_offsets(device=DEV),
+                         kw.get("aggregation", "mean"))
+    sel = ops.SelectConfig(normalize=kw.get("normalize", True), window_size=int(gold["window"]),
+                           protect_prefill=kw.get("protect_prefill", False))
+    raw, ws = ops.score_paged(kv, batch, sc)
+    keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+    torch.cuda.synchronize()
+    want = gold[f"group_{tag}_keep"]
+    got = keep.cpu().long()
+    diff = sum(len(set(got[h].tolist()) ^ set(want[h].tolist())) for h in range(hkv))
+    assert diff == 0, f"{diff} indices differ from the reference's keep set"
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("tag,kw", [("default", dict()), ("nonorm", dict(normalize=False))])
+def test_layer_selection_matches_reference_golden(tag, kw):
+    """Per-layer selection (runtime/selector_hf.py:473-677) against the reference's output for layer 1."""
+    gold = load_golden("selector_group.pt")
+    layers, hkv, t, d = gold["keys"].shape
+    hq = gold["q_mean_complex"].shape[1]
+    bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])
+    ids = gold["block_ids"].tolist()
+    caches = []
+    for l in range(layers):
+        kvc = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
+        tok = torch.arange(t)
+        blk = torch.tensor(ids)[tok // bs]
+        kvc[0, blk, tok % bs] = gold["keys"][l].transpose(0, 1)
+        caches.append(kvc.to(DEV))
+    kv = ops.PagedKV.from_kv_caches(caches)
+    batch = ops.StepBatch(DEV, [t], round_start=[int(gold["round_start"])], budgets=int(gold["budget"]),
+                          block_tables=[ids], prefill_lens=[int(gold["prefill_len"])])
+    folded = ops.fold_stats(gold["q_mean_complex"].to(DEV), gold["q_abs_mean"].to(DEV),
+                            torch.ones(layers, hq, d // 2, device=DEV))
+    sc = ops.ScoreConfig(folded, gold["omega"].to(DEV), synth.geometric_offsets(device=DEV))
+    sel = ops.SelectConfig(normalize=kw.get("normalize", True), window_size=int(gold["window"]), layer_reduce=None)
+    raw, ws = ops.score_paged(kv, batch, sc)
+    keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+    torch.cuda.synchronize()
+    got = keep.cpu().long().view(layers, hkv, -1)[1]
+    assert torch.equal(got, gold[f"layer1_{tag}_keep"])
+
+
+def test_topk_rows_ties_and_order():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(5, 3000, generator=g)
+    x[1, 100:400] = 0.5                       # a large tie class straddling the threshold
+    x[2, :] = 1.0                             # everything ties
+    x[3, -50:] = float("inf")
+    x[4, ::7] = float("-inf")
+    for k in (1, 17, 256, 2999, 3000):
+        got = ops.topk_rows(x.to(DEV), k).cpu().long()
+        want = osel.topk_ascending(x, k)
+        assert torch.equal(got[:, :k], want), k
+    lens = [3000, 10, 1, 2048, 777]
+    ks = [5, 20, 1, 2048, 0]
+    got = ops.topk_rows(x.to(DEV), ks, lens).cpu().long()
+    for r, (n, k) in enumerate(zip(lens, ks)):
+        kk = min(k, n)
+        if kk:
+            assert torch.equal(got[r, :kk], osel.topk_ascending(x[r:r + 1, :n], kk)[0])
+
+
+def _compact_case(w, kv_axis, shared, per_layer, full):
+    inp = build_inputs(w, kv_axis)
+    caches = [c.to(DEV) for c in inp["caches"]]
+    kv = ops.PagedKV.from_kv_caches(caches, kv_axis=kv_axis)
+    batch = ops.StepBatch(DEV, w.seq_lens, budgets=w.budget, block_tables=inp["tables"])
+    g = torch.Generator().manual_seed(99)
+    rows_per = (w.num_layers if per_layer else 1) * (1 if shared else w.num_kv_heads)
+    keep = torch.zeros(w.num_seqs * rows_per, batch.max_budget, dtype=torch.int32)
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        for r in range(rows_per):
+            keep[b * rows_per + r, :k] = torch.sort(torch.randperm(t, generator=g)[:k]).values.int()
+    before = [c.clone() for c in inp["caches"]]
+    ops.compact(kv, batch, keep.to(DEV), keep_per_layer=per_layer, shared=shared, full_permutation=full)
+    torch.cuda.synchronize()
+    for l in range(w.num_layers):
+        want = before[l].clone()
+        for b, t in enumerate(w.seq_lens):
+            k = min(w.budget, t)
+            base = b * rows_per + (l * (1 if shared else w.num_kv_heads) if per_layer else 0)
+            if shared:
+                ocp.compact_shared(want, inp["tables"][b], w.block_size, keep[base, :k].long(), t,
+                                   kv_axis=kv_axis, full_permutation=full)
+            else:
+                ocp.compact_per_head(want, inp["tables"][b], w.block_size,
+                                     keep[base:base + w.num_kv_heads, :k].long(), t,
+                                     kv_axis=kv_axis, full_permutation=full)
+        got = caches[l].cpu()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (l,)
+
+
+@pytest.mark.parametrize("kv_axis", [0, 1])
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("per_layer", [False, True])
+@pytest.mark.parametrize("full", [False, True])
+def test_compaction_bit_exact(kv_axis, shared, per_layer, full):
+    w = small(seq_lens=(300, 97, 40, 1234), num_layers=2, num_q_heads=8, num_kv_heads=4, budget=96)
+    print(f"compact kv_axis={kv_axis} shared={shared} per_layer={per_layer} full={full}", flush=True)
+    _compact_case(w, kv_axis, shared, per_layer, full)
+
+
+def test_compaction_large_budget_and_dims():
+    _compact_case(small(seq_lens=(5000,), budget=3000, num_kv_heads=8, num_q_heads=8), 0, False, False, False)
+    _compact_case(small(seq_lens=(700,), budget=300, head_dim=64, block_size=32), 0, False, False, False)
+    _compact_case(small(seq_lens=(700,), budget=300, head_dim=256, block_size=8), 0, True, False, False)
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_compaction_matches_reference_golden(axis):
+    """Full-permutation output written by the reference's compact_request_kv_in_place(_per_head)."""
+    g = load_golden("compaction.pt")[f"axis{axis}"]
+    bs, t = int(g["block_size"]), int(g["total_tokens"])
+    for mode, keep_key, after_key in (("per_head", "keep_per_head", "kv_after_per_head"),
+                                      ("shared", "keep_shared", "kv_after_shared")):
+        # head_dim 16 is below the kernels' 64: widen rows by viewing 4 tokens... not
+        # possible in place, so this fixture is replayed with head_dim padded to 64.
+        before = g["kv_before"]
+        pad = torch.zeros(*before.shape[:-1], 64, dtype=before.dtype)
+        pad[..., :16] = before
+        cache = pad.to(DEV)
+        kv = ops.PagedKV.from_kv_caches([cache], kv_axis=axis)
+        keep = g[keep_key].int()
+        keep = keep if keep.ndim == 2 else keep.unsqueeze(0)
+        batch = ops.StepBatch(DEV, [t], budgets=int(keep.shape[1]), block_tables=[g["block_ids"].tolist()])
+        ops.compact(kv, batch, keep.contiguous().to(DEV), shared=(mode == "shared"), full_permutation=True)
+        torch.cuda.synchronize()
+        got = cache.cpu()[..., :16]
+        assert torch.equal(got.view(torch.int16), g[after_key].view(torch.int16)), mode
+
+
+def test_compress_step_equals_chained_calls():
+    w = small(seq_lens=(300, 1000, 97, 50), num_layers=3, num_q_heads=16, num_kv_heads=4)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    raw, ws = ops.score_paged(kv, batch, sc)
+    keep_a, _ = ops.select(kv, batch, sc, sel, raw, ws)
+    ops.compact(kv, batch, keep_a)
+    torch.cuda.synchronize()
+    chained = [c.clone() for c in caches]
+    caches2, kv2, batch2, sc2 = device_objects(w, inp, DEV)
+    keep_b, _ = ops.compress_step(kv2, batch2, sc2, sel)
+    torch.cuda.synchronize()
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        rows = slice(b * w.num_kv_heads, (b + 1) * w.num_kv_heads)
+        assert torch.equal(keep_a[rows, :k], keep_b[rows, :k])
+    for a, b in zip(chained, caches2):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_end_to_end_c0_against_oracle():
+    """BASELINE config 0: score, select at budget 2048, compact; kept K/V bit-exact."""
+    w = synth.config(0)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    keep, _ = ops.compress_step(kv, batch, sc, sel)
+    torch.cuda.synchronize()
+    t, k, h = w.seq_lens[0], w.budget, w.num_kv_heads
+    oraw = oracle_raw(w, inp, 0, t)
+    want, ofin = osel.group_keep_per_head(oraw, h, k, window_size=w.window_size,
+                                          chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
+    got = keep.cpu().long()
+    scale = float(ofin[torch.isfinite(ofin)].abs().max())
+    swapped = assert_keep_matches(got, want, ofin, k, tie_tol=2e-3 * scale)
+    print("c0 swapped near-tie indices:", swapped, "of", h * k, flush=True)
+    # compaction is bit-exact given the device's own keep set
+    ref = inp["caches"][0].clone()
+    ocp.compact_per_head(ref, inp["tables"][0], w.block_size, got, t, full_permutation=False)
+    blk, off = ocp.token_slots(inp["tables"][0], w.block_size, torch.arange(k))
+    dev = caches[0].cpu()
+    assert torch.equal(dev[:, blk, off].view(torch.int16), ref[:, blk, off].view(torch.int16))
+
+
+def test_invalid_arguments_raise():
+    w = small()
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    with pytest.raises(IndexError):
+        bad = ops.StepBatch(DEV, [5000], budgets=96, block_tables=inp["tables"])
+        ops.score_paged(kv, bad, sc)
+    with pytest.raises(ValueError):
+        ops.compact(kv, batch, torch.zeros(3, 5, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError):
+        ops.PagedKV.from_kv_caches([c.cpu() for c in caches])

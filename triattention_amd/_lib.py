@@ -1,0 +1,114 @@
+"""ctypes binding of libtriattention_hip.so (the C ABI in include/triattention_hip.h).
+
+There is no fallback: if the shared library is missing, ``load()`` raises, and so
+does every operator that needs it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libtriattention_hip.so"
+
+TRI_OK = 0
+TRI_ERR_INVALID_ARGUMENT = -1
+TRI_ERR_UNSUPPORTED = -2
+TRI_ERR_WORKSPACE = -3
+TRI_ERR_LAUNCH = -4
+
+KV_BF16, KV_FP16, KV_FP8_E4M3 = 0, 1, 2
+ROPE_HALF, ROPE_INTERLEAVED = 0, 1
+REDUCE_MEAN, REDUCE_MAX, REDUCE_NONE = 0, 1, -1
+
+EXPORTS = (
+    "tri_abi_version", "tri_last_error", "tri_fold_stats", "tri_workspace_bytes", "tri_score_paged",
+    "tri_select", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
+    "tri_compact_paged_full", "tri_compress_step",
+)
+
+
+class KvLayout(C.Structure):
+    _fields_ = [
+        ("num_layers", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("block_size", C.c_int32), ("kv_dtype", C.c_int32), ("rope_style", C.c_int32),
+        ("stride_block", C.c_int64), ("stride_token", C.c_int64), ("stride_head", C.c_int64),
+        ("k_layers", C.c_void_p), ("v_layers", C.c_void_p),
+        ("k_scale_layers", C.c_void_p), ("v_scale_layers", C.c_void_p),
+    ]
+
+
+class Batch(C.Structure):
+    _fields_ = [
+        ("num_seqs", C.c_int32), ("max_seq_len", C.c_int32), ("max_budget", C.c_int32),
+        ("block_table_pitch", C.c_int32),
+        ("block_table", C.c_void_p), ("seq_lens", C.c_void_p), ("round_start", C.c_void_p),
+        ("prefill_lens", C.c_void_p), ("budgets", C.c_void_p),
+    ]
+
+
+class ScoreParams(C.Structure):
+    _fields_ = [
+        ("num_score_heads", C.c_int32), ("num_offsets", C.c_int32), ("aggregation", C.c_int32),
+        ("folded", C.c_void_p), ("omega", C.c_void_p), ("offsets", C.c_void_p),
+    ]
+
+
+class SelectParams(C.Structure):
+    _fields_ = [
+        ("normalize", C.c_int32), ("window_size", C.c_int32), ("protect_prefill", C.c_int32),
+        ("group_reduce", C.c_int32), ("layer_reduce", C.c_int32), ("shared", C.c_int32),
+    ]
+
+
+class TriError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libtriattention_hip error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m triattention_amd.build` "
+            "(hipcc, gfx950). There is no CPU or PyTorch fallback for this path.")
+    lib = C.CDLL(str(LIB_PATH))
+    P, I32, I64, U64 = C.c_void_p, C.c_int32, C.c_int64, C.c_uint64
+    lib.tri_abi_version.restype = C.c_int
+    lib.tri_last_error.restype = C.c_char_p
+    lib.tri_fold_stats.argtypes = [P, P, P, P, I32, I32, I32, I32, I32, P, P]
+    lib.tri_workspace_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams)]
+    lib.tri_workspace_bytes.restype = U64
+    lib.tri_score_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                    P, I64, I64, I64, P, U64, P]
+    lib.tri_select.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                               C.POINTER(SelectParams), P, I64, I64, I64, P, P, P, U64, P]
+    lib.tri_topk_rows.argtypes = [P, I64, I32, P, P, I32, I32, P, I32, P]
+    lib.tri_compact_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), P, I32, I32, P]
+    lib.tri_compact_full_staging_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch)]
+    lib.tri_compact_full_staging_bytes.restype = U64
+    lib.tri_compact_paged_full.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), P, I32, I32, P, U64, P]
+    lib.tri_compress_step.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                      C.POINTER(SelectParams), P, P, U64, P]
+    for name in EXPORTS:
+        fn = getattr(lib, name)
+        if fn.restype is C.c_int and name not in ("tri_abi_version",):
+            fn.restype = C.c_int
+    if lib.tri_abi_version() != 1:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 1; rebuild the library")
+    _lib = lib
+    return lib
+
+
+def check(code: int) -> None:
+    """Map a tri_status to a Python exception."""
+    if code == TRI_OK:
+        return
+    msg = load().tri_last_error().decode("utf-8", "replace")
+    raise TriError(code, msg)

@@ -1,0 +1,315 @@
+// extern "C" boundary of libtriattention_hip.so: argument validation on the host,
+// then kernel launches on the caller's stream.  Nothing here allocates or waits.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "tri_common.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int launch_status(hipError_t e, const char* what) {
+  if (e == hipSuccess) return TRI_OK;
+  return fail(TRI_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int elem_bytes(int dt) { return dt == TRI_KV_FP8_E4M3 ? 1 : 2; }
+
+int check_layout(const tri_kv_layout* kv, bool need_v) {
+  if (!kv) return fail(TRI_ERR_INVALID_ARGUMENT, "kv layout is NULL");
+  if (kv->num_layers <= 0 || kv->num_kv_heads <= 0 || kv->num_kv_heads > 256)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "bad layer/head count (%d, %d)", kv->num_layers, kv->num_kv_heads);
+  if (kv->head_dim != 64 && kv->head_dim != 128 && kv->head_dim != 256)
+    return fail(TRI_ERR_UNSUPPORTED, "head_dim %d not in {64,128,256}", kv->head_dim);
+  if (kv->block_size <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "block_size %d", kv->block_size);
+  if (kv->kv_dtype != TRI_KV_BF16 && kv->kv_dtype != TRI_KV_FP16 && kv->kv_dtype != TRI_KV_FP8_E4M3)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "kv_dtype %d", kv->kv_dtype);
+  if (kv->rope_style != TRI_ROPE_HALF && kv->rope_style != TRI_ROPE_INTERLEAVED)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "rope_style %d", kv->rope_style);
+  const int eb = elem_bytes(kv->kv_dtype);
+  const int64_t per16 = 16 / eb;   // elements per 16-byte access
+  if (kv->stride_block % per16 || kv->stride_token % per16 || kv->stride_head % per16)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "strides must be multiples of %lld elements (16 bytes)", (long long)per16);
+  if (kv->stride_head < kv->head_dim && kv->num_kv_heads > 1)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "stride_head %lld < head_dim", (long long)kv->stride_head);
+  if (!kv->k_layers) return fail(TRI_ERR_INVALID_ARGUMENT, "k_layers is NULL");
+  if (need_v && !kv->v_layers) return fail(TRI_ERR_INVALID_ARGUMENT, "v_layers is NULL");
+  if (kv->kv_dtype == TRI_KV_FP8_E4M3 && !kv->k_scale_layers)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "fp8 cache without k_scale_layers");
+  if (kv->kv_dtype == TRI_KV_FP8_E4M3 && need_v && !kv->v_scale_layers)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "fp8 cache without v_scale_layers");
+  return TRI_OK;
+}
+
+int check_batch(const tri_batch* b, bool need_budget) {
+  if (!b) return fail(TRI_ERR_INVALID_ARGUMENT, "batch is NULL");
+  if (b->num_seqs <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "num_seqs %d", b->num_seqs);
+  if (b->max_seq_len <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "max_seq_len %d", b->max_seq_len);
+  if (!b->seq_lens) return fail(TRI_ERR_INVALID_ARGUMENT, "seq_lens is NULL");
+  if (b->block_table && b->block_table_pitch <= 0)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "block_table_pitch %d", b->block_table_pitch);
+  if (need_budget) {
+    if (!b->budgets) return fail(TRI_ERR_INVALID_ARGUMENT, "budgets is NULL");
+    if (b->max_budget <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "max_budget %d", b->max_budget);
+  }
+  return TRI_OK;
+}
+
+int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
+  if (!sp) return fail(TRI_ERR_INVALID_ARGUMENT, "score params are NULL");
+  if (sp->num_score_heads <= 0 || sp->num_score_heads % kv->num_kv_heads)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "num_score_heads %d is not a multiple of num_kv_heads %d",
+                sp->num_score_heads, kv->num_kv_heads);
+  if (sp->num_offsets <= 0 || sp->num_offsets > tri::kMaxOffsets)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "num_offsets %d not in [1, %d]", sp->num_offsets, tri::kMaxOffsets);
+  if (sp->aggregation != TRI_REDUCE_MEAN && sp->aggregation != TRI_REDUCE_MAX)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "aggregation %d", sp->aggregation);
+  if (!sp->folded || !sp->omega || !sp->offsets)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "folded / omega / offsets is NULL");
+  if (!is_aligned(sp->folded, 16)) return fail(TRI_ERR_INVALID_ARGUMENT, "folded must be 16-byte aligned");
+  return TRI_OK;
+}
+
+tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
+  return tri::plan_workspace(b->num_seqs, kv->num_layers, sp->num_score_heads, kv->head_dim / 2, sp->num_offsets,
+                             kv->num_kv_heads, b->max_seq_len);
+}
+
+int check_workspace(const tri::Workspace& w, void* ws, uint64_t bytes) {
+  if (!ws) return fail(TRI_ERR_WORKSPACE, "workspace is NULL");
+  if (!is_aligned(ws, 256)) return fail(TRI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  if (bytes < (uint64_t)w.total)
+    return fail(TRI_ERR_WORKSPACE, "workspace has %llu bytes, %lld needed", (unsigned long long)bytes, (long long)w.total);
+  return TRI_OK;
+}
+
+template <typename T>
+T* at(void* ws, int64_t off) { return reinterpret_cast<T*>(reinterpret_cast<char*>(ws) + off); }
+
+int do_score(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp, float* raw,
+             int64_t rs_layer, int64_t rs_token, int64_t rs_head, void* ws, const tri::Workspace& w,
+             hipStream_t s) {
+  if (kv->kv_dtype == TRI_KV_FP8_E4M3) return fail(TRI_ERR_UNSUPPORTED, "fp8 keys: scorer not built yet");
+  const int F = kv->head_dim / 2;
+  hipError_t e = tri::launch_prepare(sp->folded, sp->omega, sp->offsets, sp->num_offsets, batch->round_start,
+                                     batch->num_seqs, kv->num_layers, sp->num_score_heads, F, sp->aggregation,
+                                     at<float>(ws, w.coef), at<float>(ws, w.trig), s);
+  if (e != hipSuccess) return launch_status(e, "prepare");
+  tri::ScoreLaunch a{};
+  a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
+  a.block_size = kv->block_size; a.kv_dtype = kv->kv_dtype; a.rope_style = kv->rope_style;
+  a.A = sp->num_score_heads; a.G = sp->num_score_heads / kv->num_kv_heads; a.NO = sp->num_offsets;
+  a.aggregation = sp->aggregation;
+  a.Tmax = batch->max_seq_len; a.num_tiles = w.num_tiles;
+  a.stride_block = kv->stride_block; a.stride_token = kv->stride_token; a.stride_head = kv->stride_head;
+  a.k_layers = kv->k_layers; a.k_scale_layers = kv->k_scale_layers;
+  a.block_table = batch->block_table; a.block_table_pitch = batch->block_table_pitch;
+  a.seq_lens = batch->seq_lens;
+  a.coef = at<float>(ws, w.coef); a.trig = at<float>(ws, w.trig); a.partial = at<float>(ws, w.partial);
+  a.raw = raw; a.raw_stride_layer = rs_layer; a.raw_stride_token = rs_token; a.raw_stride_head = rs_head;
+  return launch_status(tri::launch_score(a, s), "score");
+}
+
+int check_select(const tri_select_params* sel) {
+  if (!sel) return fail(TRI_ERR_INVALID_ARGUMENT, "select params are NULL");
+  if (sel->group_reduce != TRI_REDUCE_MEAN && sel->group_reduce != TRI_REDUCE_MAX)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "group_reduce %d", sel->group_reduce);
+  if (sel->layer_reduce != TRI_REDUCE_MEAN && sel->layer_reduce != TRI_REDUCE_MAX && sel->layer_reduce != -1)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "layer_reduce %d", sel->layer_reduce);
+  if (sel->window_size < 0) return fail(TRI_ERR_INVALID_ARGUMENT, "window_size %d", sel->window_size);
+  return TRI_OK;
+}
+
+int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+              const tri_select_params* sel, const float* raw, int64_t rs_layer, int64_t rs_token,
+              int64_t rs_head, float* fin, int32_t* keep, void* ws, const tri::Workspace& w, hipStream_t s) {
+  tri::SelectLaunch a{};
+  a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.A = sp->num_score_heads;
+  a.G = sp->num_score_heads / kv->num_kv_heads; a.Tmax = batch->max_seq_len; a.num_tiles = w.num_tiles;
+  a.max_budget = batch->max_budget;
+  a.normalize = sel->normalize; a.window_size = sel->window_size; a.protect_prefill = sel->protect_prefill;
+  a.group_reduce = sel->group_reduce; a.layer_reduce = sel->layer_reduce; a.shared = sel->shared;
+  a.seq_lens = batch->seq_lens; a.prefill_lens = batch->prefill_lens; a.budgets = batch->budgets;
+  a.partial = at<float>(ws, w.partial); a.mustd = at<float>(ws, w.mustd);
+  a.raw = raw; a.raw_stride_layer = rs_layer; a.raw_stride_token = rs_token; a.raw_stride_head = rs_head;
+  a.fin = fin ? fin : at<float>(ws, w.fin);
+  a.keep = keep;
+  return launch_status(tri::launch_select(a, s), "select");
+}
+
+int fill_compact(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep, int keep_per_layer,
+                 int shared, tri::CompactLaunch& a) {
+  int rc = check_layout(kv, true);
+  if (rc) return rc;
+  rc = check_batch(batch, true);
+  if (rc) return rc;
+  if (!batch->block_table) return fail(TRI_ERR_INVALID_ARGUMENT, "compaction needs a block table");
+  if (!keep) return fail(TRI_ERR_INVALID_ARGUMENT, "keep is NULL");
+  const int eb = elem_bytes(kv->kv_dtype);
+  const int chunks_per_slot = (shared ? kv->num_kv_heads : 1) * kv->head_dim * eb / 16;
+  if (chunks_per_slot > 1024) return fail(TRI_ERR_UNSUPPORTED, "a slot of %d bytes exceeds one tile", chunks_per_slot * 16);
+  a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
+  a.block_size = kv->block_size; a.elem_bytes = eb; a.max_budget = batch->max_budget;
+  a.keep_per_layer = keep_per_layer ? 1 : 0; a.shared = shared ? 1 : 0;
+  a.has_scales = kv->kv_dtype == TRI_KV_FP8_E4M3;
+  a.stride_block = kv->stride_block; a.stride_token = kv->stride_token; a.stride_head = kv->stride_head;
+  a.k_layers = kv->k_layers; a.v_layers = kv->v_layers;
+  a.k_scale_layers = kv->k_scale_layers; a.v_scale_layers = kv->v_scale_layers;
+  a.block_table = batch->block_table; a.block_table_pitch = batch->block_table_pitch;
+  a.seq_lens = batch->seq_lens; a.budgets = batch->budgets; a.keep = keep; a.Tmax = batch->max_seq_len;
+  a.staging = nullptr;
+  return TRI_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tri_abi_version(void) { return TRI_ABI_VERSION; }
+
+const char* tri_last_error(void) { return g_err; }
+
+int tri_fold_stats(const float* q_mean_real, const float* q_mean_imag, const float* q_abs_mean,
+                   const float* freq_scale_sq, int32_t num_layers, int32_t num_score_heads,
+                   int32_t num_pairs, int32_t disable_mlr, int32_t disable_trig, float* folded,
+                   void* stream) {
+  if (!q_mean_real || !q_mean_imag || !q_abs_mean || !freq_scale_sq || !folded)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_fold_stats: NULL pointer");
+  if (num_layers <= 0 || num_score_heads <= 0 || num_pairs <= 0)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_fold_stats: bad sizes (%d, %d, %d)", num_layers, num_score_heads, num_pairs);
+  return launch_status(tri::launch_fold_stats(q_mean_real, q_mean_imag, q_abs_mean, freq_scale_sq, num_layers,
+                                              num_score_heads, num_pairs, disable_mlr, disable_trig, folded,
+                                              (hipStream_t)stream),
+                       "fold_stats");
+}
+
+uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp) {
+  if (check_layout(kv, false) || check_batch(batch, false) || !sp || sp->num_score_heads <= 0 ||
+      sp->num_offsets <= 0)
+    return 0;
+  return (uint64_t)plan(kv, batch, sp).total;
+}
+
+int tri_score_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                    float* raw, int64_t raw_stride_layer, int64_t raw_stride_token,
+                    int64_t raw_stride_head, void* workspace, uint64_t workspace_bytes, void* stream) {
+  int rc = check_layout(kv, false);
+  if (rc) return rc;
+  rc = check_batch(batch, false);
+  if (rc) return rc;
+  rc = check_score(kv, sp);
+  if (rc) return rc;
+  if (!batch->round_start) return fail(TRI_ERR_INVALID_ARGUMENT, "round_start is NULL");
+  if (!raw) return fail(TRI_ERR_INVALID_ARGUMENT, "raw is NULL");
+  const tri::Workspace w = plan(kv, batch, sp);
+  rc = check_workspace(w, workspace, workspace_bytes);
+  if (rc) return rc;
+  return do_score(kv, batch, sp, raw, raw_stride_layer, raw_stride_token, raw_stride_head, workspace, w,
+                  (hipStream_t)stream);
+}
+
+int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+               const tri_select_params* sel, const float* raw, int64_t raw_stride_layer,
+               int64_t raw_stride_token, int64_t raw_stride_head, float* final_scores, int32_t* keep,
+               void* workspace, uint64_t workspace_bytes, void* stream) {
+  int rc = check_layout(kv, false);
+  if (rc) return rc;
+  rc = check_batch(batch, true);
+  if (rc) return rc;
+  if (!sp || sp->num_score_heads <= 0 || sp->num_score_heads % kv->num_kv_heads || sp->num_offsets <= 0)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_select: bad score params");
+  rc = check_select(sel);
+  if (rc) return rc;
+  if (!raw || !keep) return fail(TRI_ERR_INVALID_ARGUMENT, "raw / keep is NULL");
+  const tri::Workspace w = plan(kv, batch, sp);
+  rc = check_workspace(w, workspace, workspace_bytes);
+  if (rc) return rc;
+  return do_select(kv, batch, sp, sel, raw, raw_stride_layer, raw_stride_token, raw_stride_head, final_scores,
+                   keep, workspace, w, (hipStream_t)stream);
+}
+
+int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,
+                  const int32_t* row_ks, int32_t rows_per_entry, int32_t max_len, int32_t* keep,
+                  int32_t keep_pitch, void* stream) {
+  if (!scores || !row_lens || !row_ks || !keep) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_topk_rows: NULL pointer");
+  if (num_rows < 0 || rows_per_entry <= 0 || row_pitch < max_len || keep_pitch <= 0 || max_len <= 0)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_topk_rows: bad sizes");
+  return launch_status(tri::launch_topk_rows(scores, row_pitch, num_rows, row_lens, row_ks, rows_per_entry, keep,
+                                             keep_pitch, (hipStream_t)stream),
+                       "topk_rows");
+}
+
+int tri_compact_paged(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep,
+                      int32_t keep_per_layer, int32_t shared, void* stream) {
+  tri::CompactLaunch a{};
+  const int rc = fill_compact(kv, batch, keep, keep_per_layer, shared, a);
+  if (rc) return rc;
+  return launch_status(tri::launch_compact(a, (hipStream_t)stream), "compact");
+}
+
+uint64_t tri_compact_full_staging_bytes(const tri_kv_layout* kv, const tri_batch* batch) {
+  if (check_layout(kv, true) || check_batch(batch, false)) return 0;
+  // one layer: K and V of every head row of every logical slot of every sequence
+  return (uint64_t)batch->num_seqs * 2 * kv->num_kv_heads * (uint64_t)batch->max_seq_len * kv->head_dim *
+         elem_bytes(kv->kv_dtype);
+}
+
+int tri_compact_paged_full(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep,
+                           int32_t keep_per_layer, int32_t shared, void* staging, uint64_t staging_bytes,
+                           void* stream) {
+  tri::CompactLaunch a{};
+  const int rc = fill_compact(kv, batch, keep, keep_per_layer, shared, a);
+  if (rc) return rc;
+  if (a.has_scales) return fail(TRI_ERR_UNSUPPORTED, "full-permutation compaction of fp8 caches is not built");
+  if (!staging || !is_aligned(staging, 16)) return fail(TRI_ERR_WORKSPACE, "staging is NULL or unaligned");
+  if (staging_bytes < tri_compact_full_staging_bytes(kv, batch))
+    return fail(TRI_ERR_WORKSPACE, "staging has %llu bytes, %llu needed", (unsigned long long)staging_bytes,
+                (unsigned long long)tri_compact_full_staging_bytes(kv, batch));
+  a.staging = staging;
+  return launch_status(tri::launch_compact_full(a, (hipStream_t)stream), "compact_full");
+}
+
+int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                      const tri_select_params* sel, int32_t* keep, void* workspace,
+                      uint64_t workspace_bytes, void* stream) {
+  int rc = check_layout(kv, true);
+  if (rc) return rc;
+  rc = check_batch(batch, true);
+  if (rc) return rc;
+  rc = check_score(kv, sp);
+  if (rc) return rc;
+  rc = check_select(sel);
+  if (rc) return rc;
+  if (!batch->round_start) return fail(TRI_ERR_INVALID_ARGUMENT, "round_start is NULL");
+  if (!batch->block_table) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_compress_step needs a block table");
+  if (!keep) return fail(TRI_ERR_INVALID_ARGUMENT, "keep is NULL");
+  const tri::Workspace w = plan(kv, batch, sp);
+  rc = check_workspace(w, workspace, workspace_bytes);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  float* raw = at<float>(workspace, w.raw);
+  const int64_t A = sp->num_score_heads;
+  const int64_t rs_layer = (int64_t)batch->max_seq_len * A;
+  rc = do_score(kv, batch, sp, raw, rs_layer, A, 1, workspace, w, s);
+  if (rc) return rc;
+  rc = do_select(kv, batch, sp, sel, raw, rs_layer, A, 1, nullptr, keep, workspace, w, s);
+  if (rc) return rc;
+  tri::CompactLaunch c{};
+  rc = fill_compact(kv, batch, keep, sel->layer_reduce < 0, sel->shared, c);
+  if (rc) return rc;
+  return launch_status(tri::launch_compact(c, s), "compact");
+}
+
+}  // extern "C"

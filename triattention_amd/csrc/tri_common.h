@@ -1,0 +1,112 @@
+// Shared declarations of the gfx950 kernels behind include/triattention_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "triattention_hip.h"
+
+namespace tri {
+
+constexpr int kWave = 64;
+constexpr int kScoreThreads = 256;      // 4 waves per scorer workgroup
+constexpr int kScoreTileTokens = 256;   // tokens of one (sequence, layer) per scorer workgroup
+constexpr int kQPerPass = 4;            // query heads scored per wave pass
+constexpr int kPairsPerLane = 8;        // frequency pairs held by one lane
+constexpr int kMaxOffsets = 32;
+
+inline __host__ __device__ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+inline __host__ __device__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
+struct Workspace {
+  int64_t coef;      // [B][L][A][3][F] fp32: P, R, E for mean aggregation; A1, A2, E for max
+  int64_t trig;      // [B][2][F] offset means of cos / sin, then [B][NO][2][F] tables (max aggregation)
+  int64_t partial;   // [B][L][NT][A][2] fp32 per-tile sum / sum of squares
+  int64_t mustd;     // [B][L][A][2] fp32 mean / safe std
+  int64_t raw;       // [B][L][Tmax][A] fp32 raw scores (tri_compress_step)
+  int64_t fin;       // [B*L*Hkv][Tmax] fp32 selection scores (worst case: per-layer selection)
+  int64_t total;
+  int32_t num_tiles; // NT
+};
+
+inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int Tmax) {
+  Workspace w{};
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) { int64_t o = off; off = align_up(off + bytes, 256); return o; };
+  w.num_tiles = ceil_div(Tmax > 0 ? Tmax : 1, kScoreTileTokens);
+  w.coef = take((int64_t)B * L * A * 3 * F * 4);
+  w.trig = take((int64_t)B * (NO + 1) * 2 * F * 4);
+  w.partial = take((int64_t)B * L * w.num_tiles * A * 2 * 4);
+  w.mustd = take((int64_t)B * L * A * 2 * 4);
+  w.raw = take((int64_t)B * L * Tmax * A * 4);
+  w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
+  w.total = off;
+  return w;
+}
+
+// ---- launchers (defined in the .hip files; all validate nothing: tri_capi.hip does) ----
+
+struct ScoreLaunch {
+  // geometry
+  int B, L, Hkv, D, block_size, kv_dtype, rope_style, A, G, NO, aggregation;
+  int Tmax, num_tiles;
+  int64_t stride_block, stride_token, stride_head;
+  const void* const* k_layers;
+  const float* const* k_scale_layers;
+  const int32_t* block_table;
+  int block_table_pitch;
+  const int32_t* seq_lens;
+  const float* coef;     // workspace
+  const float* trig;     // workspace
+  float* partial;        // workspace
+  float* raw;
+  int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
+};
+
+hipError_t launch_fold_stats(const float* qr, const float* qi, const float* qabs, const float* fs,
+                             int L, int A, int F, int disable_mlr, int disable_trig, float* folded,
+                             hipStream_t s);
+hipError_t launch_prepare(const float* folded, const float* omega, const float* offsets, int NO,
+                          const int32_t* round_start, int B, int L, int A, int F, int aggregation,
+                          float* coef, float* trig, hipStream_t s);
+hipError_t launch_score(const ScoreLaunch& a, hipStream_t s);
+
+struct SelectLaunch {
+  int B, L, Hkv, A, G, Tmax, num_tiles, max_budget;
+  int normalize, window_size, protect_prefill, group_reduce, layer_reduce, shared;
+  const int32_t* seq_lens;
+  const int32_t* prefill_lens;
+  const int32_t* budgets;
+  const float* partial;
+  float* mustd;
+  const float* raw;
+  int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
+  float* fin;          // [rows][Tmax]
+  int32_t* keep;       // [rows][max_budget]
+};
+hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
+hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
+                            const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry,
+                            int32_t* keep, int keep_pitch, hipStream_t s);
+
+struct CompactLaunch {
+  int B, L, Hkv, D, block_size, elem_bytes, max_budget;
+  int keep_per_layer, shared, has_scales;
+  int64_t stride_block, stride_token, stride_head;   // elements
+  const void* const* k_layers;
+  const void* const* v_layers;
+  const float* const* k_scale_layers;
+  const float* const* v_scale_layers;
+  const int32_t* block_table;
+  int block_table_pitch;
+  const int32_t* seq_lens;
+  const int32_t* budgets;
+  const int32_t* keep;
+  int Tmax;
+  void* staging;       // full-permutation mode only
+};
+hipError_t launch_compact(const CompactLaunch& a, hipStream_t s);
+hipError_t launch_compact_full(const CompactLaunch& a, hipStream_t s);
+
+}  // namespace tri

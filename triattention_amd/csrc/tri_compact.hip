@@ -1,0 +1,314 @@
+// In-place, order-preserving paged K/V compaction for gfx950.
+//
+// keep[] is strictly ascending, so keep[j] >= j: destination slot j always lies at
+// or below its source.  One workgroup owns one stream -- (sequence, layer, K or V,
+// head) in per-head mode, (sequence, layer, K or V) in shared mode -- and walks the
+// destination slots in ascending tiles.  Every tile is read completely into
+// registers, the workgroup synchronises, then the tile is written: a tile's writes
+// land below the next tile's first slot while every later source lies at or above
+// it, so nothing that is still to be read is ever overwritten and no staging copy
+// of the cache is needed.  The reference gathers all T rows of K and V into
+// temporaries and scatters them back (runtime/kv_compaction.py:529-546).
+#include "tri_common.h"
+
+namespace tri {
+namespace {
+
+constexpr int kCompactThreads = 256;
+constexpr int kChunksPerThread = 4;                                  // 16-byte chunks held per thread
+constexpr int kTileChunks = kCompactThreads * kChunksPerThread;      // 16 KiB per tile
+constexpr int kSegSlots = 1024;                                      // slots whose addresses are staged in LDS
+
+struct CompactArgs {
+  const void* const* k_layers;
+  const void* const* v_layers;
+  const float* const* k_scale_layers;
+  const float* const* v_scale_layers;
+  const int32_t* block_table;
+  const int32_t* seq_lens;
+  const int32_t* budgets;
+  const int32_t* keep;
+  int64_t stride_block_b, stride_token_b, stride_head_b;   // bytes
+  int B, L, Hkv, block_size, bs_shift, block_table_pitch, max_budget;
+  int keep_per_layer, shared;
+  int chunks_per_row;      // 16-byte chunks of one head row (D * elem_bytes / 16)
+  int heads_per_slot;      // shared ? Hkv : 1
+  int streams_per_layer;   // 2 * (shared ? 1 : Hkv)
+};
+
+__device__ __forceinline__ int64_t slot_offset(const CompactArgs& a, const int32_t* bt, int tok) {
+  const int lb = a.bs_shift >= 0 ? (tok >> a.bs_shift) : (tok / a.block_size);
+  const int in_off = tok - lb * a.block_size;
+  return (int64_t)bt[lb] * a.stride_block_b + (int64_t)in_off * a.stride_token_b;
+}
+
+__global__ __launch_bounds__(kCompactThreads) void compact_kernel(CompactArgs a) {
+  __shared__ int64_t src_off[kSegSlots];
+  __shared__ int64_t dst_off[kSegSlots];
+
+  // stream -> (b, l, kv, row)
+  int sidx = blockIdx.x;
+  const int row = sidx % (a.streams_per_layer / 2); sidx /= (a.streams_per_layer / 2);
+  const int kv = sidx % 2; sidx /= 2;
+  const int l = sidx % a.L;
+  const int b = sidx / a.L;
+
+  int k = a.budgets[b];
+  const int T = a.seq_lens[b];
+  if (k > T) k = T;
+  if (k <= 0) return;
+  const int rows = a.shared ? 1 : a.Hkv;
+  const int32_t* keep = a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows + row) * a.max_budget;
+  const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
+  char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
+  const int head0 = a.shared ? 0 : row;
+
+  const int chunks_per_slot = a.heads_per_slot * a.chunks_per_row;
+  const int slots_per_tile = kTileChunks / chunks_per_slot;   // >= 1 (checked on the host)
+
+  for (int seg = 0; seg < k; seg += kSegSlots) {
+    const int nseg = min(kSegSlots, k - seg);
+    __syncthreads();   // previous segment's LDS no longer in use
+    for (int i = threadIdx.x; i < nseg; i += kCompactThreads) {
+      const int j = seg + i;
+      const int src = keep[j];
+      src_off[i] = slot_offset(a, bt, src);
+      dst_off[i] = slot_offset(a, bt, j);
+    }
+    __syncthreads();
+
+    for (int t0 = 0; t0 < nseg; t0 += slots_per_tile) {
+      const int nslots = min(slots_per_tile, nseg - t0);
+      const int nchunks = nslots * chunks_per_slot;
+      uint4 regs[kChunksPerThread];
+      int64_t dsts[kChunksPerThread];
+      bool live[kChunksPerThread];
+#pragma unroll
+      for (int c = 0; c < kChunksPerThread; ++c) {
+        const int ci = c * kCompactThreads + threadIdx.x;
+        live[c] = ci < nchunks;
+        if (live[c]) {
+          const int sl = t0 + ci / chunks_per_slot;
+          const int within = ci % chunks_per_slot;
+          const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+          const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
+          const int64_t so = src_off[sl] + inner;
+          dsts[c] = dst_off[sl] + inner;
+          live[c] = so != dsts[c];            // row already in place
+          if (live[c]) regs[c] = *reinterpret_cast<const uint4*>(base + so);
+        }
+      }
+      __syncthreads();   // every read of this tile is ordered before any write of it
+#pragma unroll
+      for (int c = 0; c < kChunksPerThread; ++c)
+        if (live[c]) *reinterpret_cast<uint4*>(base + dsts[c]) = regs[c];
+    }
+  }
+}
+
+// fp8 caches carry one fp32 scale per (token, head); they move with the rows.
+// Same ascending-tile argument, one thread per (slot, head).
+struct ScaleArgs {
+  const float* const* k_scale_layers;
+  const float* const* v_scale_layers;
+  const int32_t* block_table;
+  const int32_t* seq_lens;
+  const int32_t* budgets;
+  const int32_t* keep;
+  int B, L, Hkv, block_size, block_table_pitch, max_budget, keep_per_layer, shared;
+};
+
+__global__ __launch_bounds__(256) void compact_scales_kernel(ScaleArgs a) {
+  int sidx = blockIdx.x;
+  const int h = sidx % a.Hkv; sidx /= a.Hkv;
+  const int kv = sidx % 2; sidx /= 2;
+  const int l = sidx % a.L;
+  const int b = sidx / a.L;
+  int k = a.budgets[b];
+  const int T = a.seq_lens[b];
+  if (k > T) k = T;
+  if (k <= 0) return;
+  const int rows = a.shared ? 1 : a.Hkv;
+  const int row = a.shared ? 0 : h;
+  const int32_t* keep = a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows + row) * a.max_budget;
+  const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
+  float* sc = const_cast<float*>(kv ? a.v_scale_layers[l] : a.k_scale_layers[l]);
+  for (int t0 = 0; t0 < k; t0 += 256) {
+    const int j = t0 + threadIdx.x;
+    float v = 0.f;
+    int64_t d = 0;
+    const bool live = j < k;
+    if (live) {
+      const int src = keep[j];
+      const int64_t s = ((int64_t)bt[src / a.block_size] * a.block_size + src % a.block_size) * a.Hkv + h;
+      d = ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * a.Hkv + h;
+      v = sc[s];
+    }
+    __syncthreads();
+    if (live) sc[d] = v;
+  }
+}
+
+// ---- full permutation [kept..., dropped...] through a staging buffer ----------
+// Phase 1 copies every head row of the T logical slots into staging in permuted
+// order; phase 2 copies staging back over slots 0..T-1.  Two kernels on one stream,
+// so phase 2 starts only after phase 1 has read everything.
+struct FullArgs {
+  CompactArgs c;
+  char* staging;   // one layer's worth: [B][2][rows][Tmax] slots
+  int Tmax;
+  int layer;       // the two phases run layer by layer so the staging stays small
+};
+
+// rank[j] for dropped tokens is derived on the fly: dropped token n lands at slot
+// k + (n - number of kept tokens below n).  One thread block per (stream, tile of
+// 256 source tokens); a kept token n = keep[j] goes to slot j.
+__global__ __launch_bounds__(256) void permute_to_staging_kernel(FullArgs f) {
+  const CompactArgs& a = f.c;
+  int sidx = blockIdx.y;
+  const int row = sidx % (a.streams_per_layer / 2); sidx /= (a.streams_per_layer / 2);
+  const int kv = sidx % 2;
+  const int b = sidx / 2;
+  const int l = f.layer;
+  const int T = a.seq_lens[b];
+  int k = a.budgets[b];
+  if (k > T) k = T;
+  const int n0 = blockIdx.x * 256;
+  if (n0 >= T || k <= 0 || k >= T) return;
+  const int rows = a.shared ? 1 : a.Hkv;
+  const int32_t* keep = a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows + row) * a.max_budget;
+  const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
+  const char* base = reinterpret_cast<const char*>(kv ? a.v_layers[l] : a.k_layers[l]);
+  const int head0 = a.shared ? 0 : row;
+  const int chunks_per_slot = a.heads_per_slot * a.chunks_per_row;
+
+  __shared__ int dest[256];
+  const int n = n0 + threadIdx.x;
+  if (n < T) {
+    // lower_bound(keep, n): number of kept tokens < n, and whether n itself is kept.
+    int lo = 0, hi = k;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (keep[mid] < n) lo = mid + 1; else hi = mid;
+    }
+    const bool kept = lo < k && keep[lo] == n;
+    dest[threadIdx.x] = kept ? lo : k + (n - lo);
+  }
+  __syncthreads();
+  const int nvalid = min(256, T - n0);
+  char* stage = f.staging + (int64_t)blockIdx.y * f.Tmax * chunks_per_slot * 16;
+  for (int ci = threadIdx.x; ci < nvalid * chunks_per_slot; ci += 256) {
+    const int sl = ci / chunks_per_slot, within = ci % chunks_per_slot;
+    const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+    const int64_t so = slot_offset(a, bt, n0 + sl) + (int64_t)(head0 + hh) * a.stride_head_b + cc * 16;
+    const uint4 v = *reinterpret_cast<const uint4*>(base + so);
+    *reinterpret_cast<uint4*>(stage + ((int64_t)dest[sl] * chunks_per_slot + within) * 16) = v;
+  }
+}
+
+__global__ __launch_bounds__(256) void staging_to_cache_kernel(FullArgs f) {
+  const CompactArgs& a = f.c;
+  int sidx = blockIdx.y;
+  const int row = sidx % (a.streams_per_layer / 2); sidx /= (a.streams_per_layer / 2);
+  const int kv = sidx % 2;
+  const int b = sidx / 2;
+  const int l = f.layer;
+  const int T = a.seq_lens[b];
+  int k = a.budgets[b];
+  if (k > T) k = T;
+  const int n0 = blockIdx.x * 256;
+  if (n0 >= T || k <= 0 || k >= T) return;
+  const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
+  char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
+  const int head0 = a.shared ? 0 : row;
+  const int chunks_per_slot = a.heads_per_slot * a.chunks_per_row;
+  const int nvalid = min(256, T - n0);
+  const char* stage = f.staging + (int64_t)blockIdx.y * f.Tmax * chunks_per_slot * 16;
+  for (int ci = threadIdx.x; ci < nvalid * chunks_per_slot; ci += 256) {
+    const int sl = ci / chunks_per_slot, within = ci % chunks_per_slot;
+    const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+    const int64_t d = slot_offset(a, bt, n0 + sl) + (int64_t)(head0 + hh) * a.stride_head_b + cc * 16;
+    *reinterpret_cast<uint4*>(base + d) =
+        *reinterpret_cast<const uint4*>(stage + ((int64_t)(n0 + sl) * chunks_per_slot + within) * 16);
+  }
+}
+
+CompactArgs make_args(const CompactLaunch& a) {
+  CompactArgs c{};
+  c.k_layers = a.k_layers;
+  c.v_layers = a.v_layers;
+  c.k_scale_layers = a.k_scale_layers;
+  c.v_scale_layers = a.v_scale_layers;
+  c.block_table = a.block_table;
+  c.seq_lens = a.seq_lens;
+  c.budgets = a.budgets;
+  c.keep = a.keep;
+  c.stride_block_b = a.stride_block * a.elem_bytes;
+  c.stride_token_b = a.stride_token * a.elem_bytes;
+  c.stride_head_b = a.stride_head * a.elem_bytes;
+  c.B = a.B; c.L = a.L; c.Hkv = a.Hkv;
+  c.block_size = a.block_size;
+  c.bs_shift = -1;
+  for (int s = 0; s < 31; ++s)
+    if ((1 << s) == a.block_size) c.bs_shift = s;
+  c.block_table_pitch = a.block_table_pitch;
+  c.max_budget = a.max_budget;
+  c.keep_per_layer = a.keep_per_layer;
+  c.shared = a.shared;
+  c.chunks_per_row = a.D * a.elem_bytes / 16;
+  c.heads_per_slot = a.shared ? a.Hkv : 1;
+  c.streams_per_layer = 2 * (a.shared ? 1 : a.Hkv);
+  return c;
+}
+
+hipError_t launch_scales(const CompactLaunch& a, hipStream_t s) {
+  ScaleArgs sa{};
+  sa.k_scale_layers = a.k_scale_layers;
+  sa.v_scale_layers = a.v_scale_layers;
+  sa.block_table = a.block_table;
+  sa.seq_lens = a.seq_lens;
+  sa.budgets = a.budgets;
+  sa.keep = a.keep;
+  sa.B = a.B; sa.L = a.L; sa.Hkv = a.Hkv;
+  sa.block_size = a.block_size;
+  sa.block_table_pitch = a.block_table_pitch;
+  sa.max_budget = a.max_budget;
+  sa.keep_per_layer = a.keep_per_layer;
+  sa.shared = a.shared;
+  hipLaunchKernelGGL(compact_scales_kernel, dim3(a.B * a.L * 2 * a.Hkv), dim3(256), 0, s, sa);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
+  const CompactArgs c = make_args(a);
+  const int streams = a.B * a.L * c.streams_per_layer;
+  if (streams <= 0 || a.max_budget <= 0) return hipSuccess;
+  hipLaunchKernelGGL(compact_kernel, dim3(streams), dim3(kCompactThreads), 0, s, c);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || !a.has_scales) return e;
+  return launch_scales(a, s);
+}
+
+hipError_t launch_compact_full(const CompactLaunch& a, hipStream_t s) {
+  FullArgs f{};
+  f.c = make_args(a);
+  f.staging = reinterpret_cast<char*>(a.staging);
+  f.Tmax = a.Tmax;
+  const int streams = a.B * f.c.streams_per_layer;
+  if (streams <= 0 || a.Tmax <= 0) return hipSuccess;
+  dim3 grid(ceil_div(a.Tmax, 256), streams);
+  for (int l = 0; l < a.L; ++l) {
+    f.layer = l;
+    hipLaunchKernelGGL(permute_to_staging_kernel, grid, dim3(256), 0, s, f);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(staging_to_cache_kernel, grid, dim3(256), 0, s, f);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+}  // namespace tri

@@ -1,0 +1,617 @@
+// Fused paged key scorer for gfx950 (wave64).
+//
+// One key row (D elements of one KV head of one token) is shared by LPH = D/16
+// lanes; every lane holds 8 frequency pairs: it loads 16 bytes of real parts and
+// 16 bytes of imaginary parts ("half" RoPE layout) or 32 contiguous bytes
+// ("interleaved").  The per-pair coefficients of the four query heads a wave pass
+// scores live in registers (3 x 8 x 4 floats per lane), so one read of a key
+// serves the whole GQA group; the reference instead expands K G-fold and reads it
+// per query head (runtime/selector_hf.py:308-312).
+//
+// Mean aggregation over offsets is linear in cos/sin, so the 17 offsets collapse
+// into per-pair coefficients before the kernel runs (launch_prepare):
+//   raw = sum_f  k_r*P_f + k_i*R_f + |k_f|*E_f
+//   P = s*(q_r*C - q_i*S), R = s*(q_i*C + q_r*S), E = s*(q_abs - |q|),
+//   C = mean_j cos(t_j*w_f), S = mean_j sin(t_j*w_f)          (core/scoring.py:290-355)
+// Max aggregation keeps the per-offset sums and takes cos/sin tables from LDS.
+//
+// The sum over a row's pairs is a transposed butterfly on DPP lane permutes: after
+// two exchange steps each lane of a quad owns one query head, a half-row mirror
+// adds the two quads, so lanes 0-3 / 4-7 of a row hold duplicates; those two quads
+// store two different tokens with a single instruction.
+#include "tri_common.h"
+
+namespace tri {
+namespace {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // row_half_mirror
+constexpr int kDppRor8 = 0x128;       // row_ror:8
+
+// Sum four per-lane partials over the LPH lanes of a row.  Returns the total of
+// query head (2*b0 + b1) of this lane.
+template <int LPH>
+__device__ __forceinline__ float reduce_row(const float (&a)[4], bool b0, bool b1) {
+  const float keep_a = b0 ? a[2] : a[0];
+  const float keep_b = b0 ? a[3] : a[1];
+  const float send_a = b0 ? a[0] : a[2];
+  const float send_b = b0 ? a[1] : a[3];
+  const float ra = keep_a + dpp<kDppXor1>(send_a);
+  const float rb = keep_b + dpp<kDppXor1>(send_b);
+  const float keep = b1 ? rb : ra;
+  const float send = b1 ? ra : rb;
+  float r = keep + dpp<kDppXor2>(send);
+  if (LPH >= 8) r += dpp<kDppHalfMirror>(r);
+  if (LPH >= 16) r += dpp<kDppRor8>(r);
+  return r;
+}
+
+template <int DT>
+__device__ __forceinline__ float elem_lo(uint32_t w);
+template <int DT>
+__device__ __forceinline__ float elem_hi(uint32_t w);
+template <>
+__device__ __forceinline__ float elem_lo<TRI_KV_BF16>(uint32_t w) { return __uint_as_float(w << 16); }
+template <>
+__device__ __forceinline__ float elem_hi<TRI_KV_BF16>(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+template <>
+__device__ __forceinline__ float elem_lo<TRI_KV_FP16>(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(w & 0xffffu));
+}
+template <>
+__device__ __forceinline__ float elem_hi<TRI_KV_FP16>(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
+}
+
+struct RowData {
+  uint4 lo;  // half: 8 real parts          interleaved: pairs 0-3
+  uint4 hi;  // half: 8 imaginary parts     interleaved: pairs 4-7
+};
+
+// Real and imaginary part of this lane's pair p (0..7).
+template <int DT, bool IL>
+__device__ __forceinline__ void unpack_pair(const RowData& d, int p, float& kr, float& ki) {
+  const uint32_t* lo = reinterpret_cast<const uint32_t*>(&d.lo);
+  const uint32_t* hi = reinterpret_cast<const uint32_t*>(&d.hi);
+  if (IL) {
+    const uint32_t w = (p < 4) ? lo[p] : hi[p - 4];
+    kr = elem_lo<DT>(w);
+    ki = elem_hi<DT>(w);
+  } else {
+    const uint32_t wr = lo[p >> 1], wi = hi[p >> 1];
+    kr = (p & 1) ? elem_hi<DT>(wr) : elem_lo<DT>(wr);
+    ki = (p & 1) ? elem_hi<DT>(wi) : elem_lo<DT>(wi);
+  }
+}
+
+struct ScoreArgs {
+  const void* const* k_layers;
+  const int32_t* block_table;
+  const int32_t* seq_lens;
+  const float* coef;
+  const float* trig;
+  float* partial;
+  float* raw;
+  int64_t stride_block, stride_token, stride_head;
+  int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
+  int L, Hkv, A, G, NO;
+  int block_size, bs_shift;     // bs_shift >= 0 when block_size is a power of two
+  int block_table_pitch;        // < 0: dense, physical block = sequence index
+  int num_tiles, QC, Hpad;
+};
+
+// Lane geometry shared by the mean and max kernels.
+template <int LPH>
+struct LaneMap {
+  int m, g, head, tsub, tpi, q0, nq, qsel;
+  bool b0, b1, store_lane, slot_b;
+  __device__ LaneMap(const ScoreArgs& a, int lane, int sib) {
+    constexpr int UPW = kWave / LPH;
+    m = lane % LPH;
+    g = lane / LPH;
+    const int hc = sib / a.QC, qc = sib % a.QC;
+    if (a.Hpad >= UPW) {
+      tpi = 1; tsub = 0; head = hc * UPW + g;
+    } else {
+      tpi = UPW / a.Hpad; head = g % a.Hpad; tsub = g / a.Hpad;
+    }
+    const int flip = (LPH >= 8) ? ((m >> 2) & 1) : 0;
+    b0 = ((m & 1) ^ flip) != 0;
+    b1 = (((m >> 1) & 1) ^ flip) != 0;
+    qsel = 2 * (int)b0 + (int)b1;
+    q0 = qc * kQPerPass;
+    nq = min(kQPerPass, a.G - q0);
+    store_lane = (LPH >= 8) ? (m < 8) : true;
+    slot_b = (LPH >= 8) && (m >= 4);
+  }
+};
+
+template <int LPH, int DT, bool IL>
+__device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbase, int b, int tok,
+                                            int last_tok, const int* lds_blk, int lb0,
+                                            int64_t lane_off_elems) {
+  // Rows past the tile are clamped to its last token (loaded, never stored), so
+  // every address stays inside the blocks whose ids were staged in LDS.
+  const int t = min(tok, last_tok);
+  int64_t phys, in_off;
+  if (a.block_table_pitch < 0) {
+    phys = b; in_off = t;
+  } else {
+    const int lb = a.bs_shift >= 0 ? (t >> a.bs_shift) : (t / a.block_size);
+    phys = lds_blk[lb - lb0];
+    in_off = t - lb * a.block_size;
+  }
+  const int64_t e = phys * a.stride_block + in_off * a.stride_token + lane_off_elems;
+  const char* p = kbase + e * 2;
+  RowData d;
+  d.lo = *reinterpret_cast<const uint4*>(p);
+  d.hi = *reinterpret_cast<const uint4*>(p + (IL ? 16 : LPH * 16));
+  return d;
+}
+
+// ------------------------------------------------------------------ mean
+template <int LPH, int DT, bool IL, int SP>
+__global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) {
+  constexpr int F = LPH * kPairsPerLane;
+  __shared__ int lds_blk[kScoreTileTokens + 2];
+  __shared__ float lds_s1[kScoreThreads];
+  __shared__ float lds_s2[kScoreThreads];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x, sib = blockIdx.y;
+  const int b = blockIdx.z / a.L, l = blockIdx.z % a.L;
+  const int seq_len = a.seq_lens[b];
+  const int n0 = tile * kScoreTileTokens;
+  if (n0 >= seq_len) return;
+  const int n1 = min(n0 + kScoreTileTokens, seq_len);
+
+  int lb0 = 0;
+  if (a.block_table_pitch >= 0) {
+    lb0 = n0 / a.block_size;
+    const int lb1 = (n1 - 1) / a.block_size;
+    for (int i = threadIdx.x; i <= lb1 - lb0; i += kScoreThreads)
+      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
+  }
+  __syncthreads();
+
+  const LaneMap<LPH> lm(a, lane, sib);
+  const bool head_ok = lm.head < a.Hkv;
+  const int head_c = head_ok ? lm.head : 0;
+
+  // Coefficients of the (up to) four query heads of this pass.
+  float P[4][8], R[4][8], E[4][8];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const bool ok = head_ok && q < lm.nq;
+    const int ah = head_c * a.G + lm.q0 + (q < lm.nq ? q : 0);
+    const float* c = a.coef + (((int64_t)(b * a.L + l) * a.A + ah) * 3) * F + lm.m * kPairsPerLane;
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+      float4 p4 = ok ? *reinterpret_cast<const float4*>(c + v * 4) : float4{0, 0, 0, 0};
+      float4 r4 = ok ? *reinterpret_cast<const float4*>(c + F + v * 4) : float4{0, 0, 0, 0};
+      float4 e4 = ok ? *reinterpret_cast<const float4*>(c + 2 * F + v * 4) : float4{0, 0, 0, 0};
+      P[q][v * 4 + 0] = p4.x; P[q][v * 4 + 1] = p4.y; P[q][v * 4 + 2] = p4.z; P[q][v * 4 + 3] = p4.w;
+      R[q][v * 4 + 0] = r4.x; R[q][v * 4 + 1] = r4.y; R[q][v * 4 + 2] = r4.z; R[q][v * 4 + 3] = r4.w;
+      E[q][v * 4 + 0] = e4.x; E[q][v * 4 + 1] = e4.y; E[q][v * 4 + 2] = e4.z; E[q][v * 4 + 3] = e4.w;
+    }
+  }
+
+  const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
+  const int64_t lane_off = (int64_t)head_c * a.stride_head + (IL ? lm.m * 16 : lm.m * 8);
+
+  // This wave's tokens: a quarter of the tile, walked in stages of SP token pairs.
+  constexpr int TW = kScoreTileTokens / 4;
+  const int wstart = n0 + wave * TW;
+  const int wend = min(wstart + TW, n1);
+  const int tok_per_pair = 2 * lm.tpi;
+  const int tok_per_stage = SP * tok_per_pair;
+
+  const int a_out = head_c * a.G + lm.q0 + lm.qsel;
+  const bool out_ok = head_ok && lm.store_lane && lm.qsel < lm.nq;
+  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)a_out * a.raw_stride_head;
+
+  float s1 = 0.f, s2 = 0.f;
+
+  auto load_stage = [&](RowData (&buf)[SP][2], int base) {
+#pragma unroll
+    for (int p = 0; p < SP; ++p) {
+      const int ta = base + p * tok_per_pair + lm.tsub;
+      buf[p][0] = load_row<LPH, DT, IL>(a, kbase, b, ta, n1 - 1, lds_blk, lb0, lane_off);
+      buf[p][1] = load_row<LPH, DT, IL>(a, kbase, b, ta + lm.tpi, n1 - 1, lds_blk, lb0, lane_off);
+    }
+  };
+
+  auto score_row = [&](const RowData& d) -> float {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      float kr, ki;
+      unpack_pair<DT, IL>(d, p, kr, ki);
+      const float mag = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[q] = fmaf(kr, P[q][p], acc[q]);
+        acc[q] = fmaf(ki, R[q][p], acc[q]);
+        acc[q] = fmaf(mag, E[q][p], acc[q]);
+      }
+    }
+    return reduce_row<LPH>(acc, lm.b0, lm.b1);
+  };
+
+  auto compute_stage = [&](const RowData (&buf)[SP][2], int base) {
+#pragma unroll
+    for (int p = 0; p < SP; ++p) {
+      const int ta = base + p * tok_per_pair + lm.tsub;
+      const int tb = ta + lm.tpi;
+      const float ra = score_row(buf[p][0]);
+      const float rb = score_row(buf[p][1]);
+      if (LPH >= 8) {
+        const float v = lm.slot_b ? rb : ra;
+        const int t = lm.slot_b ? tb : ta;
+        if (out_ok && t < wend) {
+          raw_row[(int64_t)t * a.raw_stride_token] = v;
+          s1 += v;
+          s2 = fmaf(v, v, s2);
+        }
+      } else {
+        if (out_ok && ta < wend) {
+          raw_row[(int64_t)ta * a.raw_stride_token] = ra;
+          s1 += ra;
+          s2 = fmaf(ra, ra, s2);
+        }
+        if (out_ok && tb < wend) {
+          raw_row[(int64_t)tb * a.raw_stride_token] = rb;
+          s1 += rb;
+          s2 = fmaf(rb, rb, s2);
+        }
+      }
+    }
+  };
+
+  if (wstart < wend) {
+    RowData buf_a[SP][2], buf_b[SP][2];
+    int base = wstart;
+    load_stage(buf_a, base);
+    while (base < wend) {
+      load_stage(buf_b, base + tok_per_stage);
+      compute_stage(buf_a, base);
+      base += tok_per_stage;
+      if (base >= wend) break;
+      load_stage(buf_a, base + tok_per_stage);
+      compute_stage(buf_b, base);
+      base += tok_per_stage;
+    }
+  }
+
+  // Per-tile sum and sum of squares of every (head, query head) of this pass, in
+  // a fixed order so that the statistics are reproducible run to run.
+  lds_s1[threadIdx.x] = s1;
+  lds_s2[threadIdx.x] = s2;
+  __syncthreads();
+  constexpr int UPW = kWave / LPH;
+  const int heads_here = (a.Hpad >= UPW) ? UPW : a.Hpad;
+  const int tpi = (a.Hpad >= UPW) ? 1 : UPW / a.Hpad;
+  if ((int)threadIdx.x < heads_here * kQPerPass) {
+    const int hl = threadIdx.x / kQPerPass, q = threadIdx.x % kQPerPass;
+    const int hc = sib / a.QC, qc = sib % a.QC;
+    const int head = (a.Hpad >= UPW) ? hc * UPW + hl : hl;
+    const int qq = qc * kQPerPass + q;
+    if (head < a.Hkv && qq < a.G) {
+      const int ma = (q >> 1) | ((q & 1) << 1);                           // token-A lane of q
+      const int mb = 4 + (1 - (q >> 1)) + 2 * (1 - (q & 1));              // token-B lane of q
+      float t1 = 0.f, t2 = 0.f;
+      for (int w = 0; w < 4; ++w)
+        for (int ts = 0; ts < tpi; ++ts) {
+          const int g = ts * heads_here + hl;
+          const int la = w * kWave + g * LPH + ma;
+          t1 += lds_s1[la];
+          t2 += lds_s2[la];
+          if (LPH >= 8) {
+            const int lb = w * kWave + g * LPH + mb;
+            t1 += lds_s1[lb];
+            t2 += lds_s2[lb];
+          }
+        }
+      float* out = a.partial + (((int64_t)(b * a.L + l) * a.num_tiles + tile) * a.A + head * a.G + qq) * 2;
+      out[0] = t1;
+      out[1] = t2;
+    }
+  }
+}
+
+// ------------------------------------------------------------------- max
+// Per-offset sums, max over offsets (core/scoring.py:338-339).  Not the default
+// setting; written for correctness, not tuned.
+template <int LPH, int DT, bool IL>
+__global__ __launch_bounds__(kScoreThreads) void score_max_kernel(ScoreArgs a) {
+  constexpr int F = LPH * kPairsPerLane;
+  __shared__ int lds_blk[kScoreTileTokens + 2];
+  __shared__ float lds_s1[kScoreThreads];
+  __shared__ float lds_s2[kScoreThreads];
+  __shared__ float lds_cos[kMaxOffsets * F];
+  __shared__ float lds_sin[kMaxOffsets * F];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x, sib = blockIdx.y;
+  const int b = blockIdx.z / a.L, l = blockIdx.z % a.L;
+  const int seq_len = a.seq_lens[b];
+  const int n0 = tile * kScoreTileTokens;
+  if (n0 >= seq_len) return;
+  const int n1 = min(n0 + kScoreTileTokens, seq_len);
+
+  int lb0 = 0;
+  if (a.block_table_pitch >= 0) {
+    lb0 = n0 / a.block_size;
+    const int lb1 = (n1 - 1) / a.block_size;
+    for (int i = threadIdx.x; i <= lb1 - lb0; i += kScoreThreads)
+      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
+  }
+  for (int i = threadIdx.x; i < a.NO * F; i += kScoreThreads) {
+    const int j = i / F, f = i % F;
+    lds_cos[i] = a.trig[((int64_t)(b * a.NO + j) * 2 + 0) * F + f];
+    lds_sin[i] = a.trig[((int64_t)(b * a.NO + j) * 2 + 1) * F + f];
+  }
+  __syncthreads();
+
+  const LaneMap<LPH> lm(a, lane, sib);
+  const bool head_ok = lm.head < a.Hkv;
+  const int head_c = head_ok ? lm.head : 0;
+
+  float A1[4][8], A2[4][8], E[4][8];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const bool ok = head_ok && q < lm.nq;
+    const int ah = head_c * a.G + lm.q0 + (q < lm.nq ? q : 0);
+    const float* c = a.coef + (((int64_t)(b * a.L + l) * a.A + ah) * 3) * F + lm.m * kPairsPerLane;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      A1[q][p] = ok ? c[p] : 0.f;
+      A2[q][p] = ok ? c[F + p] : 0.f;
+      E[q][p] = ok ? c[2 * F + p] : 0.f;
+    }
+  }
+
+  const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
+  const int64_t lane_off = (int64_t)head_c * a.stride_head + (IL ? lm.m * 16 : lm.m * 8);
+  constexpr int TW = kScoreTileTokens / 4;
+  const int wstart = n0 + wave * TW;
+  const int wend = min(wstart + TW, n1);
+  const int a_out = head_c * a.G + lm.q0 + lm.qsel;
+  const bool out_ok = head_ok && lm.store_lane && lm.qsel < lm.nq;
+  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)a_out * a.raw_stride_head;
+  float s1 = 0.f, s2 = 0.f;
+
+  auto score_row = [&](const RowData& d) -> float {
+    float kr[8], ki[8], ext[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      unpack_pair<DT, IL>(d, p, kr[p], ki[p]);
+      const float mag = __builtin_amdgcn_sqrtf(fmaf(ki[p], ki[p], kr[p] * kr[p]));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ext[q] = fmaf(mag, E[q][p], ext[q]);
+    }
+    const float extra = reduce_row<LPH>(ext, lm.b0, lm.b1);
+    float best = -INFINITY;
+    for (int j = 0; j < a.NO; ++j) {
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const float c = lds_cos[j * F + lm.m * kPairsPerLane + p];
+        const float s = lds_sin[j * F + lm.m * kPairsPerLane + p];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float pa = fmaf(A1[q][p], kr[p], A2[q][p] * ki[p]);   // s*Re(q conj k)
+          const float pb = fmaf(A2[q][p], kr[p], -A1[q][p] * ki[p]);  // s*Im(q conj k)
+          acc[q] = fmaf(pa, c, acc[q]);
+          acc[q] = fmaf(-pb, s, acc[q]);
+        }
+      }
+      best = fmaxf(best, reduce_row<LPH>(acc, lm.b0, lm.b1));
+    }
+    return best + extra;
+  };
+
+  const int step = 2 * lm.tpi;
+  for (int base = wstart; base < wend; base += step) {
+    const int ta = base + lm.tsub, tb = ta + lm.tpi;
+    const RowData da = load_row<LPH, DT, IL>(a, kbase, b, ta, n1 - 1, lds_blk, lb0, lane_off);
+    const RowData db = load_row<LPH, DT, IL>(a, kbase, b, tb, n1 - 1, lds_blk, lb0, lane_off);
+    const float ra = score_row(da);
+    const float rb = score_row(db);
+    if (LPH >= 8) {
+      const float v = lm.slot_b ? rb : ra;
+      const int t = lm.slot_b ? tb : ta;
+      if (out_ok && t < wend) {
+        raw_row[(int64_t)t * a.raw_stride_token] = v;
+        s1 += v; s2 = fmaf(v, v, s2);
+      }
+    } else {
+      if (out_ok && ta < wend) { raw_row[(int64_t)ta * a.raw_stride_token] = ra; s1 += ra; s2 = fmaf(ra, ra, s2); }
+      if (out_ok && tb < wend) { raw_row[(int64_t)tb * a.raw_stride_token] = rb; s1 += rb; s2 = fmaf(rb, rb, s2); }
+    }
+  }
+
+  lds_s1[threadIdx.x] = s1;
+  lds_s2[threadIdx.x] = s2;
+  __syncthreads();
+  constexpr int UPW = kWave / LPH;
+  const int heads_here = (a.Hpad >= UPW) ? UPW : a.Hpad;
+  const int tpi = (a.Hpad >= UPW) ? 1 : UPW / a.Hpad;
+  if ((int)threadIdx.x < heads_here * kQPerPass) {
+    const int hl = threadIdx.x / kQPerPass, q = threadIdx.x % kQPerPass;
+    const int hc = sib / a.QC, qc = sib % a.QC;
+    const int head = (a.Hpad >= UPW) ? hc * UPW + hl : hl;
+    const int qq = qc * kQPerPass + q;
+    if (head < a.Hkv && qq < a.G) {
+      const int ma = (q >> 1) | ((q & 1) << 1);
+      const int mb = 4 + (1 - (q >> 1)) + 2 * (1 - (q & 1));
+      float t1 = 0.f, t2 = 0.f;
+      for (int w = 0; w < 4; ++w)
+        for (int ts = 0; ts < tpi; ++ts) {
+          const int g = ts * heads_here + hl;
+          t1 += lds_s1[w * kWave + g * LPH + ma];
+          t2 += lds_s2[w * kWave + g * LPH + ma];
+          if (LPH >= 8) {
+            t1 += lds_s1[w * kWave + g * LPH + mb];
+            t2 += lds_s2[w * kWave + g * LPH + mb];
+          }
+        }
+      float* out = a.partial + (((int64_t)(b * a.L + l) * a.num_tiles + tile) * a.A + head * a.G + qq) * 2;
+      out[0] = t1;
+      out[1] = t2;
+    }
+  }
+}
+
+// -------------------------------------------------------------- prologues
+__global__ void fold_stats_kernel(const float* qr, const float* qi, const float* qabs, const float* fs,
+                                  int n_heads_total, int F, int disable_mlr, int disable_trig,
+                                  float* folded) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_heads_total * F) return;
+  const int la = idx / F, f = idx % F;
+  const float r = qr[idx], i = qi[idx], s = fs[idx];
+  const float qmag = __fsqrt_rn(__fadd_rn(__fadd_rn(__fmul_rn(r, r), __fmul_rn(i, i)), 1e-8f));
+  const float coef = disable_mlr ? qabs[idx] : __fsub_rn(qabs[idx], qmag);
+  float* o = folded + (int64_t)la * 3 * F;
+  o[f] = disable_trig ? 0.f : s * r;
+  o[F + f] = disable_trig ? 0.f : s * i;
+  o[2 * F + f] = s * coef;
+}
+
+// cos/sin of the fp32-rounded phase t*w, evaluated in double and rounded once:
+// the correctly rounded value of what torch.cos(t * omega) approximates in fp32
+// (core/scoring.py:322-324).
+__global__ void trig_kernel(const float* omega, const float* offsets, int NO, const int32_t* round_start,
+                            int F, float* trig, float* mean_cs) {
+  const int b = blockIdx.x, f = threadIdx.x;
+  if (f >= F) return;
+  const float w = omega[f];
+  const float rs = (float)round_start[b];
+  double sc = 0.0, ss = 0.0;
+  for (int j = 0; j < NO; ++j) {
+    const float t = __fadd_rn(rs, offsets[j]);
+    const double ph = (double)__fmul_rn(t, w);
+    const float c = (float)cos(ph), s = (float)sin(ph);
+    if (trig) {
+      trig[((int64_t)(b * NO + j) * 2 + 0) * F + f] = c;
+      trig[((int64_t)(b * NO + j) * 2 + 1) * F + f] = s;
+    }
+    sc += c;
+    ss += s;
+  }
+  mean_cs[(int64_t)b * 2 * F + f] = (float)(sc / NO);
+  mean_cs[(int64_t)b * 2 * F + F + f] = (float)(ss / NO);
+}
+
+__global__ void coef_kernel(const float* folded, const float* mean_cs, int LA, int F, int mean_mode,
+                            float* coef) {
+  const int b = blockIdx.y;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= LA * F) return;
+  const int la = idx / F, f = idx % F;
+  const float* in = folded + (int64_t)la * 3 * F;
+  float* o = coef + ((int64_t)b * LA + la) * 3 * F;
+  const float a1 = in[f], a2 = in[F + f], e = in[2 * F + f];
+  if (mean_mode) {
+    const float c = mean_cs[(int64_t)b * 2 * F + f], s = mean_cs[(int64_t)b * 2 * F + F + f];
+    o[f] = fmaf(a1, c, -a2 * s);
+    o[F + f] = fmaf(a2, c, a1 * s);
+  } else {
+    o[f] = a1;
+    o[F + f] = a2;
+  }
+  o[2 * F + f] = e;
+}
+
+template <int LPH, int DT, bool IL>
+hipError_t launch_score_t(const ScoreArgs& args, dim3 grid, int aggregation, hipStream_t s) {
+  if (aggregation == TRI_REDUCE_MEAN)
+    hipLaunchKernelGGL((score_mean_kernel<LPH, DT, IL, 2>), grid, dim3(kScoreThreads), 0, s, args);
+  else
+    hipLaunchKernelGGL((score_max_kernel<LPH, DT, IL>), grid, dim3(kScoreThreads), 0, s, args);
+  return hipGetLastError();
+}
+
+template <int LPH>
+hipError_t launch_score_lph(const ScoreArgs& args, dim3 grid, int dt, int il, int aggregation, hipStream_t s) {
+  if (dt == TRI_KV_BF16)
+    return il ? launch_score_t<LPH, TRI_KV_BF16, true>(args, grid, aggregation, s)
+              : launch_score_t<LPH, TRI_KV_BF16, false>(args, grid, aggregation, s);
+  if (dt == TRI_KV_FP16)
+    return il ? launch_score_t<LPH, TRI_KV_FP16, true>(args, grid, aggregation, s)
+              : launch_score_t<LPH, TRI_KV_FP16, false>(args, grid, aggregation, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t launch_fold_stats(const float* qr, const float* qi, const float* qabs, const float* fs,
+                             int L, int A, int F, int disable_mlr, int disable_trig, float* folded,
+                             hipStream_t s) {
+  const int n = L * A * F;
+  hipLaunchKernelGGL(fold_stats_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s, qr, qi, qabs, fs, L * A, F,
+                     disable_mlr, disable_trig, folded);
+  return hipGetLastError();
+}
+
+hipError_t launch_prepare(const float* folded, const float* omega, const float* offsets, int NO,
+                          const int32_t* round_start, int B, int L, int A, int F, int aggregation,
+                          float* coef, float* trig, hipStream_t s) {
+  // The first 2*F floats per sequence of the trig area hold the offset means; the
+  // per-offset tables (max aggregation) follow the means of all sequences.
+  float* mean_cs = trig;
+  float* tables = (aggregation == TRI_REDUCE_MAX) ? trig + (int64_t)B * 2 * F : nullptr;
+  hipLaunchKernelGGL(trig_kernel, dim3(B), dim3(F), 0, s, omega, offsets, NO, round_start, F, tables, mean_cs);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(coef_kernel, dim3(ceil_div(L * A * F, 256), B), dim3(256), 0, s, folded, mean_cs, L * A, F,
+                     aggregation == TRI_REDUCE_MEAN ? 1 : 0, coef);
+  return hipGetLastError();
+}
+
+hipError_t launch_score(const ScoreLaunch& a, hipStream_t s) {
+  ScoreArgs k{};
+  k.k_layers = a.k_layers;
+  k.block_table = a.block_table;
+  k.seq_lens = a.seq_lens;
+  k.coef = a.coef;
+  k.trig = (a.aggregation == TRI_REDUCE_MAX) ? a.trig + (int64_t)a.B * 2 * (a.D / 2) : nullptr;
+  k.partial = a.partial;
+  k.raw = a.raw;
+  k.stride_block = a.stride_block;
+  k.stride_token = a.stride_token;
+  k.stride_head = a.stride_head;
+  k.raw_stride_layer = a.raw_stride_layer;
+  k.raw_stride_token = a.raw_stride_token;
+  k.raw_stride_head = a.raw_stride_head;
+  k.L = a.L; k.Hkv = a.Hkv; k.A = a.A; k.G = a.G; k.NO = a.NO;
+  k.block_size = a.block_size;
+  k.bs_shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == a.block_size) k.bs_shift = sft;
+  k.block_table_pitch = a.block_table ? a.block_table_pitch : -1;
+  k.num_tiles = a.num_tiles;
+  k.QC = ceil_div(a.G, kQPerPass);
+  int hpad = 1;
+  while (hpad < a.Hkv) hpad <<= 1;
+  k.Hpad = hpad;
+  const int lph = a.D / 16;
+  const int upw = kWave / lph;
+  const int HC = hpad >= upw ? hpad / upw : 1;
+  dim3 grid(a.num_tiles, HC * k.QC, a.B * a.L);
+  const int il = a.rope_style == TRI_ROPE_INTERLEAVED;
+  switch (lph) {
+    case 4: return launch_score_lph<4>(k, grid, a.kv_dtype, il, a.aggregation, s);
+    case 8: return launch_score_lph<8>(k, grid, a.kv_dtype, il, a.aggregation, s);
+    case 16: return launch_score_lph<16>(k, grid, a.kv_dtype, il, a.aggregation, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace tri

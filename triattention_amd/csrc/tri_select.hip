@@ -1,0 +1,264 @@
+// Score normalisation, guards, head / layer reduction and per-row top-k for gfx950.
+//
+//  finalize_stats_kernel : per-(sequence, layer, score head) mean and safe std from the
+//                          scorer's per-tile sums (runtime/selector_hf.py:896-913).
+//  combine_kernel        : z-score, +inf guards, reduce over the query heads of a KV
+//                          head, reduce over layers (runtime/selector_hf.py:916-989).
+//  topk_rows_kernel      : order-preserving radix select on the monotone integer
+//                          image of the float, then an ordered compaction that emits
+//                          the kept token indices ascending; ties at the threshold
+//                          keep the lowest index (replaces torch.topk + chunk merge +
+//                          torch.sort, runtime/selector_hf.py:990-1025).
+#include "tri_common.h"
+
+namespace tri {
+namespace {
+
+__global__ void finalize_stats_kernel(const float* partial, const int32_t* seq_lens, int B, int L, int A,
+                                      int num_tiles, int normalize, float* mustd) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= B * L * A) return;
+  const int a = idx % A, bl = idx / A, b = bl / L;
+  float mean = 0.f, sd = 1.f;
+  if (normalize) {
+    const int T = seq_lens[b];
+    const int nt = ceil_div(T, kScoreTileTokens);
+    double s = 0.0, q = 0.0;
+    for (int t = 0; t < nt; ++t) {
+      const float* p = partial + (((int64_t)bl * num_tiles + t) * A + a) * 2;
+      s += (double)p[0];
+      q += (double)p[1];
+    }
+    // The reference's formula on fp32 sums (runtime/selector_hf.py:902-909).
+    const float sum = (float)s, sumsq = (float)q, cnt = (float)T;
+    mean = __fdiv_rn(sum, cnt);
+    float var = 0.f;
+    if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(mean, mean))), (float)(T - 1));
+    var = fmaxf(var, 0.f);
+    sd = __fsqrt_rn(var);
+    if (sd < 1e-8f) sd = 1.f;
+  }
+  mustd[(int64_t)idx * 2] = mean;
+  mustd[(int64_t)idx * 2 + 1] = sd;
+}
+
+struct CombineArgs {
+  const float* raw;
+  const float* mustd;
+  const int32_t* seq_lens;
+  const int32_t* prefill_lens;
+  float* fin;
+  int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
+  int B, L, Hkv, A, G, Tmax;
+  int window_size, protect_prefill, group_reduce, layer_reduce, shared;
+  int rows_per_seq;   // rows per (sequence[, layer]): shared ? 1 : Hkv
+  int tokens_per_wg;  // 256 / rows_per_seq
+};
+
+// One thread per (token, output row).  Grid: (token tiles, layers or 1, B).
+__global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
+  extern __shared__ float tile[];  // [rows_per_seq][tokens_per_wg]
+  const int b = blockIdx.z;
+  const int T = a.seq_lens[b];
+  const int n0 = blockIdx.x * a.tokens_per_wg;
+  if (n0 >= T) return;
+  const int R = a.rows_per_seq;
+  const int tn = threadIdx.x / R, r = threadIdx.x % R;
+  const int n = n0 + tn;
+  const bool per_layer = a.layer_reduce < 0;
+  const int l_begin = per_layer ? blockIdx.y : 0;
+  const int l_end = per_layer ? blockIdx.y + 1 : a.L;
+
+  if (tn < a.tokens_per_wg && n < T) {
+    bool guard = false;
+    if (a.window_size > 0) guard = n >= T - min(a.window_size, T);
+    if (a.protect_prefill && a.prefill_lens) guard = guard || (n < a.prefill_lens[b]);
+    const int h_begin = a.shared ? 0 : r;
+    const int h_end = a.shared ? a.Hkv : r + 1;
+    float acc = 0.f;
+    for (int l = l_begin; l < l_end; ++l) {
+      const float* raw_l = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)n * a.raw_stride_token;
+      const float* ms = a.mustd + (int64_t)(b * a.L + l) * a.A * 2;
+      float v = -INFINITY;
+      for (int h = h_begin; h < h_end; ++h) {
+        float gv = (a.group_reduce == TRI_REDUCE_MAX) ? -INFINITY : 0.f;
+        for (int q = 0; q < a.G; ++q) {
+          const int ah = h * a.G + q;
+          const float x = raw_l[(int64_t)ah * a.raw_stride_head];
+          const float z = __fdiv_rn(__fsub_rn(x, ms[ah * 2]), ms[ah * 2 + 1]);
+          gv = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(gv, z) : __fadd_rn(gv, z);
+        }
+        if (a.group_reduce != TRI_REDUCE_MAX) gv = __fdiv_rn(gv, (float)a.G);
+        v = fmaxf(v, gv);
+      }
+      if (guard) v = INFINITY;
+      if (l == l_begin) acc = v;
+      else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
+    }
+    if (a.layer_reduce == TRI_REDUCE_MEAN) acc = __fdiv_rn(acc, (float)a.L);
+    tile[r * a.tokens_per_wg + tn] = acc;
+  }
+  __syncthreads();
+  // Coalesced write of the [rows][tokens] tile.
+  const int nvalid = min(a.tokens_per_wg, T - n0);
+  const int64_t row0 = per_layer ? ((int64_t)(b * a.L + blockIdx.y) * R) : ((int64_t)b * R);
+  for (int i = threadIdx.x; i < R * a.tokens_per_wg; i += 256) {
+    const int rr = i / a.tokens_per_wg, tt = i % a.tokens_per_wg;
+    if (tt < nvalid) a.fin[(row0 + rr) * a.Tmax + n0 + tt] = tile[i];
+  }
+}
+
+// Monotone map float -> uint32: a < b  <=>  key(a) < key(b).
+__device__ __forceinline__ uint32_t float_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+constexpr int kTopkThreads = 1024;
+
+// One workgroup per row.
+__global__ __launch_bounds__(kTopkThreads) void topk_rows_kernel(const float* scores, int64_t row_pitch,
+                                                                const int32_t* row_lens,
+                                                                const int32_t* row_ks, int rows_per_entry,
+                                                                int32_t* keep, int keep_pitch) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t scan[256];
+  __shared__ uint32_t sh_prefix, sh_remaining;
+  __shared__ uint32_t cnt_gt[kTopkThreads];
+  __shared__ uint32_t cnt_eq[kTopkThreads];
+
+  const int row = blockIdx.x;
+  const int entry = row / rows_per_entry;
+  const int T = row_lens[entry];
+  int k = row_ks[entry];
+  if (k > T) k = T;
+  if (k <= 0 || T <= 0) return;
+  const float* x = scores + (int64_t)row * row_pitch;
+  int32_t* out = keep + (int64_t)row * keep_pitch;
+  const int tid = threadIdx.x;
+
+  if (k >= T) {
+    for (int i = tid; i < T; i += kTopkThreads) out[i] = i;
+    return;
+  }
+
+  // ---- radix select of the k-th largest key, 8 bits per pass from the top.
+  uint32_t prefix = 0, mask = 0, remaining = (uint32_t)k;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < T; i += kTopkThreads) {
+      const uint32_t key = float_key(x[i]);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    // suffix[d] = number of candidates with digit >= d (Hillis-Steele over 256 bins).
+    if (tid < 256) scan[tid] = hist[tid];
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      uint32_t v = 0;
+      if (tid < 256 && tid + off < 256) v = scan[tid + off];
+      __syncthreads();
+      if (tid < 256) scan[tid] += v;
+      __syncthreads();
+    }
+    if (tid < 256) {
+      const uint32_t ge = scan[tid];
+      const uint32_t gt = (tid < 255) ? scan[tid + 1] : 0u;
+      if (gt < remaining && remaining <= ge) {   // exactly one digit satisfies this
+        sh_prefix = prefix | ((uint32_t)tid << shift);
+        sh_remaining = remaining - gt;
+      }
+    }
+    __syncthreads();
+    prefix = sh_prefix;
+    remaining = sh_remaining;
+    mask |= 255u << shift;
+    __syncthreads();
+  }
+  const uint32_t thr = prefix;        // key of the k-th largest element
+  const uint32_t need_eq = remaining; // how many elements equal to it are kept (lowest index first)
+
+  // ---- ordered compaction: every thread owns a contiguous chunk of the row.
+  const int chunk = ceil_div(T, kTopkThreads);
+  const int c0 = min(tid * chunk, T), c1 = min(c0 + chunk, T);
+  uint32_t g = 0, e = 0;
+  for (int i = c0; i < c1; ++i) {
+    const uint32_t key = float_key(x[i]);
+    g += key > thr;
+    e += key == thr;
+  }
+  cnt_gt[tid] = g;
+  cnt_eq[tid] = e;
+  __syncthreads();
+  // Exclusive scan of both counters over threads (Hillis-Steele, inclusive then shift).
+  for (int off = 1; off < kTopkThreads; off <<= 1) {
+    uint32_t vg = 0, ve = 0;
+    if (tid >= off) { vg = cnt_gt[tid - off]; ve = cnt_eq[tid - off]; }
+    __syncthreads();
+    cnt_gt[tid] += vg;
+    cnt_eq[tid] += ve;
+    __syncthreads();
+  }
+  uint32_t gt_before = cnt_gt[tid] - g;
+  uint32_t eq_before = cnt_eq[tid] - e;
+  uint32_t pos = gt_before + min(eq_before, need_eq);
+  for (int i = c0; i < c1; ++i) {
+    const uint32_t key = float_key(x[i]);
+    if (key > thr) {
+      out[pos++] = i;
+    } else if (key == thr) {
+      if (eq_before < need_eq) out[pos++] = i;
+      ++eq_before;
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
+                            const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry,
+                            int32_t* keep, int keep_pitch, hipStream_t s) {
+  if (num_rows <= 0) return hipSuccess;
+  hipLaunchKernelGGL(topk_rows_kernel, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
+                     row_ks, rows_per_entry, keep, keep_pitch);
+  return hipGetLastError();
+}
+
+hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
+  const int n = a.B * a.L * a.A;
+  hipLaunchKernelGGL(finalize_stats_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s, a.partial, a.seq_lens,
+                     a.B, a.L, a.A, a.num_tiles, a.normalize, a.mustd);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+
+  CombineArgs c{};
+  c.raw = a.raw;
+  c.mustd = a.mustd;
+  c.seq_lens = a.seq_lens;
+  c.prefill_lens = a.prefill_lens;
+  c.fin = a.fin;
+  c.raw_stride_layer = a.raw_stride_layer;
+  c.raw_stride_token = a.raw_stride_token;
+  c.raw_stride_head = a.raw_stride_head;
+  c.B = a.B; c.L = a.L; c.Hkv = a.Hkv; c.A = a.A; c.G = a.G; c.Tmax = a.Tmax;
+  c.window_size = a.window_size;
+  c.protect_prefill = a.protect_prefill;
+  c.group_reduce = a.group_reduce;
+  c.layer_reduce = a.layer_reduce;
+  c.shared = a.shared;
+  c.rows_per_seq = a.shared ? 1 : a.Hkv;
+  c.tokens_per_wg = 256 / c.rows_per_seq;
+  const bool per_layer = a.layer_reduce < 0;
+  dim3 grid(ceil_div(a.Tmax, c.tokens_per_wg), per_layer ? a.L : 1, a.B);
+  const size_t smem = (size_t)c.rows_per_seq * c.tokens_per_wg * sizeof(float);
+  hipLaunchKernelGGL(combine_kernel, grid, dim3(256), smem, s, c);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+
+  const int rows_per_entry = c.rows_per_seq * (per_layer ? a.L : 1);
+  return launch_topk_rows(a.fin, a.Tmax, a.B * rows_per_entry, a.seq_lens, a.budgets, rows_per_entry, a.keep,
+                          a.max_budget, s);
+}
+
+}  // namespace tri

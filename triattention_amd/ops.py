@@ -1,0 +1,355 @@
+"""Tensor-level wrappers over the C ABI: device pointers, strides and the current
+HIP stream are taken from torch tensors; every byte of arithmetic on the hot path
+runs in the gfx950 kernels of libtriattention_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Sequence
+
+import torch
+
+from . import _lib
+from ._lib import (KV_BF16, KV_FP16, KV_FP8_E4M3, REDUCE_MAX, REDUCE_MEAN, REDUCE_NONE, ROPE_HALF,
+                   ROPE_INTERLEAVED, Batch, KvLayout, ScoreParams, SelectParams)
+
+_DTYPES = {torch.bfloat16: KV_BF16, torch.float16: KV_FP16}
+if hasattr(torch, "float8_e4m3fn"):
+    _DTYPES[torch.float8_e4m3fn] = KV_FP8_E4M3
+
+
+def _stream() -> int:
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else int(t.data_ptr())
+
+
+def _i32(values, device) -> torch.Tensor:
+    if isinstance(values, torch.Tensor):
+        return values.to(device=device, dtype=torch.int32).contiguous()
+    return torch.tensor([int(v) for v in values], dtype=torch.int32, device=device)
+
+
+def split_kv_axes(kv_cache: torch.Tensor, kv_axis: int | None = None):
+    """K and V views [num_blocks, block_size, H, D] of a 5-D vLLM cache tensor.
+
+    Accepts [2, nb, bs, H, D] and [nb, 2, bs, H, D]; when both leading dims are 2 the
+    caller must say which one is the K/V axis (runtime/kv_compaction.py:94-117).
+    """
+    if kv_cache.ndim != 5:
+        raise ValueError(f"Unsupported kv_cache ndim={kv_cache.ndim}, expect 5")
+    d0, d1 = int(kv_cache.shape[0]) == 2, int(kv_cache.shape[1]) == 2
+    if d0 and d1:
+        if kv_axis not in (0, 1):
+            raise ValueError(
+                "Ambiguous KV layout for compaction: both dim0 and dim1 have size 2. "
+                "Register an explicit layout hint via register_kv_layout_axis_hint(...).")
+        d0, d1 = kv_axis == 0, kv_axis == 1
+    if d0:
+        return kv_cache[0], kv_cache[1]
+    if d1:
+        return kv_cache[:, 0], kv_cache[:, 1]
+    raise ValueError("Unsupported KV layout for compaction: expected a dimension with size 2")
+
+
+class PagedKV:
+    """Key/value storage of the layers of one KV-cache group, as the kernels see it."""
+
+    def __init__(self, k_views: Sequence[torch.Tensor], v_views: Sequence[torch.Tensor] | None = None,
+                 rope_style: str = "half", k_scales: Sequence[torch.Tensor] | None = None,
+                 v_scales: Sequence[torch.Tensor] | None = None):
+        if not k_views:
+            raise ValueError("no layers")
+        k0 = k_views[0]
+        if k0.ndim != 4:
+            raise ValueError(f"expected [num_blocks, block_size, H, D] views, got {tuple(k0.shape)}")
+        if not k0.is_cuda:
+            raise RuntimeError("the scoring/compaction kernels need device memory; got a CPU tensor "
+                               "(there is no CPU fallback)")
+        if k0.dtype not in _DTYPES:
+            raise TypeError(f"unsupported KV dtype {k0.dtype}")
+        if k0.stride(3) != 1:
+            raise ValueError("head_dim must be contiguous")
+        views = list(k_views) + (list(v_views) if v_views is not None else [])
+        for t in views:
+            if t.shape != k0.shape or t.stride() != k0.stride() or t.dtype != k0.dtype or t.device != k0.device:
+                raise ValueError("all layers must share shape, strides, dtype and device")
+            if t.data_ptr() % 16:
+                raise ValueError("KV base pointers must be 16-byte aligned")
+        if rope_style not in ("half", "interleaved"):
+            raise ValueError(f"rope_style must be 'half' or 'interleaved', got {rope_style!r}")
+        self.device = k0.device
+        self.dtype = k0.dtype
+        self.num_layers = len(k_views)
+        self.num_blocks, self.block_size, self.num_kv_heads, self.head_dim = (int(x) for x in k0.shape)
+        self.rope_style = rope_style
+        self._keep = (list(k_views), list(v_views) if v_views is not None else None, k_scales, v_scales)
+        self.k_ptrs = torch.tensor([t.data_ptr() for t in k_views], dtype=torch.int64, device=self.device)
+        self.v_ptrs = (torch.tensor([t.data_ptr() for t in v_views], dtype=torch.int64, device=self.device)
+                       if v_views is not None else None)
+        self.ks_ptrs = self.vs_ptrs = None
+        if self.dtype == getattr(torch, "float8_e4m3fn", None):
+            if k_scales is None:
+                raise ValueError("fp8 cache needs per-(token, head) scales")
+            self.ks_ptrs = torch.tensor([t.data_ptr() for t in k_scales], dtype=torch.int64, device=self.device)
+            if v_scales is not None:
+                self.vs_ptrs = torch.tensor([t.data_ptr() for t in v_scales], dtype=torch.int64, device=self.device)
+        self.struct = KvLayout(
+            num_layers=self.num_layers, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+            block_size=self.block_size, kv_dtype=_DTYPES[self.dtype],
+            rope_style=ROPE_INTERLEAVED if rope_style == "interleaved" else ROPE_HALF,
+            stride_block=int(k0.stride(0)), stride_token=int(k0.stride(1)), stride_head=int(k0.stride(2)),
+            k_layers=_ptr(self.k_ptrs), v_layers=_ptr(self.v_ptrs),
+            k_scale_layers=_ptr(self.ks_ptrs), v_scale_layers=_ptr(self.vs_ptrs))
+
+    @classmethod
+    def from_kv_caches(cls, kv_caches: Sequence[torch.Tensor], rope_style: str = "half",
+                       kv_axis: int | None = None) -> "PagedKV":
+        ks, vs = zip(*(split_kv_axes(t, kv_axis) for t in kv_caches))
+        return cls(ks, vs, rope_style)
+
+    @classmethod
+    def from_dense_keys(cls, key_states: torch.Tensor, rope_style: str = "half") -> "PagedKV":
+        """[B, H, T, D] keys as one 'block' per sequence (score-only)."""
+        if key_states.ndim != 4:
+            raise ValueError(f"expected [B, H, T, D], got {tuple(key_states.shape)}")
+        view = key_states.permute(0, 2, 1, 3)          # [B, T, H, D], no copy
+        return cls([view], None, rope_style)
+
+
+class StepBatch:
+    """The sequences of one compression step, on the device."""
+
+    def __init__(self, device, seq_lens, round_start=None, budgets=None, block_tables=None,
+                 prefill_lens=None):
+        self.device = device
+        self.seq_lens_host = [int(x) for x in (seq_lens.tolist() if isinstance(seq_lens, torch.Tensor) else seq_lens)]
+        self.num_seqs = len(self.seq_lens_host)
+        if self.num_seqs == 0:
+            raise ValueError("empty batch")
+        self.seq_lens = _i32(self.seq_lens_host, device)
+        self.round_start = _i32(round_start if round_start is not None else self.seq_lens_host, device)
+        self.prefill_lens = _i32(prefill_lens, device) if prefill_lens is not None else None
+        self.budgets_host = None
+        self.budgets = None
+        if budgets is not None:
+            b = budgets.tolist() if isinstance(budgets, torch.Tensor) else budgets
+            if isinstance(b, int):
+                b = [b] * self.num_seqs
+            self.budgets_host = [min(int(x), t) for x, t in zip(b, self.seq_lens_host)]
+            self.budgets = _i32(self.budgets_host, device)
+        self.block_table = None
+        pitch = 0
+        if block_tables is not None:
+            if isinstance(block_tables, torch.Tensor):
+                bt = block_tables.to(device=device, dtype=torch.int32)
+                if bt.ndim == 1:
+                    bt = bt.unsqueeze(0)
+                self.block_table = bt.contiguous()
+            else:
+                pitch = max(len(r) for r in block_tables)
+                rows = [list(map(int, r)) + [0] * (pitch - len(r)) for r in block_tables]
+                self.block_table = torch.tensor(rows, dtype=torch.int32, device=device)
+            pitch = int(self.block_table.shape[1])
+            if int(self.block_table.shape[0]) != self.num_seqs:
+                raise ValueError("block table rows != number of sequences")
+        self.max_seq_len = max(self.seq_lens_host)
+        self.max_budget = max(self.budgets_host) if self.budgets_host else 0
+        self.struct = Batch(
+            num_seqs=self.num_seqs, max_seq_len=self.max_seq_len, max_budget=self.max_budget,
+            block_table_pitch=pitch, block_table=_ptr(self.block_table), seq_lens=_ptr(self.seq_lens),
+            round_start=_ptr(self.round_start), prefill_lens=_ptr(self.prefill_lens),
+            budgets=_ptr(self.budgets))
+
+    def check_capacity(self, block_size: int) -> None:
+        """Host-side bounds check: every sequence owns enough blocks for its tokens."""
+        if self.block_table is None:
+            return
+        pitch = int(self.block_table.shape[1])
+        for t in self.seq_lens_host:
+            if (t + block_size - 1) // block_size > pitch:
+                raise IndexError(f"sequence of {t} tokens needs more than {pitch} blocks of {block_size}")
+
+
+@dataclass
+class ScoreConfig:
+    folded: torch.Tensor        # [L, A, 3, F] fp32 from fold_stats
+    omega: torch.Tensor         # [F] fp32
+    offsets: torch.Tensor       # [NO] fp32
+    aggregation: str = "mean"
+
+    @property
+    def num_score_heads(self) -> int:
+        return int(self.folded.shape[1])
+
+    def struct(self) -> ScoreParams:
+        return ScoreParams(num_score_heads=self.num_score_heads, num_offsets=int(self.offsets.numel()),
+                           aggregation=REDUCE_MAX if self.aggregation == "max" else REDUCE_MEAN,
+                           folded=_ptr(self.folded), omega=_ptr(self.omega), offsets=_ptr(self.offsets))
+
+
+@dataclass
+class SelectConfig:
+    normalize: bool = True
+    window_size: int = 128
+    protect_prefill: bool = False
+    group_reduce: str = "max"
+    layer_reduce: str | None = "mean"    # None: one keep set per layer
+    shared: bool = False
+
+    def struct(self) -> SelectParams:
+        lr = REDUCE_NONE if self.layer_reduce is None else (REDUCE_MAX if self.layer_reduce == "max" else REDUCE_MEAN)
+        return SelectParams(normalize=int(self.normalize), window_size=int(self.window_size),
+                            protect_prefill=int(self.protect_prefill),
+                            group_reduce=REDUCE_MAX if self.group_reduce == "max" else REDUCE_MEAN,
+                            layer_reduce=lr, shared=int(self.shared))
+
+
+def fold_stats(q_mean_complex: torch.Tensor, q_abs_mean: torch.Tensor, freq_scale_sq: torch.Tensor,
+               disable_mlr: bool = False, disable_trig: bool = False) -> torch.Tensor:
+    """[L, A, F, 2], [L, A, F], [L, A, F] device fp32 -> folded [L, A, 3, F]."""
+    lib = _lib.load()
+    if not q_mean_complex.is_cuda:
+        raise RuntimeError("fold_stats needs device tensors (there is no CPU fallback)")
+    qr = q_mean_complex[..., 0].to(torch.float32).contiguous()
+    qi = q_mean_complex[..., 1].to(torch.float32).contiguous()
+    qa = q_abs_mean.to(torch.float32).contiguous()
+    fs = freq_scale_sq.to(torch.float32).contiguous()
+    if qr.ndim != 3 or qa.shape != qr.shape or fs.shape != qr.shape:
+        raise ValueError("stats must be [L, A, F]")
+    L, A, F = (int(x) for x in qr.shape)
+    out = torch.empty(L, A, 3, F, dtype=torch.float32, device=qr.device)
+    _lib.check(lib.tri_fold_stats(_ptr(qr), _ptr(qi), _ptr(qa), _ptr(fs), L, A, F, int(disable_mlr),
+                                  int(disable_trig), _ptr(out), _stream()))
+    return out
+
+
+class Workspace:
+    """Device scratch for one (layout, batch, score config); reusable across steps."""
+
+    def __init__(self, kv: PagedKV, batch: StepBatch, sc: ScoreConfig):
+        lib = _lib.load()
+        sp = sc.struct()
+        self.bytes = int(lib.tri_workspace_bytes(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp)))
+        if self.bytes == 0:
+            raise ValueError("invalid layout / batch / score parameters: " +
+                             lib.tri_last_error().decode("utf-8", "replace"))
+        self.buf = torch.empty(self.bytes + 256, dtype=torch.uint8, device=kv.device)
+        off = (-self.buf.data_ptr()) % 256
+        self.ptr = self.buf.data_ptr() + off
+
+    def fits(self, kv, batch, sc) -> bool:
+        sp = sc.struct()
+        need = int(_lib.load().tri_workspace_bytes(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp)))
+        return 0 < need <= self.bytes
+
+
+def _check_devices(kv: PagedKV, sc: ScoreConfig):
+    for t in (sc.folded, sc.omega, sc.offsets):
+        if t.device != kv.device or t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("score parameters must be contiguous fp32 tensors on the cache's device")
+    if int(sc.folded.shape[0]) != kv.num_layers or int(sc.folded.shape[3]) != kv.head_dim // 2:
+        raise ValueError(f"folded stats {tuple(sc.folded.shape)} do not match {kv.num_layers} layers / "
+                         f"head_dim {kv.head_dim}")
+
+
+def score_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, ws: Workspace | None = None,
+                head_major: bool = False):
+    """Raw scores of every key.  Returns (raw, ws); raw is [B, L, Tmax, A] fp32, or
+    [B, L, A, Tmax] when head_major (the reference's [batch, heads, seq] order)."""
+    lib = _lib.load()
+    _check_devices(kv, sc)
+    batch.check_capacity(kv.block_size)
+    ws = ws if ws is not None and ws.fits(kv, batch, sc) else Workspace(kv, batch, sc)
+    B, L, T, A = batch.num_seqs, kv.num_layers, batch.max_seq_len, sc.num_score_heads
+    if head_major:
+        raw = torch.empty(B, L, A, T, dtype=torch.float32, device=kv.device)
+        strides = (A * T, 1, T)
+    else:
+        raw = torch.empty(B, L, T, A, dtype=torch.float32, device=kv.device)
+        strides = (T * A, A, 1)
+    sp = sc.struct()
+    _lib.check(lib.tri_score_paged(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), _ptr(raw),
+                                   strides[0], strides[1], strides[2], ws.ptr, ws.bytes, _stream()))
+    return raw, ws
+
+
+def select(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, raw: torch.Tensor,
+           ws: Workspace, head_major: bool = False, want_scores: bool = False):
+    """keep int32 [rows, max_budget] (ascending) and optionally the selection scores."""
+    lib = _lib.load()
+    if batch.budgets is None:
+        raise ValueError("batch has no budgets")
+    B, L, T, A = batch.num_seqs, kv.num_layers, batch.max_seq_len, sc.num_score_heads
+    strides = (A * T, 1, T) if head_major else (T * A, A, 1)
+    rows = B * (L if sel.layer_reduce is None else 1) * (1 if sel.shared else kv.num_kv_heads)
+    keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+    fin = torch.empty(rows, T, dtype=torch.float32, device=kv.device) if want_scores else None
+    sp, ss = sc.struct(), sel.struct()
+    _lib.check(lib.tri_select(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss), _ptr(raw),
+                              strides[0], strides[1], strides[2], _ptr(fin), _ptr(keep), ws.ptr, ws.bytes,
+                              _stream()))
+    return keep, fin
+
+
+def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] | None = None) -> torch.Tensor:
+    """Ascending int32 indices of the k largest entries of every row of a 2-D fp32 tensor."""
+    lib = _lib.load()
+    if not scores.is_cuda:
+        raise RuntimeError("topk_rows needs a device tensor (there is no CPU fallback)")
+    if scores.ndim != 2 or scores.dtype != torch.float32 or scores.stride(1) != 1:
+        raise ValueError("scores must be a 2-D fp32 tensor with contiguous rows")
+    R, T = (int(x) for x in scores.shape)
+    ks = [int(k)] * R if isinstance(k, int) else [int(x) for x in k]
+    ls = [T] * R if lens is None else [int(x) for x in lens]
+    kmax = max(max(ks), 1)
+    keep = torch.empty(R, kmax, dtype=torch.int32, device=scores.device)
+    lens_t, ks_t = _i32(ls, scores.device), _i32(ks, scores.device)
+    _lib.check(lib.tri_topk_rows(_ptr(scores), int(scores.stride(0)), R, _ptr(lens_t), _ptr(ks_t), 1, T,
+                                 _ptr(keep), kmax, _stream()))
+    return keep
+
+
+def compact(kv: PagedKV, batch: StepBatch, keep: torch.Tensor, keep_per_layer: bool = False,
+            shared: bool = False, full_permutation: bool = False) -> None:
+    """In-place compaction of K and V of every layer.  keep: ascending int32 rows."""
+    lib = _lib.load()
+    if batch.budgets is None or batch.block_table is None:
+        raise ValueError("compaction needs budgets and block tables")
+    batch.check_capacity(kv.block_size)
+    rows = batch.num_seqs * (kv.num_layers if keep_per_layer else 1) * (1 if shared else kv.num_kv_heads)
+    if keep.dtype != torch.int32 or not keep.is_contiguous() or keep.device != kv.device:
+        raise ValueError("keep must be a contiguous int32 tensor on the cache's device")
+    if keep.numel() != rows * batch.max_budget:
+        raise ValueError(f"keep has {keep.numel()} entries, expected {rows} x {batch.max_budget}")
+    if full_permutation:
+        need = int(lib.tri_compact_full_staging_bytes(C.byref(kv.struct), C.byref(batch.struct)))
+        staging = torch.empty(need + 16, dtype=torch.uint8, device=kv.device)
+        _lib.check(lib.tri_compact_paged_full(C.byref(kv.struct), C.byref(batch.struct), _ptr(keep),
+                                              int(keep_per_layer), int(shared), _ptr(staging), need, _stream()))
+        # The staging tensor is released to torch's caching allocator, which keeps it
+        # alive until work already queued on this stream has finished with it.
+        return
+    _lib.check(lib.tri_compact_paged(C.byref(kv.struct), C.byref(batch.struct), _ptr(keep),
+                                     int(keep_per_layer), int(shared), _stream()))
+
+
+def compress_step(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig,
+                  ws: Workspace | None = None, keep: torch.Tensor | None = None):
+    """score + select + compact for every layer of every sequence.  Returns (keep, ws)."""
+    lib = _lib.load()
+    _check_devices(kv, sc)
+    if batch.budgets is None or batch.block_table is None:
+        raise ValueError("compress_step needs budgets and block tables")
+    batch.check_capacity(kv.block_size)
+    ws = ws if ws is not None and ws.fits(kv, batch, sc) else Workspace(kv, batch, sc)
+    rows = batch.num_seqs * (kv.num_layers if sel.layer_reduce is None else 1) * (1 if sel.shared else kv.num_kv_heads)
+    if keep is None:
+        keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+    sp, ss = sc.struct(), sel.struct()
+    _lib.check(lib.tri_compress_step(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss),
+                                     _ptr(keep), ws.ptr, ws.bytes, _stream()))
+    return keep, ws
