@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV compression step (score + select + compact) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch of synthetic paged KV: every layer
+of every sequence is scored, the budget is selected per KV head, K and V are compacted
+in place.  Inputs are resident in HBM before the timed region; compaction is
+destructive, so the blocks it overwrites are restored between steps outside the timed
+region (each step is timed with HIP events on the stream the kernels run on).
+Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=1, help="BASELINE.json config index (default 1)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-layers", type=int, default=2, help="layers of one sequence the CPU baseline scores")
+    return ap.parse_args()
+
+
+def cpu_baseline(w, layers: int):
+    """The CPU oracle (a port of the reference's PyTorch path) on a bounded sample:
+    one sequence, `layers` layers, same shapes and seeded distributions."""
+    from oracle import compaction as ocp
+    from oracle import scoring as osc
+    from oracle import selection as osel
+    from triattention_amd import synth
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    sample = w.scaled(seq_lens=(w.seq_lens[0],), num_layers=layers, kv_dtype="bf16" if w.kv_dtype == "fp8" else w.kv_dtype)
+    tables = synth.make_block_tables(sample)
+    caches = synth.make_kv_pool(sample, tables, "cpu")
+    qc, qa = synth.make_stats(sample, "cpu")
+    omega, offsets = synth.rope_inv_freq(sample), synth.geometric_offsets()
+    fs = torch.ones(layers, sample.num_q_heads, sample.head_dim // 2)
+    t = sample.seq_lens[0]
+    g = sample.num_q_heads // sample.num_kv_heads
+    t0 = time.perf_counter()
+    raw = []
+    for l in range(layers):
+        kc, _ = ocp.split_kv(caches[l])
+        keys = ocp.gather_dense(kc, tables[0], sample.block_size, 0, t)[0].float().repeat_interleave(g, dim=0)
+        raw.append(osc.raw_scores(keys, qc[l], qa[l], omega, offsets, fs[l], t))
+    keep, _ = osel.group_keep_per_head(raw, sample.num_kv_heads, sample.budget, window_size=sample.window_size,
+                                       chunk_tokens=osel.score_chunk_tokens(sample.block_size, t))
+    for l in range(layers):
+        ocp.compact_per_head(caches[l], tables[0], sample.block_size, keep, t, full_permutation=True)
+    dt = time.perf_counter() - t0
+    # one "key" is one cached token across ALL layers of the model: scale the sample's layer count up
+    keys_per_s = t / (dt * w.num_layers / layers)
+    return {"value": keys_per_s, "unit": "keys/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 sequence x {t} tokens x {layers} of {w.num_layers} layers, {dt:.2f} s on the host; "
+                      f"rate scaled to all {w.num_layers} layers"}
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the path shards by sequence and KV head with no exchange, "
+              f"and this build has no multi-GPU leg (got --gpus {args.gpus}).", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
+        return 2
+
+    from triattention_amd import ops, synth
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = synth.config(args.config)
+    t_setup = time.perf_counter()
+    tables = synth.make_block_tables(w)
+    pool = synth.make_kv_pool(w, tables, dev)
+    if w.kv_dtype == "fp8":
+        caches, k_scales, v_scales = pool
+        kv = ops.PagedKV([c[0] for c in caches], [c[1] for c in caches], w.rope_style, k_scales, v_scales)
+    else:
+        caches = pool
+        kv = ops.PagedKV.from_kv_caches(caches, w.rope_style)
+    qc, qa = synth.make_stats(w, dev)
+    fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2, device=dev)
+    sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev))
+    sel = ops.SelectConfig(window_size=w.window_size)
+    batch = ops.StepBatch(dev, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=tables)
+    ws = ops.Workspace(kv, batch, sc)
+    keep = torch.empty(w.num_seqs * w.num_kv_heads, batch.max_budget, dtype=torch.int32, device=dev)
+
+    # Blocks that compaction overwrites (the first ceil(k/bs) of every sequence), saved for restore.
+    nkeep_blocks = (w.budget + w.block_size - 1) // w.block_size
+    ids = torch.tensor([b for tbl in tables for b in tbl[:nkeep_blocks]], device=dev, dtype=torch.long)
+    saved = [c[:, ids].clone() for c in caches]
+    saved_scales = None
+    if w.kv_dtype == "fp8":
+        slot = (ids.unsqueeze(1) * w.block_size + torch.arange(w.block_size, device=dev)).flatten()
+        saved_scales = [(ks[slot].clone(), vs[slot].clone()) for ks, vs in zip(k_scales, v_scales)]
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t_setup
+
+    def restore():
+        for i, c in enumerate(caches):
+            c[:, ids] = saved[i]
+            if saved_scales is not None:
+                k_scales[i][slot] = saved_scales[i][0]
+                v_scales[i][slot] = saved_scales[i][1]
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
+        if events is not None:
+            events[1].record()
+        ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
+        if events is not None:
+            events[2].record()
+        ops.compact(kv, batch, keep)
+        if events is not None:
+            events[3].record()
+
+    raw_buf = torch.empty(w.num_seqs, w.num_layers, batch.max_seq_len, w.num_q_heads, dtype=torch.float32, device=dev)
+
+    for _ in range(args.warmup):
+        step()
+        restore()
+    torch.cuda.synchronize()
+
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    wall0 = time.perf_counter()
+    for i in range(args.steps):
+        torch.cuda.synchronize()
+        step(evs[i])
+        torch.cuda.synchronize()
+        if i + 1 < args.steps:
+            restore()
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - wall0
+
+    ms = lambda a, b: a.elapsed_time(b)
+    step_ms = [ms(e[0], e[3]) for e in evs]
+    score_ms = [ms(e[0], e[1]) for e in evs]
+    select_ms = [ms(e[1], e[2]) for e in evs]
+    compact_ms = [ms(e[2], e[3]) for e in evs]
+    mean = lambda xs: sum(xs) / len(xs)
+    ms_per_step = mean(step_ms)
+    total_keys = sum(w.seq_lens)
+    algo = w.algorithmic_bytes()
+    keys_per_s = total_keys / (ms_per_step * 1e-3)
+    step_gbs = algo["total"] / (ms_per_step * 1e-3) / 1e9
+    score_gbs = algo["score"] / (mean(score_ms) * 1e-3) / 1e9
+    compact_gbs = algo["compact"] / (mean(compact_ms) * 1e-3) / 1e9
+
+    out = {
+        "metric": "keys scored+compacted/sec & achieved HBM GB/s (% peak), Qwen3-8B 16k ctx",
+        "value": keys_per_s,
+        "unit": "keys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": w.name, "layers": w.num_layers, "sequences": w.num_seqs,
+                   "tokens_per_sequence": max(w.seq_lens), "budget": w.budget, "kv_heads": w.num_kv_heads,
+                   "q_heads": w.num_q_heads, "head_dim": w.head_dim, "block_size": w.block_size,
+                   "kv_dtype": w.kv_dtype},
+        "achieved_gbs": step_gbs,
+        "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
+        "algorithmic_bytes": algo,
+        "stage_ms": {"score": mean(score_ms), "select": mean(select_ms), "compact": mean(compact_ms)},
+        "stage_gbs": {"score": score_gbs, "compact": compact_gbs},
+        "key_vectors_per_s": total_keys * w.num_layers * w.num_kv_heads / (ms_per_step * 1e-3),
+        "timed_region_wall_s": wall_s,
+        "setup_s": setup_s,
+        "roofline": {"kernel": "score_mean_kernel", "bound": "hbm", "achieved": score_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS, "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        del saved, caches, pool
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(w, args.cpu_layers)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

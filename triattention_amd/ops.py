@@ -257,7 +257,7 @@ def _check_devices(kv: PagedKV, sc: ScoreConfig):
 
 
 def score_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, ws: Workspace | None = None,
-                head_major: bool = False):
+                head_major: bool = False, out: torch.Tensor | None = None):
     """Raw scores of every key.  Returns (raw, ws); raw is [B, L, Tmax, A] fp32, or
     [B, L, A, Tmax] when head_major (the reference's [batch, heads, seq] order)."""
     lib = _lib.load()
@@ -265,12 +265,14 @@ def score_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, ws: Workspace | 
     batch.check_capacity(kv.block_size)
     ws = ws if ws is not None and ws.fits(kv, batch, sc) else Workspace(kv, batch, sc)
     B, L, T, A = batch.num_seqs, kv.num_layers, batch.max_seq_len, sc.num_score_heads
-    if head_major:
-        raw = torch.empty(B, L, A, T, dtype=torch.float32, device=kv.device)
-        strides = (A * T, 1, T)
+    shape = (B, L, A, T) if head_major else (B, L, T, A)
+    strides = (A * T, 1, T) if head_major else (T * A, A, 1)
+    if out is not None:
+        if tuple(out.shape) != shape or out.dtype != torch.float32 or not out.is_contiguous() or out.device != kv.device:
+            raise ValueError(f"out must be a contiguous fp32 tensor of shape {shape} on the cache's device")
+        raw = out
     else:
-        raw = torch.empty(B, L, T, A, dtype=torch.float32, device=kv.device)
-        strides = (T * A, A, 1)
+        raw = torch.empty(shape, dtype=torch.float32, device=kv.device)
     sp = sc.struct()
     _lib.check(lib.tri_score_paged(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), _ptr(raw),
                                    strides[0], strides[1], strides[2], ws.ptr, ws.bytes, _stream()))
@@ -278,7 +280,8 @@ def score_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, ws: Workspace | 
 
 
 def select(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, raw: torch.Tensor,
-           ws: Workspace, head_major: bool = False, want_scores: bool = False):
+           ws: Workspace, head_major: bool = False, want_scores: bool = False,
+           keep: torch.Tensor | None = None):
     """keep int32 [rows, max_budget] (ascending) and optionally the selection scores."""
     lib = _lib.load()
     if batch.budgets is None:
@@ -286,7 +289,13 @@ def select(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, ra
     B, L, T, A = batch.num_seqs, kv.num_layers, batch.max_seq_len, sc.num_score_heads
     strides = (A * T, 1, T) if head_major else (T * A, A, 1)
     rows = B * (L if sel.layer_reduce is None else 1) * (1 if sel.shared else kv.num_kv_heads)
-    keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+    if keep is None:
+        keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+    elif (keep.numel() != rows * batch.max_budget or keep.dtype != torch.int32 or not keep.is_contiguous()
+          or keep.device != kv.device):
+        raise ValueError(f"keep must be a contiguous int32 tensor with {rows} x {batch.max_budget} entries")
+    if raw.numel() != B * L * T * A or raw.dtype != torch.float32 or not raw.is_contiguous():
+        raise ValueError("raw must be the contiguous fp32 tensor returned by score_paged for this batch")
     fin = torch.empty(rows, T, dtype=torch.float32, device=kv.device) if want_scores else None
     sp, ss = sc.struct(), sel.struct()
     _lib.check(lib.tri_select(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss), _ptr(raw),
