@@ -8,7 +8,10 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libtriattention_hip.so"
+import os
+
+# TRIATTN_HIP_LIBRARY points at another build of the same ABI (e.g. an instrumented one).
+LIB_PATH = Path(os.environ.get("TRIATTN_HIP_LIBRARY") or Path(__file__).resolve().parent / "libtriattention_hip.so")
 
 TRI_OK = 0
 TRI_ERR_INVALID_ARGUMENT = -1

@@ -158,8 +158,6 @@ int fill_compact(const tri_kv_layout* kv, const tri_batch* batch, const int32_t*
   if (!batch->block_table) return fail(TRI_ERR_INVALID_ARGUMENT, "compaction needs a block table");
   if (!keep) return fail(TRI_ERR_INVALID_ARGUMENT, "keep is NULL");
   const int eb = elem_bytes(kv->kv_dtype);
-  const int chunks_per_slot = (shared ? kv->num_kv_heads : 1) * kv->head_dim * eb / 16;
-  if (chunks_per_slot > 1024) return fail(TRI_ERR_UNSUPPORTED, "a slot of %d bytes exceeds one tile", chunks_per_slot * 16);
   a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
   a.block_size = kv->block_size; a.elem_bytes = eb; a.max_budget = batch->max_budget;
   a.keep_per_layer = keep_per_layer ? 1 : 0; a.shared = shared ? 1 : 0;

@@ -10,7 +10,7 @@ namespace tri {
 
 constexpr int kWave = 64;
 constexpr int kScoreThreads = 256;      // 4 waves per scorer workgroup
-constexpr int kScoreTileTokens = 256;   // tokens of one (sequence, layer) per scorer workgroup
+constexpr int kScoreTileTokens = 512;   // tokens of one (sequence, layer) per scorer workgroup
 constexpr int kQPerPass = 4;            // query heads scored per wave pass
 constexpr int kPairsPerLane = 8;        // frequency pairs held by one lane
 constexpr int kMaxOffsets = 32;

@@ -29,8 +29,10 @@ struct CompactArgs {
   const int32_t* budgets;
   const int32_t* keep;
   int64_t stride_block_b, stride_token_b, stride_head_b;   // bytes
+  uint32_t block_units, token_units, head_units;           // the same strides in 16-byte units
   int B, L, Hkv, block_size, bs_shift, block_table_pitch, max_budget;
   int keep_per_layer, shared;
+  int split_bulk;          // 1: the ordered kernel stops at the first source >= budget
   int chunks_per_row;      // 16-byte chunks of one head row (D * elem_bytes / 16)
   int heads_per_slot;      // shared ? Hkv : 1
   int streams_per_layer;   // 2 * (shared ? 1 : Hkv)
@@ -63,46 +65,129 @@ __global__ __launch_bounds__(kCompactThreads) void compact_kernel(CompactArgs a)
   char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
   const int head0 = a.shared ? 0 : row;
 
+  // Only slots whose source lies inside the kept prefix [0, k) can be overwritten
+  // before they are read; with keep ascending those form a prefix of the list.  The
+  // rest (source >= k) is moved by compact_bulk_kernel, which needs no ordering.
+  if (a.split_bulk) {
+    // keep is ascending: the number of entries below k is the length of that prefix.
+    __shared__ int prefix_len;
+    int below = 0;
+    for (int j = threadIdx.x; j < k; j += kCompactThreads) below += keep[j] < k;
+    if (threadIdx.x == 0) prefix_len = 0;
+    __syncthreads();
+    if (below) atomicAdd(&prefix_len, below);
+    __syncthreads();
+    k = prefix_len;
+    if (k <= 0) return;
+  }
+
   const int chunks_per_slot = a.heads_per_slot * a.chunks_per_row;
-  const int slots_per_tile = kTileChunks / chunks_per_slot;   // >= 1 (checked on the host)
+  const int slots_per_tile = max(kTileChunks / chunks_per_slot, 1);
 
   for (int seg = 0; seg < k; seg += kSegSlots) {
     const int nseg = min(kSegSlots, k - seg);
     __syncthreads();   // previous segment's LDS no longer in use
     for (int i = threadIdx.x; i < nseg; i += kCompactThreads) {
       const int j = seg + i;
-      const int src = keep[j];
-      src_off[i] = slot_offset(a, bt, src);
+      src_off[i] = slot_offset(a, bt, keep[j]);
       dst_off[i] = slot_offset(a, bt, j);
     }
     __syncthreads();
 
     for (int t0 = 0; t0 < nseg; t0 += slots_per_tile) {
-      const int nslots = min(slots_per_tile, nseg - t0);
-      const int nchunks = nslots * chunks_per_slot;
-      uint4 regs[kChunksPerThread];
-      int64_t dsts[kChunksPerThread];
-      bool live[kChunksPerThread];
+      const int nchunks = min(slots_per_tile, nseg - t0) * chunks_per_slot;
+      // A slot wider than a tile is moved in several passes; every pass is read
+      // completely before it is written, and passes of one slot never overlap.
+      for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
+        uint4 regs[kChunksPerThread];
+        int64_t dsts[kChunksPerThread];
+        bool live[kChunksPerThread];
 #pragma unroll
-      for (int c = 0; c < kChunksPerThread; ++c) {
-        const int ci = c * kCompactThreads + threadIdx.x;
-        live[c] = ci < nchunks;
-        if (live[c]) {
-          const int sl = t0 + ci / chunks_per_slot;
-          const int within = ci % chunks_per_slot;
-          const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
-          const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
-          const int64_t so = src_off[sl] + inner;
-          dsts[c] = dst_off[sl] + inner;
-          live[c] = so != dsts[c];            // row already in place
-          if (live[c]) regs[c] = *reinterpret_cast<const uint4*>(base + so);
+        for (int c = 0; c < kChunksPerThread; ++c) {
+          const int ci = c0 + c * kCompactThreads + threadIdx.x;
+          live[c] = ci < nchunks;
+          if (live[c]) {
+            const int sl = t0 + ci / chunks_per_slot;
+            const int within = ci % chunks_per_slot;
+            const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+            const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
+            const int64_t so = src_off[sl] + inner;
+            dsts[c] = dst_off[sl] + inner;
+            live[c] = so != dsts[c];            // row already in place
+            if (live[c]) regs[c] = *reinterpret_cast<const uint4*>(base + so);
+          }
         }
-      }
-      __syncthreads();   // every read of this tile is ordered before any write of it
+        __syncthreads();   // every read of this tile is ordered before any write of it
 #pragma unroll
-      for (int c = 0; c < kChunksPerThread; ++c)
-        if (live[c]) *reinterpret_cast<uint4*>(base + dsts[c]) = regs[c];
+        for (int c = 0; c < kChunksPerThread; ++c)
+          if (live[c]) *reinterpret_cast<uint4*>(base + dsts[c]) = regs[c];
+      }
     }
+  }
+}
+
+// Slots whose source token lies at or beyond the budget: sources (>= k) and
+// destinations (< k) cannot overlap, so this is a flat gather copy.  One workgroup
+// moves a tile of destination slots for all heads, i.e. whole contiguous token rows.
+// Offsets are kept in 16-byte units so the per-row index arithmetic stays 32-bit.
+__device__ __forceinline__ uint32_t slot_units(const CompactArgs& a, const int32_t* bt, int tok) {
+  const int lb = a.bs_shift >= 0 ? (tok >> a.bs_shift) : (tok / a.block_size);
+  const int in_off = tok - lb * a.block_size;
+  return (uint32_t)bt[lb] * a.block_units + (uint32_t)in_off * a.token_units;
+}
+
+__global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactArgs a) {
+  int sidx = blockIdx.y;
+  const int kv = sidx % 2; sidx /= 2;
+  const int l = sidx % a.L;
+  const int b = sidx / a.L;
+  int k = a.budgets[b];
+  const int T = a.seq_lens[b];
+  if (k > T) k = T;
+  const int lists = a.shared ? 1 : a.Hkv;
+  const int chunks_per_entry = a.heads_per_slot * a.chunks_per_row;
+  const int slots_per_tile = max(kTileChunks / (lists * chunks_per_entry), 1);
+  const int j0 = blockIdx.x * slots_per_tile;
+  if (j0 >= k) return;
+  const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * lists * a.max_budget;
+  const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
+  char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
+  const int nchunks = min(slots_per_tile, k - j0) * lists * chunks_per_entry;
+
+  // Three dependent lookups per chunk (keep -> block table -> row).  Each level is
+  // issued for all of a thread's chunks before the next one, without branches: idle
+  // chunks are clamped onto valid entries and only their final store is masked.
+  for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
+    bool live[kChunksPerThread];
+    int jj[kChunksPerThread], src[kChunksPerThread];
+    uint32_t inner[kChunksPerThread];
+#pragma unroll
+    for (int c = 0; c < kChunksPerThread; ++c) {
+      const int ci = c0 + c * kCompactThreads + threadIdx.x;
+      live[c] = ci < nchunks;
+      const int cic = live[c] ? ci : 0;
+      const int e = cic / chunks_per_entry, within = cic % chunks_per_entry;
+      const int h = e % lists;
+      jj[c] = j0 + e / lists;
+      const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+      inner[c] = (uint32_t)((a.shared ? 0 : h) + hh) * a.head_units + (uint32_t)cc;
+      src[c] = keep[(int64_t)h * a.max_budget + jj[c]];
+    }
+    uint32_t so[kChunksPerThread], dsto[kChunksPerThread];
+#pragma unroll
+    for (int c = 0; c < kChunksPerThread; ++c) {
+      live[c] = live[c] && src[c] >= k;
+      const int sc = live[c] ? src[c] : jj[c];           // idle chunk: read its own destination row
+      so[c] = slot_units(a, bt, sc) + inner[c];
+      dsto[c] = slot_units(a, bt, jj[c]) + inner[c];
+    }
+    uint4 regs[kChunksPerThread];
+#pragma unroll
+    for (int c = 0; c < kChunksPerThread; ++c)
+      regs[c] = *reinterpret_cast<const uint4*>(base + ((uint64_t)so[c] << 4));
+#pragma unroll
+    for (int c = 0; c < kChunksPerThread; ++c)
+      if (live[c]) *reinterpret_cast<uint4*>(base + ((uint64_t)dsto[c] << 4)) = regs[c];
   }
 }
 
@@ -246,6 +331,9 @@ CompactArgs make_args(const CompactLaunch& a) {
   c.stride_block_b = a.stride_block * a.elem_bytes;
   c.stride_token_b = a.stride_token * a.elem_bytes;
   c.stride_head_b = a.stride_head * a.elem_bytes;
+  c.block_units = (uint32_t)(c.stride_block_b / 16);
+  c.token_units = (uint32_t)(c.stride_token_b / 16);
+  c.head_units = (uint32_t)(c.stride_head_b / 16);
   c.B = a.B; c.L = a.L; c.Hkv = a.Hkv;
   c.block_size = a.block_size;
   c.bs_shift = -1;
@@ -255,6 +343,7 @@ CompactArgs make_args(const CompactLaunch& a) {
   c.max_budget = a.max_budget;
   c.keep_per_layer = a.keep_per_layer;
   c.shared = a.shared;
+  c.split_bulk = 1;
   c.chunks_per_row = a.D * a.elem_bytes / 16;
   c.heads_per_slot = a.shared ? a.Hkv : 1;
   c.streams_per_layer = 2 * (a.shared ? 1 : a.Hkv);
@@ -285,7 +374,18 @@ hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
   const CompactArgs c = make_args(a);
   const int streams = a.B * a.L * c.streams_per_layer;
   if (streams <= 0 || a.max_budget <= 0) return hipSuccess;
+  // Ordered pass over the slots whose sources lie inside the kept prefix, then the
+  // unordered bulk pass over the rest; the first must finish reading before the second
+  // writes, which stream order guarantees.
   hipLaunchKernelGGL(compact_kernel, dim3(streams), dim3(kCompactThreads), 0, s, c);
+  if (c.split_bulk) {
+    hipError_t e0 = hipGetLastError();
+    if (e0 != hipSuccess) return e0;
+    const int lists = a.shared ? 1 : a.Hkv;
+    const int slots_per_tile = kTileChunks / (lists * c.heads_per_slot * c.chunks_per_row);
+    dim3 grid(ceil_div(a.max_budget, slots_per_tile > 0 ? slots_per_tile : 1), a.B * a.L * 2);
+    hipLaunchKernelGGL(compact_bulk_kernel, grid, dim3(kCompactThreads), 0, s, c);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || !a.has_scales) return e;
   return launch_scales(a, s);

@@ -68,6 +68,13 @@ __device__ __forceinline__ float elem_hi<TRI_KV_FP16>(uint32_t w) {
   return (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
 }
 
+// Pointers fetched from the per-layer pointer table are generic to the compiler;
+// the casts below tell it they are global memory, so it emits global (not flat) loads
+// and can keep a wave-uniform base in scalar registers.
+typedef const __attribute__((address_space(1))) char* GlobalBytes;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) u32x4* GlobalU4;
+
 struct RowData {
   uint4 lo;  // half: 8 real parts          interleaved: pairs 0-3
   uint4 hi;  // half: 8 imaginary parts     interleaved: pairs 4-7
@@ -147,22 +154,34 @@ __device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbas
     in_off = t - lb * a.block_size;
   }
   const int64_t e = phys * a.stride_block + in_off * a.stride_token + lane_off_elems;
-  const char* p = kbase + e * 2;
+  GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + e * 2;
   RowData d;
-  d.lo = *reinterpret_cast<const uint4*>(p);
-  d.hi = *reinterpret_cast<const uint4*>(p + (IL ? 16 : LPH * 16));
+  const u32x4 lo = *(GlobalU4)(p);
+  const u32x4 hi = *(GlobalU4)(p + (IL ? 16 : LPH * 16));
+  d.lo = uint4{lo.x, lo.y, lo.z, lo.w};
+  d.hi = uint4{hi.x, hi.y, hi.z, hi.w};
   return d;
 }
 
+// 16-byte buffer load: scalar descriptor (row base) + scalar byte offset + per-lane
+// byte offset, so a wave-uniform row costs no vector instruction for addressing.
+__device__ __forceinline__ uint4 buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t sgpr_off) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, (int)sgpr_off, 0);
+  return uint4{v.x, v.y, v.z, v.w};
+}
+
 // ------------------------------------------------------------------ mean
-template <int LPH, int DT, bool IL, int SP>
+// UNI: one token per wave iteration (the KV heads fill the wave's rows) and the tokens
+// of a stage share a block (or the keys are dense): scalar addressing, buffer loads.
+template <int LPH, int DT, bool IL, int SP, bool UNI>
 __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) {
   constexpr int F = LPH * kPairsPerLane;
   __shared__ int lds_blk[kScoreTileTokens + 2];
   __shared__ float lds_s1[kScoreThreads];
   __shared__ float lds_s2[kScoreThreads];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int tile = blockIdx.x, sib = blockIdx.y;
   const int b = blockIdx.z / a.L, l = blockIdx.z % a.L;
   const int seq_len = a.seq_lens[b];
@@ -203,30 +222,69 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
 
   const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
   const int64_t lane_off = (int64_t)head_c * a.stride_head + (IL ? lm.m * 16 : lm.m * 8);
+  const uint32_t lane_off_bytes = (uint32_t)(lane_off * 2);
 
   // This wave's tokens: a quarter of the tile, walked in stages of SP token pairs.
   constexpr int TW = kScoreTileTokens / 4;
   const int wstart = n0 + wave * TW;
   const int wend = min(wstart + TW, n1);
-  const int tok_per_pair = 2 * lm.tpi;
+  const int tok_per_pair = UNI ? 2 : 2 * lm.tpi;
   const int tok_per_stage = SP * tok_per_pair;
 
   const int a_out = head_c * a.G + lm.q0 + lm.qsel;
   const bool out_ok = head_ok && lm.store_lane && lm.qsel < lm.nq;
-  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)a_out * a.raw_stride_head;
+  float* raw_bl = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer;
+  float* raw_row = raw_bl + (int64_t)a_out * a.raw_stride_head;
+  // UNI: per-lane element offset from the (scalar) address of token A's row.
+  const uint32_t store_off = (uint32_t)((int64_t)a_out * a.raw_stride_head + (lm.slot_b ? a.raw_stride_token : 0));
+  const bool out_ok_a = out_ok && !lm.slot_b;   // lanes that store when token B is out of range
 
   float s1 = 0.f, s2 = 0.f;
 
+  const int last_tok = n1 - 1;
+  const uint32_t tok_bytes = (uint32_t)(a.stride_token * 2);
   auto load_stage = [&](RowData (&buf)[SP][2], int base) {
+    if (UNI) {
+      // Rows past the tile are clamped to its last token (loaded, never stored).
+      const int t0 = min(base, last_tok);
+      int64_t row_elems;
+      if (a.block_table_pitch < 0) {
+        row_elems = (int64_t)b * a.stride_block + (int64_t)t0 * a.stride_token;
+      } else {
+        const int lb = t0 >> a.bs_shift;
+        const int64_t phys = __builtin_amdgcn_readfirstlane(lds_blk[lb - lb0]);
+        row_elems = phys * a.stride_block + (int64_t)(t0 - (lb << a.bs_shift)) * a.stride_token;
+      }
+      const __amdgpu_buffer_rsrc_t rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(kbase + row_elems * 2), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
-    for (int p = 0; p < SP; ++p) {
-      const int ta = base + p * tok_per_pair + lm.tsub;
-      buf[p][0] = load_row<LPH, DT, IL>(a, kbase, b, ta, n1 - 1, lds_blk, lb0, lane_off);
-      buf[p][1] = load_row<LPH, DT, IL>(a, kbase, b, ta + lm.tpi, n1 - 1, lds_blk, lb0, lane_off);
+      for (int p = 0; p < SP; ++p) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const uint32_t soff = (uint32_t)(min(base + p * 2 + r, last_tok) - t0) * tok_bytes;
+#ifdef TRI_EXP_NOLOAD
+          buf[p][r].lo = uint4{soff + lane, 0x3f803f80u, lane_off_bytes, 0x40004000u};
+          buf[p][r].hi = uint4{0x3f003f00u, soff, 0x3f803f80u, lane_off_bytes};
+#else
+          buf[p][r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
+          buf[p][r].hi = buffer_load16(rsrc, lane_off_bytes + (IL ? 16 : LPH * 16), soff);
+#endif
+        }
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < SP; ++p) {
+        const int ta = base + p * tok_per_pair + lm.tsub;
+        buf[p][0] = load_row<LPH, DT, IL>(a, kbase, b, ta, last_tok, lds_blk, lb0, lane_off);
+        buf[p][1] = load_row<LPH, DT, IL>(a, kbase, b, ta + lm.tpi, last_tok, lds_blk, lb0, lane_off);
+      }
     }
   };
 
   auto score_row = [&](const RowData& d) -> float {
+#ifdef TRI_EXP_NOCOMPUTE
+    return __uint_as_float((d.lo.x ^ d.lo.y ^ d.lo.z ^ d.lo.w ^ d.hi.x ^ d.hi.y ^ d.hi.z ^ d.hi.w) & 0x3fffffffu) * P[0][0];
+#endif
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
@@ -246,10 +304,25 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
   auto compute_stage = [&](const RowData (&buf)[SP][2], int base) {
 #pragma unroll
     for (int p = 0; p < SP; ++p) {
-      const int ta = base + p * tok_per_pair + lm.tsub;
-      const int tb = ta + lm.tpi;
       const float ra = score_row(buf[p][0]);
       const float rb = score_row(buf[p][1]);
+      if (UNI && LPH >= 8) {
+        // Token A = base + 2p (uniform), token B the next one: quad 0 stores A, quad 1 stores B.
+        const int ta = base + p * 2;
+        if (ta < wend) {
+          const float v = lm.slot_b ? rb : ra;
+          float* row = raw_bl + (int64_t)ta * a.raw_stride_token;
+          const bool ok = (ta + 1 < wend) ? out_ok : out_ok_a;
+          if (ok) {
+            row[store_off] = v;
+            s1 += v;
+            s2 = fmaf(v, v, s2);
+          }
+        }
+        continue;
+      }
+      const int ta = base + p * tok_per_pair + lm.tsub;
+      const int tb = ta + lm.tpi;
       if (LPH >= 8) {
         const float v = lm.slot_b ? rb : ra;
         const int t = lm.slot_b ? tb : ta;
@@ -531,9 +604,16 @@ __global__ void coef_kernel(const float* folded, const float* mean_cs, int LA, i
 
 template <int LPH, int DT, bool IL>
 hipError_t launch_score_t(const ScoreArgs& args, dim3 grid, int aggregation, hipStream_t s) {
-  if (aggregation == TRI_REDUCE_MEAN)
-    hipLaunchKernelGGL((score_mean_kernel<LPH, DT, IL, 2>), grid, dim3(kScoreThreads), 0, s, args);
-  else
+  // Scalar addressing needs one token per wave iteration (the padded KV heads fill the
+  // wave's rows) and a stage of 4 tokens inside one block (or dense keys).
+  const bool uni = args.Hpad >= kWave / LPH &&
+                   (args.block_table_pitch < 0 || (args.bs_shift >= 2));
+  if (aggregation == TRI_REDUCE_MEAN) {
+    if (uni)
+      hipLaunchKernelGGL((score_mean_kernel<LPH, DT, IL, 2, true>), grid, dim3(kScoreThreads), 0, s, args);
+    else
+      hipLaunchKernelGGL((score_mean_kernel<LPH, DT, IL, 2, false>), grid, dim3(kScoreThreads), 0, s, args);
+  } else
     hipLaunchKernelGGL((score_max_kernel<LPH, DT, IL>), grid, dim3(kScoreThreads), 0, s, args);
   return hipGetLastError();
 }
