@@ -55,7 +55,14 @@ struct CombineArgs {
   int tokens_per_wg;  // 256 / rows_per_seq
 };
 
+// z-score of one raw value with the reference's operation order: (x - mean) / std.
+__device__ __forceinline__ float zscore(float x, float mean, float sd) {
+  return __fdiv_rn(__fsub_rn(x, mean), sd);
+}
+
 // One thread per (token, output row).  Grid: (token tiles, layers or 1, B).
+// VEC4: groups of four query heads, raw scores head-contiguous and 16-byte aligned.
+template <bool VEC4>
 __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
   extern __shared__ float tile[];  // [rows_per_seq][tokens_per_wg]
   const int b = blockIdx.z;
@@ -76,24 +83,67 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     const int h_begin = a.shared ? 0 : r;
     const int h_end = a.shared ? a.Hkv : r + 1;
     float acc = 0.f;
-    for (int l = l_begin; l < l_end; ++l) {
-      const float* raw_l = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)n * a.raw_stride_token;
-      const float* ms = a.mustd + (int64_t)(b * a.L + l) * a.A * 2;
-      float v = -INFINITY;
-      for (int h = h_begin; h < h_end; ++h) {
-        float gv = (a.group_reduce == TRI_REDUCE_MAX) ? -INFINITY : 0.f;
-        for (int q = 0; q < a.G; ++q) {
-          const int ah = h * a.G + q;
-          const float x = raw_l[(int64_t)ah * a.raw_stride_head];
-          const float z = __fdiv_rn(__fsub_rn(x, ms[ah * 2]), ms[ah * 2 + 1]);
-          gv = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(gv, z) : __fadd_rn(gv, z);
+    if (VEC4 && !a.shared) {
+      // Default shape: one KV head per thread, four query heads in one 16-byte load;
+      // four layers in flight per thread.
+      const float* raw0 = a.raw + (int64_t)b * a.L * a.raw_stride_layer + (int64_t)n * a.raw_stride_token + r * 4;
+      const float* ms0 = a.mustd + ((int64_t)b * a.L * a.A + r * 4) * 2;
+      auto layer_value = [&](const float4& x, const float4& m01, const float4& m23) {
+        // mustd is [head][mean, std]: m01 = (mean0, std0, mean1, std1), m23 likewise.
+        float v;
+        if (a.group_reduce == TRI_REDUCE_MAX) {
+          v = fmaxf(fmaxf(zscore(x.x, m01.x, m01.y), zscore(x.y, m01.z, m01.w)),
+                    fmaxf(zscore(x.z, m23.x, m23.y), zscore(x.w, m23.z, m23.w)));
+        } else {
+          v = __fadd_rn(__fadd_rn(__fadd_rn(zscore(x.x, m01.x, m01.y), zscore(x.y, m01.z, m01.w)),
+                                  zscore(x.z, m23.x, m23.y)), zscore(x.w, m23.z, m23.w));
+          v = __fdiv_rn(v, 4.f);
         }
-        if (a.group_reduce != TRI_REDUCE_MAX) gv = __fdiv_rn(gv, (float)a.G);
-        v = fmaxf(v, gv);
+        return guard ? INFINITY : v;
+      };
+      int l = l_begin;
+      for (; l + 4 <= l_end; l += 4) {
+        float4 x[4], m01[4], m23[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          x[u] = *reinterpret_cast<const float4*>(raw0 + (int64_t)(l + u) * a.raw_stride_layer);
+          const float* ms = ms0 + (int64_t)(l + u) * a.A * 2;
+          m01[u] = *reinterpret_cast<const float4*>(ms);
+          m23[u] = *reinterpret_cast<const float4*>(ms + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float v = layer_value(x[u], m01[u], m23[u]);
+          if (l + u == l_begin) acc = v;
+          else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
+        }
       }
-      if (guard) v = INFINITY;
-      if (l == l_begin) acc = v;
-      else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
+      for (; l < l_end; ++l) {
+        const float4 x = *reinterpret_cast<const float4*>(raw0 + (int64_t)l * a.raw_stride_layer);
+        const float* ms = ms0 + (int64_t)l * a.A * 2;
+        const float v = layer_value(x, *reinterpret_cast<const float4*>(ms), *reinterpret_cast<const float4*>(ms + 4));
+        if (l == l_begin) acc = v;
+        else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
+      }
+    } else {
+      for (int l = l_begin; l < l_end; ++l) {
+        const float* raw_l = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer + (int64_t)n * a.raw_stride_token;
+        const float* ms = a.mustd + (int64_t)(b * a.L + l) * a.A * 2;
+        float v = -INFINITY;
+        for (int h = h_begin; h < h_end; ++h) {
+          float gv = (a.group_reduce == TRI_REDUCE_MAX) ? -INFINITY : 0.f;
+          for (int q = 0; q < a.G; ++q) {
+            const int ah = h * a.G + q;
+            const float z = zscore(raw_l[(int64_t)ah * a.raw_stride_head], ms[ah * 2], ms[ah * 2 + 1]);
+            gv = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(gv, z) : __fadd_rn(gv, z);
+          }
+          if (a.group_reduce != TRI_REDUCE_MAX) gv = __fdiv_rn(gv, (float)a.G);
+          v = fmaxf(v, gv);
+        }
+        if (guard) v = INFINITY;
+        if (l == l_begin) acc = v;
+        else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
+      }
     }
     if (a.layer_reduce == TRI_REDUCE_MEAN) acc = __fdiv_rn(acc, (float)a.L);
     tile[r * a.tokens_per_wg + tn] = acc;
@@ -252,7 +302,13 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const bool per_layer = a.layer_reduce < 0;
   dim3 grid(ceil_div(a.Tmax, c.tokens_per_wg), per_layer ? a.L : 1, a.B);
   const size_t smem = (size_t)c.rows_per_seq * c.tokens_per_wg * sizeof(float);
-  hipLaunchKernelGGL(combine_kernel, grid, dim3(256), smem, s, c);
+  const bool vec4 = a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
+                    a.raw_stride_layer % 4 == 0 && (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 &&
+                    (reinterpret_cast<uintptr_t>(a.mustd) % 16) == 0;
+  if (vec4)
+    hipLaunchKernelGGL(combine_kernel<true>, grid, dim3(256), smem, s, c);
+  else
+    hipLaunchKernelGGL(combine_kernel<false>, grid, dim3(256), smem, s, c);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
 
