@@ -201,6 +201,29 @@ def main() -> int:
                                "keep_shared": keep_sh, "kv_after_per_head": a, "kv_after_shared": b,
                                "block_size": torch.tensor(bs), "total_tokens": torch.tensor(t)}
     torch.save(comp, HERE / "compaction.pt")
+
+    # ------------------------------------- slice of a shipped calibration file
+    # Two layers of the reference's Qwen3-8B statistics (a data file, loaded with
+    # weights_only=True), plus what the reference's loader makes of the slice.
+    shipped = REF / "triattention" / "calibration" / "for_aime24_experiment" / "qwen3_8b.pt"
+    full = torch.load(shipped, map_location="cpu", weights_only=True)
+    keep_keys = [k for k in full["stats"] if k.startswith("layer00_") or k.startswith("layer01_")]
+    meta = {k: v for k, v in full["metadata"].items() if k != "sampled_heads"}
+    meta["sampled_heads"] = [p for p in full["metadata"]["sampled_heads"] if p[0] in (0, 1)]
+    sl = {"metadata": meta, "stats": {k: {n: t.clone() for n, t in full["stats"][k].items()} for k in keep_keys}}
+    torch.save(sl, HERE / "qwen3_8b_stats_slice.pt")
+    sl_noname = {"metadata": {k: v for k, v in meta.items() if k not in ("model_name", "model_path")},
+                 "stats": sl["stats"]}
+    with tempfile.TemporaryDirectory() as tmp:
+        sp = Path(tmp) / "slice.pt"
+        torch.save(sl_noname, sp)
+        m, hs = load_frequency_stats(sp, device=cpu, dtype=torch.float32, num_kv_heads=None)
+        torch.save({"num_attention_heads": torch.tensor(m["num_attention_heads"]),
+                    "num_layers": torch.tensor(m["num_layers"]), "head_dim": torch.tensor(m["head_dim"]),
+                    "q_mean_complex": torch.stack([hs[l]["q_mean_complex"] for l in (0, 1)]),
+                    "q_abs_mean": torch.stack([hs[l]["q_abs_mean"] for l in (0, 1)]),
+                    "freq_scale_sq": torch.stack([hs[l]["freq_scale_sq"] for l in (0, 1)])},
+                   HERE / "qwen3_8b_stats_slice_loaded.pt")
     print("golden fixtures written to", HERE)
     return 0
 

@@ -1,0 +1,264 @@
+"""The reference-shaped Python API (selector, compaction functions, runner hook, dense
+compressor) on an MI355X, against the reference's own outputs and the oracle."""
+from __future__ import annotations
+
+import types
+from pathlib import Path
+
+import pytest
+import torch
+
+from conftest import load_golden
+from helpers import assert_keep_matches, score_tolerance
+from oracle import compaction as ocp
+from oracle import scoring as osc
+from oracle import selection as osel
+from triattention_amd.core.compressor import TriAttentionCompressor
+from triattention_amd.core.config import TriAttentionConfig
+from triattention_amd.core.scoring import compute_scores, compute_scores_triton
+from triattention_amd.runtime import (CompressionSignal, RunnerHookCompressionExecutor, TriAttentionRuntimeConfig,
+                                      build_triattention_selector, compact_request_kv_in_place,
+                                      compact_request_kv_in_place_per_head, gather_request_k_dense_range,
+                                      install_runner_compression_hook, register_kv_layout_axis_hint)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _write_stats(path: Path, qc, qa, inv_freq, head_dim):
+    layers, hq = qc.shape[:2]
+    entries = {f"layer{l:02d}_head{h:02d}": {"q_mean_real": qc[l, h, :, 0].clone(), "q_mean_imag": qc[l, h, :, 1].clone(),
+                                            "q_abs_mean": qa[l, h].clone()} for l in range(layers) for h in range(hq)}
+    torch.save({"metadata": {"head_dim": head_dim, "rope_style": "half", "inv_freq": inv_freq.clone(),
+                             "sampled_heads": [[l, h] for l in range(layers) for h in range(hq)]},
+                "stats": entries}, path)
+
+
+def _golden_caches(gold):
+    layers, hkv, t, d = gold["keys"].shape
+    bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])
+    ids = gold["block_ids"].tolist()
+    tok = torch.arange(t)
+    blk = torch.tensor(ids)[tok // bs]
+    caches = []
+    for l in range(layers):
+        kvc = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
+        kvc[0, blk, tok % bs] = gold["keys"][l].transpose(0, 1)
+        kvc[1, blk, tok % bs] = gold["values"][l].transpose(0, 1)
+        caches.append(kvc)
+    return caches, ids, bs
+
+
+@pytest.mark.parametrize("tag,kw", [("default", {}), ("nonorm", {"sparse_normalize_scores": False}),
+                                    ("aggmax", {"sparse_score_aggregation": "max"}),
+                                    ("chunk64_prefill", {"score_chunk_max_tokens": 64, "protect_prefill": True})])
+def test_selector_api_matches_reference_outputs(tmp_path, tag, kw):
+    gold = load_golden("selector_group.pt")
+    layers, hkv, t, d = gold["keys"].shape
+    _write_stats(tmp_path / "s.pt", gold["q_mean_complex"], gold["q_abs_mean"], gold["omega"], d)
+    cfg = TriAttentionRuntimeConfig(kv_budget=96, divide_length=16, window_size=12, sparse_stats_path=tmp_path / "s.pt", **kw)
+    layer_sel, group_sel, status = build_triattention_selector(cfg)
+    assert status == "enabled"
+    caches, ids, bs = _golden_caches(gold)
+    caches = [c.to(DEV) for c in caches]
+    common = dict(total_tokens=t, prefill_len=int(gold["prefill_len"]), protect_prefill=cfg.protect_prefill,
+                  round_start=int(gold["round_start"]), budget_total=96)
+    res = group_sel(layer_inputs=None, layer_input_iter=None,
+                    layer_kv_iter=lambda: [(l, caches[l], ids, bs) for l in range(layers)], **common)
+    assert res["mode"] == "per_head" and res["semantic"] == "hf_aligned_global_per_head"
+    assert res["group_agg_mode"] == "mean" and res["debug_recent_count"] == 12
+    assert res["indices"].dtype == torch.long and torch.equal(res["indices"].cpu(), gold[f"group_{tag}_keep"])
+    res_l = layer_sel(keys_dense=None, kv_cache=caches[1], block_ids=torch.tensor(ids), block_size=bs, layer_idx=1, **common)
+    assert res_l["mode"] == "per_head" and torch.equal(res_l["indices"].cpu(), gold[f"layer1_{tag}_keep"])
+    # dense inputs give the same answer as paged ones
+    dense = [(l, gather_request_k_dense_range(caches[l], ids, bs, 0, t)) for l in range(layers)]
+    res_d = group_sel(layer_inputs=dense, **common)
+    assert torch.equal(res_d["indices"], res["indices"])
+    res_ld = layer_sel(keys_dense=dense[1][1], layer_idx=1, **common)
+    assert torch.equal(res_ld["indices"], res_l["indices"])
+
+
+def test_selector_modes(tmp_path):
+    gold = load_golden("selector_group.pt")
+    layers, hkv, t, d = gold["keys"].shape
+    hq = gold["q_mean_complex"].shape[1]
+    _write_stats(tmp_path / "s.pt", gold["q_mean_complex"], gold["q_abs_mean"], gold["omega"], d)
+    caches, ids, bs = _golden_caches(gold)
+    cache1 = caches[1].to(DEV)
+    common = dict(keys_dense=None, kv_cache=cache1, block_ids=ids, block_size=bs, total_tokens=t, prefill_len=0,
+                  protect_prefill=False, layer_idx=1, round_start=t, budget_total=96)
+    offs = osc.geometric_offsets()
+    keys = gold["keys"][1].float()
+    raw_q = osc.raw_scores(keys.repeat_interleave(hq // hkv, 0), gold["q_mean_complex"][1], gold["q_abs_mean"][1],
+                           gold["omega"], offs, torch.ones(hq, d // 2), t)
+    # per_layer_per_head with mean over the query heads of a KV head
+    cfg = TriAttentionRuntimeConfig(kv_budget=96, window_size=12, sparse_stats_path=tmp_path / "s.pt",
+                                    pruning_mode="per_layer_per_head", layer_perhead_aggregation="mean")
+    res = build_triattention_selector(cfg)[0](**common)
+    fin = osel.layer_final_scores(raw_q, hkv, window_size=12, group_agg="mean")
+    assert_keep_matches(res["indices"].cpu(), osel.topk_ascending(fin, 96), fin, 96, 1e-4)
+    # legacy_layer_local: statistics mean-pooled to the KV heads
+    cfg = TriAttentionRuntimeConfig(kv_budget=96, window_size=12, sparse_stats_path=tmp_path / "s.pt",
+                                    per_head_selection_semantics="legacy_layer_local")
+    sel_l, sel_g, _ = build_triattention_selector(cfg)
+    assert sel_g(layer_inputs=[], total_tokens=t, prefill_len=0, protect_prefill=False, round_start=t, budget_total=96) is None
+    qc_p = gold["q_mean_complex"][1].reshape(hkv, hq // hkv, d // 2, 2).mean(1)
+    qa_p = gold["q_abs_mean"][1].reshape(hkv, hq // hkv, d // 2).mean(1)
+    raw_p = osc.raw_scores(keys, qc_p, qa_p, gold["omega"], offs, torch.ones(hkv, d // 2), t)
+    fin = osel.layer_final_scores(raw_p, hkv, window_size=12)
+    assert_keep_matches(sel_l(**common)["indices"].cpu(), osel.topk_ascending(fin, 96), fin, 96, 1e-4)
+    # per_layer: one shared list, max over heads
+    cfg = TriAttentionRuntimeConfig(kv_budget=96, window_size=12, sparse_stats_path=tmp_path / "s.pt",
+                                    pruning_mode="per_layer", allow_per_layer_mode=True)
+    res = build_triattention_selector(cfg)[0](**common)
+    fin = osel.layer_final_scores(raw_p, hkv, window_size=12, shared=True)
+    assert res["mode"] == "shared" and res["indices"].ndim == 1
+    assert_keep_matches(res["indices"].cpu().unsqueeze(0), osel.topk_ascending(fin, 96), fin, 96, 1e-4)
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_compaction_api_matches_reference_and_raises_like_it(axis):
+    g = load_golden("compaction.pt")[f"axis{axis}"]
+    bs, t = int(g["block_size"]), int(g["total_tokens"])
+    pad = torch.zeros(*g["kv_before"].shape[:-1], 64, dtype=torch.bfloat16)
+    pad[..., :16] = g["kv_before"]
+    a = pad.to(DEV)
+    n = compact_request_kv_in_place_per_head(a, g["block_ids"], bs, g["keep_per_head"].to(DEV), t)
+    assert n == g["keep_per_head"].shape[1]
+    assert torch.equal(a.cpu()[..., :16].view(torch.int16), g["kv_after_per_head"].view(torch.int16))
+    b = pad.to(DEV)
+    assert compact_request_kv_in_place(b, g["block_ids"].tolist(), bs, g["keep_shared"].tolist(), t) == g["keep_shared"].numel()
+    assert torch.equal(b.cpu()[..., :16].view(torch.int16), g["kv_after_shared"].view(torch.int16))
+    # prefix-only mode agrees with the reference on the kept slots
+    c = pad.to(DEV)
+    compact_request_kv_in_place_per_head(c, g["block_ids"], bs, g["keep_per_head"], t, preserve_dropped_tokens=False)
+    k = g["keep_per_head"].shape[1]
+    blk, off = ocp.token_slots(g["block_ids"], bs, torch.arange(k))
+    kc, vc = ocp.split_kv(c.cpu()[..., :16].contiguous())
+    kr, vr = ocp.split_kv(g["kv_after_per_head"])
+    assert torch.equal(kc[blk, off].view(torch.int16), kr[blk, off].view(torch.int16))
+    assert torch.equal(vc[blk, off].view(torch.int16), vr[blk, off].view(torch.int16))
+    d = pad.to(DEV)
+    before = d.clone()
+    with pytest.raises(IndexError):
+        compact_request_kv_in_place(d, g["block_ids"], bs, [0, t], t)
+    with pytest.raises(ValueError):
+        compact_request_kv_in_place(d, g["block_ids"], bs, [3, 3, 4], t)
+    with pytest.raises(ValueError):
+        compact_request_kv_in_place(d, g["block_ids"], bs, [5, 2], t)
+    with pytest.raises(ValueError):
+        compact_request_kv_in_place_per_head(d, g["block_ids"], bs, torch.zeros(2, 3, dtype=torch.long), t)
+    with pytest.raises(ValueError):
+        compact_request_kv_in_place_per_head(d, g["block_ids"], bs, torch.zeros(3, dtype=torch.long), t)
+    assert compact_request_kv_in_place(d, g["block_ids"], bs, [], t) == 0
+    assert compact_request_kv_in_place_per_head(d, g["block_ids"], bs, [], t) == 0
+    assert compact_request_kv_in_place(d, g["block_ids"], bs, list(range(t)), t) == t
+    assert torch.equal(d, before)
+    from triattention_amd.runtime.kv_compaction import clear_kv_layout_axis_hints_for_tests
+    clear_kv_layout_axis_hints_for_tests()       # hints are keyed by address; the allocator reuses addresses
+    amb = torch.zeros(2, 2, 4, 2, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        compact_request_kv_in_place(amb, [0, 1], 4, [1, 2], 8)
+    register_kv_layout_axis_hint(amb, 1)
+    assert compact_request_kv_in_place(amb, [0, 1], 4, [1, 2], 8) == 2
+
+
+def _signal(**kw):
+    base = dict(req_id="r", should_compress=True, reason="length_threshold", estimated_cache_len=301, step=1,
+                kv_usage=None, protect_prefill=False, prefill_len=20, scheduled_tokens=1)
+    base.update(kw)
+    return CompressionSignal(**base)
+
+
+def test_runner_hook_end_to_end(tmp_path):
+    """Fake runner -> hook -> keep sets equal to the reference's, K/V compacted bit-exactly,
+    block table truncated, result dictionary as the scheduler expects it."""
+    gold = load_golden("selector_group.pt")
+    layers, hkv, t, d = gold["keys"].shape
+    _write_stats(tmp_path / "s.pt", gold["q_mean_complex"], gold["q_abs_mean"], gold["omega"], d)
+    cfg = TriAttentionRuntimeConfig(kv_budget=96, divide_length=16, window_size=12, sparse_stats_path=tmp_path / "s.pt")
+    cpu_caches, ids, bs = _golden_caches(gold)
+    caches = [c.to(DEV) for c in cpu_caches]
+    req = types.SimpleNamespace(num_computed_tokens=int(gold["round_start"]), block_ids=(list(ids),))
+    runner = types.SimpleNamespace(requests={"r": req}, kv_caches=caches, cache_config=types.SimpleNamespace(block_size=bs))
+    install_runner_compression_hook(runner, cfg)
+    sched = types.SimpleNamespace(num_scheduled_tokens={"r": 1})
+    # estimated length = cached tokens + the token scheduled this step
+    res = RunnerHookCompressionExecutor(runner).execute("r", _signal(estimated_cache_len=t + 1), sched)
+    torch.cuda.synchronize()
+    assert res.applied and res.reason == "kv_compacted:per_head:hf_aligned_global_per_head"
+    assert res.cache_len_after == 96 and res.details["budget_total"] == 96
+    assert res.details["effective_tokens_before"] == t and res.details["selector_status"] == "enabled"
+    nkeep = (96 + bs - 1) // bs
+    assert req.block_ids == (ids[:nkeep],)
+    grp = res.details["block_reclaim"]["groups"][0]
+    assert grp["block_ids_before"] == ids and grp["block_ids_after"] == ids[:nkeep] and grp["block_ids_removed"] == ids[nkeep:]
+    assert res.details["reclaimed_block_count"] == len(ids) - nkeep
+    want_keep = gold["group_default_keep"]
+    blk, off = ocp.token_slots(ids, bs, torch.arange(96))
+    for l in range(layers):
+        ref = cpu_caches[l].clone()
+        ocp.compact_per_head(ref, ids, bs, want_keep, t, full_permutation=False)
+        got = caches[l].cpu()
+        assert torch.equal(got[:, blk, off].view(torch.int16), ref[:, blk, off].view(torch.int16))
+    # second trigger right away: below budget + divide_length -> deferred
+    req.num_computed_tokens += 1
+    again = runner.triattention_apply_compression(req_id="r", signal=_signal(estimated_cache_len=98), scheduler_output=sched)
+    assert again["applied"] is False and again["reason"] == "under_budget"
+
+
+def test_dense_scoring_api_against_reference_scores():
+    gold = load_golden("scoring_pytorch.pt")
+    for name, style in (("d128_half", "half"), ("d64_inter", "interleaved")):
+        case = gold[name]
+        for agg in ("mean", "max"):
+            for mlr, trig in ((1, 1), (0, 1), (1, 0)):
+                cfg = TriAttentionConfig(device=torch.device(DEV), score_aggregation=agg, disable_mlr=not mlr,
+                                         disable_trig=not trig, rope_style=style)
+                got = compute_scores(key_states=case["keys"].unsqueeze(0).to(DEV), cache_positions=None,
+                                     head_stats={"q_mean_complex": case["q_mean_complex"].to(DEV),
+                                                 "q_abs_mean": case["q_abs_mean"].to(DEV)},
+                                     omega=case["omega"].to(DEV), offsets=case["offsets"].to(DEV),
+                                     freq_scale_sq=case["freq_scale_sq"].to(DEV), config=cfg,
+                                     round_start=int(case["round_start"]))
+                want = case[f"scores_{agg}_mlr{mlr}_trig{trig}"]
+                assert got.shape == (1,) + tuple(want.shape) and got.dtype == torch.float32
+                err = (got[0].cpu() - want).abs()
+                assert bool((err <= score_tolerance(want) + 1e-6).all()), (name, agg, mlr, trig, float(err.max()))
+    assert compute_scores_triton is compute_scores
+    with pytest.raises(TypeError):
+        compute_scores(key_states=torch.zeros(1, 2, 8, 64, device=DEV), cache_positions=None,
+                       head_stats={"q_mean_complex": torch.zeros(2, 32, 2)}, omega=torch.zeros(32),
+                       offsets=torch.ones(1), freq_scale_sq=torch.ones(2, 32),
+                       config=TriAttentionConfig(device=torch.device(DEV)), round_start=1)
+
+
+def test_dense_compressor_against_oracle(tmp_path):
+    g = torch.Generator().manual_seed(17)
+    h, t, d, budget = 4, 600, 128, 128
+    omega = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    qc = torch.randn(1, h, d // 2, 2, generator=g)
+    qa = qc.pow(2).sum(-1).sqrt() + torch.randn(1, h, d // 2, generator=g).abs()
+    _write_stats(tmp_path / "s.pt", qc, qa, omega, d)
+    keys = (torch.randn(1, h, t, d, generator=g) + 1.0).to(torch.bfloat16)
+    vals = torch.randn(1, h, t, d, generator=g).to(torch.bfloat16)
+    cfg = TriAttentionConfig(device=torch.device(DEV), stats_path=tmp_path / "s.pt", kv_budget=budget, divide_length=16,
+                             window_size=16, protect_prefill=False, compute_dtype=torch.float32)
+    comp = TriAttentionCompressor(cfg)
+    k2, v2, keep = comp.compress(keys.to(DEV), vals.to(DEV), layer_idx=0)
+    assert k2.shape == (1, h, budget, d) and keep.shape == (1, h, budget)
+    raw = osc.raw_scores(keys[0], qc[0], qa[0], omega, osc.geometric_offsets(), torch.ones(h, d // 2), t)
+    fin = osel.protect_window(osel.znorm_two_pass(raw), 16)
+    assert_keep_matches(keep[0].cpu(), osel.topk_ascending(fin, budget), fin, budget, 1e-3)
+    kk = keep[0].cpu()
+    for hh in range(h):
+        assert torch.equal(k2[0, hh].cpu().view(torch.int16), keys[0, hh, kk[hh]].view(torch.int16))
+        assert torch.equal(v2[0, hh].cpu().view(torch.int16), vals[0, hh, kk[hh]].view(torch.int16))
+    assert comp.get_state()["compression_count"] == 1 and comp.get_state()["current_cache_len"] == budget
+    # below budget + divide_length nothing happens
+    small = TriAttentionCompressor(cfg)
+    k3, v3, ident = small.compress(keys[:, :, :100].to(DEV), vals[:, :, :100].to(DEV))
+    assert k3.shape[2] == 100 and ident.tolist() == list(range(100))
+    with pytest.raises(ValueError):
+        TriAttentionCompressor(cfg).compress(torch.zeros(2, h, 600, d, dtype=torch.bfloat16, device=DEV),
+                                             torch.zeros(2, h, 600, d, dtype=torch.bfloat16, device=DEV))

@@ -1,0 +1,469 @@
+"""The runner hook ``triattention_apply_compression(req_id, signal, scheduler_output)``.
+
+This is the plug-in seam of the reference (runtime/executor.py:31-85,
+runtime/hook_impl.py:30-185): ``install_runner_compression_hook`` puts a callable of
+that name on the base runner unless one is already there, and the executor calls it
+once per triggered request.  Request-state lookup follows runtime/hook_preflight.py and
+runtime/runner_struct_compat.py, the length bookkeeping runtime/hook_runtime_context.py,
+the KV tensors per cache group runtime/kv_group_resolver.py.  Only plain attribute
+access is used on the runner, so any object with ``requests``, ``kv_caches`` and
+``cache_config.block_size`` works.
+"""
+from __future__ import annotations
+
+import re
+from dataclasses import dataclass
+from typing import Any, Callable
+
+import torch
+
+from .config import TriAttentionRuntimeConfig
+from .kv_compaction import (build_keep_token_indices, compact_request_kv_in_place,
+                            compact_request_kv_in_place_per_head, gather_request_k_dense,
+                            register_kv_layout_axis_hint)
+from .models import TRITON_SCORING_REQUIRED_MARKER as MARK, CompressionSignal
+from .pipeline import (finalize_hook_placement_result, normalize_mutable_block_ids_by_group,
+                       run_group_compaction_pipeline)
+from .selector import build_triattention_selector as _build_triattention_selector
+
+
+# --------------------------------------------------------------- executor side
+@dataclass(frozen=True)
+class CompressionExecutionResult:
+    applied: bool
+    reason: str
+    cache_len_after: int | None = None
+    details: dict | None = None
+
+
+class CompressionExecutor:
+    def execute(self, req_id: str, signal: CompressionSignal, scheduler_output: Any) -> CompressionExecutionResult:
+        raise NotImplementedError
+
+
+class RunnerHookCompressionExecutor(CompressionExecutor):
+    """Delegates to the hook on the base runner (runtime/executor.py:31-85)."""
+
+    hook_name = "triattention_apply_compression"
+
+    def __init__(self, base_runner: Any):
+        self._base_runner = base_runner
+
+    def execute(self, req_id, signal, scheduler_output) -> CompressionExecutionResult:
+        hook = getattr(self._base_runner, self.hook_name, None)
+        if not callable(hook):
+            return CompressionExecutionResult(False, "runner_hook_missing")
+        out = hook(req_id=req_id, signal=signal, scheduler_output=scheduler_output)
+        if isinstance(out, bool):
+            return CompressionExecutionResult(out, "applied" if out else "runner_hook_rejected")
+        if isinstance(out, dict):
+            d = dict(out)
+            return CompressionExecutionResult(bool(d.get("applied", False)), str(d.get("reason", "runner_hook_result")),
+                                              d.get("cache_len_after"), d)
+        return CompressionExecutionResult(False, f"unsupported_hook_result:{type(out).__name__}")
+
+
+# ------------------------------------------------------------- request lookup
+def req_id_from_scheduled_key(key: Any):
+    if isinstance(key, (str, int)):
+        return key
+    for attr in ("request_id", "req_id"):
+        v = getattr(key, attr, None)
+        if isinstance(v, (str, int)):
+            return v
+    return None
+
+
+def scheduled_tokens_for_req(scheduler_output: Any, req_id: str) -> int:
+    """Tokens scheduled for the request this step, at least 1
+    (runtime/hook_runtime_context.py:57-76, runtime/request_key_compat.py)."""
+    table = getattr(scheduler_output, "num_scheduled_tokens", None)
+    if not isinstance(table, dict):
+        return 1
+    for raw_key, raw_val in table.items():
+        if req_id_from_scheduled_key(raw_key) == req_id:
+            try:
+                return max(1, int(raw_val))
+            except (TypeError, ValueError):
+                return 1
+    return 1
+
+
+@dataclass
+class _SchedulerRequestView:
+    req_id: str
+    num_computed_tokens: int
+    block_ids: Any
+
+
+class _MergedRequestView:
+    """Runner-side state whose num_computed_tokens lags the scheduler's
+    (runtime/hook_preflight.py:40-61)."""
+
+    def __init__(self, base, num_computed_tokens: int, fallback_block_ids):
+        self._base, self._nct, self._fallback = base, int(num_computed_tokens), fallback_block_ids
+
+    @property
+    def num_computed_tokens(self) -> int:
+        return self._nct
+
+    @property
+    def block_ids(self):
+        ids = getattr(self._base, "block_ids", None)
+        return ids if ids is not None else self._fallback
+
+    @block_ids.setter
+    def block_ids(self, value) -> None:
+        setattr(self._base, "block_ids", value)
+
+
+class _IndexedRequestView:
+    """Request addressed by its row in the runner's batch tables
+    (runtime/runner_struct_compat.py:61-141)."""
+
+    def __init__(self, runner, req_id, index, requests_state):
+        self._runner, self.req_id, self._index, self._requests_state = runner, req_id, index, requests_state
+
+    @property
+    def num_computed_tokens(self) -> int:
+        gpu = getattr(getattr(getattr(self._runner, "req_states", None), "num_computed_tokens", None), "gpu", None)
+        if torch.is_tensor(gpu):
+            return int(gpu[self._index].item())
+        cpu = getattr(getattr(self._runner, "input_batch", None), "num_computed_tokens_cpu", None)
+        try:
+            return int(cpu[self._index]) if cpu is not None else 0
+        except Exception:
+            return 0
+
+    @property
+    def block_ids(self):
+        tables = getattr(self._runner, "block_tables", None)
+        rows = getattr(tables, "block_tables", None)
+        counts = getattr(getattr(tables, "num_blocks", None), "np", None)
+        if isinstance(rows, list) and counts is not None:
+            out, ok = [], True
+            for gid, table in enumerate(rows):
+                try:
+                    n = int(counts[gid, self._index])
+                except Exception:
+                    ok = False
+                    break
+                gpu = getattr(table, "gpu", None)
+                if n <= 0:
+                    out.append([])
+                elif torch.is_tensor(gpu):
+                    out.append([int(x) for x in gpu[self._index, :n].tolist()])
+                else:
+                    ok = False
+                    break
+            if ok and any(out):
+                return tuple(out)
+        ids = getattr(self._requests_state, "block_ids", None)
+        if isinstance(ids, (list, tuple)):
+            return tuple([int(b) for b in g] if isinstance(g, (list, tuple)) else [] for g in ids)
+        return None
+
+    @block_ids.setter
+    def block_ids(self, new_ids) -> None:
+        if not isinstance(new_ids, (list, tuple)):
+            raise TypeError("block_ids must be a list/tuple by group")
+        norm = tuple([int(b) for b in g] if isinstance(g, (list, tuple)) else [] for g in new_ids)
+        tables = getattr(self._runner, "block_tables", None)
+        if tables is not None:
+            tables.append_block_ids(self._index, norm, overwrite=True)
+            tables.apply_staged_writes()
+        if self._requests_state is not None:
+            setattr(self._requests_state, "block_ids", norm)
+
+
+def _scheduler_view(scheduler_output, req_id):
+    for new_req in getattr(scheduler_output, "scheduled_new_reqs", None) or []:
+        if getattr(new_req, "req_id", None) != req_id or getattr(new_req, "block_ids", None) is None:
+            continue
+        lens = []
+        for attr in ("prompt_token_ids", "prefill_token_ids"):
+            v = getattr(new_req, attr, None)
+            if v is not None:
+                try:
+                    lens.append(len(v))
+                except Exception:
+                    pass
+        for attr in ("prompt_token_ids_len", "num_prompt_tokens"):
+            v = getattr(new_req, attr, None)
+            try:
+                if v is not None:
+                    lens.append(int(v))
+            except (TypeError, ValueError):
+                pass
+        return _SchedulerRequestView(req_id, max(lens, default=0), new_req.block_ids)
+    cached = getattr(scheduler_output, "scheduled_cached_reqs", None)
+    ids, ncts = getattr(cached, "req_ids", None), getattr(cached, "num_computed_tokens", None)
+    if isinstance(ids, list) and isinstance(ncts, list):
+        for i, rid in enumerate(ids):
+            if rid == req_id and i < len(ncts):
+                try:
+                    return _SchedulerRequestView(req_id, int(ncts[i]), None)
+                except Exception:
+                    return None
+    return None
+
+
+def resolve_request_state(base_runner: Any, req_id: str, scheduler_output: Any = None):
+    """The request's state object (has ``num_computed_tokens`` and settable
+    ``block_ids``), or None (runtime/hook_preflight.py:124-219)."""
+    requests = getattr(base_runner, "requests", None)
+    requests_state = requests.get(req_id) if isinstance(requests, dict) else None
+    state = None
+    for owner_name in ("req_states", "input_batch"):
+        index_map = getattr(getattr(base_runner, owner_name, None), "req_id_to_index", None)
+        if isinstance(index_map, dict) and isinstance(index_map.get(req_id), int):
+            state = _IndexedRequestView(base_runner, req_id, index_map[req_id], requests_state)
+            break
+    if state is None:
+        batch = getattr(base_runner, "input_batch", None)
+        ids = getattr(batch, "req_ids", None)
+        try:
+            ids = ids() if callable(ids) else ids
+        except Exception:
+            ids = None
+        if not isinstance(ids, list):
+            ids = getattr(batch, "_req_ids", None)
+        if isinstance(ids, list) and req_id in ids:
+            state = _IndexedRequestView(base_runner, req_id, ids.index(req_id), requests_state)
+    if state is None:
+        state = requests_state
+    sched = _scheduler_view(scheduler_output, req_id) if scheduler_output is not None else None
+    if state is None:
+        return sched
+    if sched is not None:
+        try:
+            mine = int(getattr(state, "num_computed_tokens", 0) or 0)
+            if int(sched.num_computed_tokens) > mine:
+                return _MergedRequestView(state, sched.num_computed_tokens, sched.block_ids)
+        except Exception:
+            pass
+    return state
+
+
+# ------------------------------------------------------------- KV tensors by group
+def infer_layer_idx(layer_name: str, layer_obj: Any, fallback_idx: int) -> int:
+    for attr in ("layer_idx", "layer_id", "idx"):
+        v = getattr(layer_obj, attr, None)
+        if isinstance(v, int):
+            return v
+    digits = re.findall(r"\d+", layer_name)
+    return int(digits[-1]) if digits else fallback_idx
+
+
+def _kv_axis_of_backend(base_runner: Any, gid: int):
+    """0 for [2, nb, ...] backends, 1 for [nb, 2, ...] (runtime/kv_group_resolver.py:24-66)."""
+    groups = getattr(base_runner, "attn_groups", None)
+    if not isinstance(groups, (list, tuple)) or not 0 <= gid < len(groups):
+        return None
+    backend = getattr(groups[gid], "backend", None)
+    if backend is None:
+        return None
+    cls = backend if isinstance(backend, type) else backend.__class__
+    shape_fn = getattr(cls, "get_kv_cache_shape", None)
+    if callable(shape_fn):
+        try:
+            shape = tuple(int(x) for x in shape_fn(3, 16, 1, 1))
+            if len(shape) >= 2 and (shape[0] == 2) != (shape[1] == 2):
+                return 0 if shape[0] == 2 else 1
+        except Exception:
+            pass
+    ident = f"{getattr(cls, '__module__', '')}.{getattr(cls, '__name__', '')}".lower()
+    if "flash_attn" in ident:
+        return 0
+    if "triton_attn" in ident:
+        return 1
+    return None
+
+
+def resolve_group_tensors(base_runner: Any) -> dict:
+    """gid -> [(layer_idx, kv_cache tensor)] (runtime/kv_group_resolver.py:69-141)."""
+    out: dict = {}
+    kv_cfg = getattr(base_runner, "kv_cache_config", None)
+    ctx = getattr(getattr(base_runner, "compilation_config", None), "static_forward_context", None)
+    if kv_cfg is None or not isinstance(ctx, dict):
+        caches = getattr(base_runner, "kv_caches", None)
+        if isinstance(caches, list):
+            pairs = [(i, t) for i, t in enumerate(caches) if isinstance(t, torch.Tensor)]
+            if pairs:
+                out[0] = pairs
+        return out
+    for gid, group in enumerate(getattr(kv_cfg, "kv_cache_groups", None) or []):
+        names = getattr(group, "layer_names", None)
+        if not isinstance(names, (list, tuple)):
+            continue
+        pairs, seen = [], set()
+        for local_idx, name in enumerate(names):
+            layer = ctx.get(name)
+            caches = getattr(layer, "kv_cache", None)
+            if not isinstance(caches, list) or not caches or not isinstance(caches[0], torch.Tensor):
+                continue
+            if caches[0].data_ptr() in seen:
+                continue
+            seen.add(caches[0].data_ptr())
+            pairs.append((infer_layer_idx(name, layer, local_idx), caches[0]))
+        if pairs:
+            axis = _kv_axis_of_backend(base_runner, gid)
+            if axis is not None:
+                for _, t in pairs:
+                    try:
+                        register_kv_layout_axis_hint(t, axis)
+                    except ValueError:
+                        pass
+            out[gid] = pairs
+    return out
+
+
+# ------------------------------------------------------------- length bookkeeping
+@dataclass(frozen=True)
+class HookRuntimeContext:
+    scheduled_tokens: int
+    num_computed_tokens: int
+    estimated_effective_tokens: int
+    effective_tokens: int
+    budget_total: int
+    recent_unabsorbed_tokens: int | None
+    should_defer_recompress: bool
+
+
+def effective_budget_for_signal(config, signal, total_tokens: int) -> int:
+    budget = config.kv_budget
+    if signal.protect_prefill and not config.include_prefill_in_budget:
+        budget += max(signal.prefill_len, 0)
+    return min(total_tokens, budget)
+
+
+def build_hook_runtime_context(*, base_runner: Any, config: TriAttentionRuntimeConfig, req_id: str, req_state: Any,
+                               req_runtime_state: Any, signal: CompressionSignal, scheduler_output: Any,
+                               compressed_once: set, original_block_ids_by_group: Any,
+                               block_size_hint: int) -> HookRuntimeContext:
+    """Effective cached tokens, budget and the re-compression gate
+    (runtime/hook_runtime_context.py:106-209)."""
+    capacities = [len(g) * block_size_hint for g in (original_block_ids_by_group or ())
+                  if isinstance(g, (list, tuple))] if isinstance(original_block_ids_by_group, (list, tuple)) else []
+    capacity = min(capacities) if capacities and block_size_hint > 0 else None
+
+    scheduled = scheduled_tokens_for_req(scheduler_output, req_id)
+    nct = int(getattr(req_state, "num_computed_tokens", 0))
+    estimated = max(0, int(getattr(signal, "estimated_cache_len", 0)))
+    if req_runtime_state is not None:
+        cnt = getattr(req_runtime_state, "compression_count", None)
+        cur = getattr(req_runtime_state, "current_cache_len", None)
+        if isinstance(cnt, int) and cnt > 0 and isinstance(cur, int) and cur > 0:
+            estimated = max(0, cur)
+
+    post_forward = getattr(signal, "_post_forward", False)
+    effective = max(0, estimated) if post_forward else max(0, estimated - max(0, scheduled))
+    effective = min(effective, nct + (scheduled if post_forward else 0))
+    if isinstance(capacity, int):
+        effective = min(effective, capacity + block_size_hint)
+
+    recent = None
+    if req_runtime_state is not None:
+        recent = max(0, effective - int(getattr(req_runtime_state, "last_absorbed_cache_len", 0)))
+    setattr(base_runner, "_triattention_active_recent_unabsorbed_tokens", recent)
+
+    prefill_len = int(getattr(signal, "prefill_len", 0) or 0)
+    if (config.fail_on_effective_len_regression and config.enable_experimental_block_reclaim
+            and req_id in compressed_once and not (prefill_len > 0 and nct < prefill_len)):
+        upper = config.kv_budget + (max(signal.prefill_len, 0) if signal.protect_prefill
+                                    and not config.include_prefill_in_budget else 0)
+        upper += max(1, config.effective_len_guard_divide_multiples) * max(1, config.divide_length)
+        slack = block_size_hint + max(1, int(getattr(signal, "estimated_cache_len", 0)) - nct) + max(1, scheduled)
+        if (effective > upper + slack and nct > upper + slack
+                and effective >= int(config.effective_len_regression_ratio * nct)):
+            raise RuntimeError(f"{MARK}:effective_len_regressed:req={req_id}:effective_tokens={effective}:"
+                               f"num_computed_tokens={nct}:guard_upper={upper}")
+
+    budget_total = effective_budget_for_signal(config, signal, effective)
+    gate_hit = estimated >= budget_total + max(1, config.divide_length)
+    defer = (config.enable_experimental_kv_compaction and req_id in compressed_once
+             and str(getattr(signal, "reason", "")) != "kv_usage_threshold" and not gate_hit)
+    return HookRuntimeContext(int(scheduled), int(nct), int(estimated), int(effective), int(budget_total),
+                              int(recent) if isinstance(recent, int) else None, bool(defer))
+
+
+# ------------------------------------------------------------------- the hook
+def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeConfig) -> Callable[..., dict]:
+    """runtime/hook_impl.py:30-165."""
+    try:
+        select_layer, select_group, selector_status = _build_triattention_selector(config, base_runner=base_runner)
+    except TypeError:
+        select_layer, select_group, selector_status = _build_triattention_selector(config)
+    group_tensors: dict | None = None
+    compressed_once: set = set()
+
+    def _hook(req_id: str, signal: CompressionSignal, scheduler_output: Any) -> dict:
+        nonlocal group_tensors
+        setattr(base_runner, "_triattention_active_req_id", req_id)
+        strict = bool(config.enable_experimental_kv_compaction and config.require_triton_scoring)
+        req_state = resolve_request_state(base_runner, req_id, scheduler_output)
+        if req_state is None:
+            return {"applied": False, "reason": "req_state_not_found"}
+        store = getattr(base_runner, "_triattention_state_store", None)
+        runtime_state = store.get(req_id) if store is not None and hasattr(store, "get") else None
+        block_size_hint = int(getattr(getattr(base_runner, "cache_config", None), "block_size", 0))
+        if block_size_hint <= 0:
+            block_size_hint = 1
+        original_ids = getattr(req_state, "block_ids", None)
+        ctx = build_hook_runtime_context(
+            base_runner=base_runner, config=config, req_id=req_id, req_state=req_state,
+            req_runtime_state=runtime_state, signal=signal, scheduler_output=scheduler_output,
+            compressed_once=compressed_once, original_block_ids_by_group=original_ids,
+            block_size_hint=block_size_hint)
+        if ctx.effective_tokens <= ctx.budget_total or ctx.should_defer_recompress:
+            return {"applied": False, "reason": "under_budget", "cache_len_after": ctx.effective_tokens}
+
+        if not config.enable_experimental_kv_compaction:
+            plan = build_keep_token_indices(total_tokens=ctx.effective_tokens, kv_budget=config.kv_budget,
+                                            prefill_len=signal.prefill_len, protect_prefill=signal.protect_prefill,
+                                            include_prefill_in_budget=config.include_prefill_in_budget)
+            if plan is None:
+                return {"applied": False, "reason": "prefill_exceeds_budget"}
+            return {"applied": False, "reason": "plan_only", "cache_len_after": len(plan)}
+        if strict and select_layer is None:
+            raise RuntimeError(f"{MARK}:selector_unavailable:{selector_status}")
+
+        kv_caches = getattr(base_runner, "kv_caches", None)
+        cache_config = getattr(base_runner, "cache_config", None)
+        if not isinstance(kv_caches, list) or cache_config is None:
+            return {"applied": False, "reason": "kv_cache_unavailable"}
+        block_size = int(getattr(cache_config, "block_size", 0))
+        if block_size <= 0:
+            return {"applied": False, "reason": "invalid_block_size"}
+        if not original_ids:
+            return {"applied": False, "reason": "missing_block_ids"}
+        mutable_ids = normalize_mutable_block_ids_by_group(original_ids)
+        if mutable_ids is None:
+            return {"applied": False, "reason": "invalid_block_ids_container"}
+
+        if group_tensors is None:
+            group_tensors = resolve_group_tensors(base_runner)
+        out = run_group_compaction_pipeline(
+            req_id=req_id, signal=signal, config=config, strict_triton_required=strict,
+            num_computed_tokens=ctx.num_computed_tokens, effective_tokens=ctx.effective_tokens,
+            budget_total=ctx.budget_total, block_size=block_size, mutable_block_ids_by_group=mutable_ids,
+            group_tensors=group_tensors, select_keep_indices=select_layer,
+            select_keep_indices_for_group=select_group, shared_compact_fn=compact_request_kv_in_place,
+            per_head_compact_fn=compact_request_kv_in_place_per_head, gather_dense_fn=gather_request_k_dense)
+        if isinstance(out, dict):
+            return out
+        compressed_once.add(req_id)
+        return finalize_hook_placement_result(
+            req_state=req_state, original_block_ids_by_group=original_ids, config=config,
+            selector_status=str(selector_status), outcome=out, effective_tokens=ctx.effective_tokens,
+            budget_total=ctx.budget_total, recent_unabsorbed_tokens=ctx.recent_unabsorbed_tokens)
+
+    return _hook
+
+
+def install_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeConfig) -> None:
+    """Install the hook unless the runner already has one (runtime/hook_impl.py:174-185)."""
+    if hasattr(base_runner, "triattention_apply_compression"):
+        return
+    setattr(base_runner, "triattention_apply_compression",
+            make_runner_compression_hook(base_runner=base_runner, config=config))

@@ -1,0 +1,243 @@
+"""Keep-set selection for the runtime hook: the callable pair the reference builds in
+``build_triattention_selector`` (triattention/vllm/runtime/selector_hf.py:15-1083), same
+keyword signatures, result dictionaries and failure markers, executed by the HIP scorer,
+the combine kernel and the radix top-k.
+
+Nothing is chunked and K is neither gathered nor repeated per query head: the scorer
+reads the paged blocks of every layer once.  Ties at the budget keep the lowest token
+index (the reference's ``torch.topk`` leaves them undefined).
+"""
+from __future__ import annotations
+
+import os
+from pathlib import Path
+from typing import Any, Callable, Iterable
+
+import torch
+
+from .. import ops
+from ..core import stats as stats_mod
+from .config import TriAttentionRuntimeConfig
+from .kv_compaction import kv_axis_hint
+from .models import TRITON_SCORING_REQUIRED_MARKER as MARK
+
+
+class _DeviceStats:
+    """Statistics of one stats file resident on one device, folded once per head layout."""
+
+    def __init__(self, config: TriAttentionRuntimeConfig, stats_path: Path, model_path):
+        self.config = config
+        self.metadata, self.head_stats = stats_mod.load_frequency_stats(
+            stats_path, device="cpu", dtype=torch.float32, num_kv_heads=None, model_path=model_path)
+        if not self.head_stats:
+            raise RuntimeError("empty_head_stats")
+        self.layers = tuple(sorted(self.head_stats.keys()))
+        self.head_dim = int(self.metadata["head_dim"])
+        self.rope_style = str(self.metadata.get("rope_style", "half"))
+        self.inv_freq = stats_mod.resolve_inv_freq(self.metadata, self.head_dim, model_path)
+        self.offsets = stats_mod.geometric_offsets(65536)
+        self.stats_heads = int(self.head_stats[self.layers[0]]["freq_scale_sq"].shape[0])
+        self._folded: dict = {}
+        self._vectors: dict = {}
+
+    def resolve_layer(self, layer_idx: int) -> int:
+        """Layer index modulo the layers the file has (selector_hf.py:132-143)."""
+        if layer_idx in self.head_stats:
+            return layer_idx
+        return self.layers[layer_idx % len(self.layers)]
+
+    def vectors(self, device):
+        v = self._vectors.get(device)
+        if v is None:
+            v = (self.inv_freq.to(device).contiguous(), self.offsets.to(device).contiguous())
+            self._vectors[device] = v
+        return v
+
+    def folded(self, layer_ids: tuple, score_heads: int, device) -> torch.Tensor:
+        """[L, score_heads, 3, F] for the given runtime layers; heads mean-pooled when the
+        caller scores fewer heads than the file holds (selector_hf.py:147-203)."""
+        key = (layer_ids, score_heads, str(device))
+        hit = self._folded.get(key)
+        if hit is not None:
+            return hit
+        qc, qa, fs = [], [], []
+        for layer in layer_ids:
+            entry = self.head_stats[self.resolve_layer(layer)]
+            if "q_mean_complex" not in entry:
+                raise RuntimeError("stats file has no q_mean_real/q_mean_imag entries")
+            qc.append(stats_mod.pool_heads(entry["q_mean_complex"], score_heads))
+            qa.append(stats_mod.pool_heads(entry["q_abs_mean"], score_heads))
+            fs.append(stats_mod.pool_heads(entry["freq_scale_sq"], score_heads))
+        out = ops.fold_stats(torch.stack(qc).to(device), torch.stack(qa).to(device), torch.stack(fs).to(device),
+                             disable_mlr=self.config.disable_mlr, disable_trig=self.config.disable_trig)
+        self._folded[key] = out
+        return out
+
+
+def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: Any | None = None):
+    """(select_keep_indices, select_keep_indices_for_group, status)."""
+    mode = config.pruning_mode
+    if mode == "per_layer" and not bool(getattr(config, "allow_per_layer_mode", False)):
+        raise RuntimeError(f"{MARK}:per_layer_mode_disabled:set allow_per_layer_mode=True for explicit opt-in")
+    strict = bool(config.enable_experimental_kv_compaction and config.require_triton_scoring)
+
+    def _unavailable(reason: str):
+        if strict:
+            raise RuntimeError(f"{MARK}:{reason}")
+        return None, None, reason
+
+    if config.sparse_stats_path is None:
+        return _unavailable("stats_path_not_set")
+    stats_path = Path(config.sparse_stats_path).expanduser()
+    if not stats_path.exists():
+        return _unavailable("stats_path_not_found")
+    if mode not in {"per_layer", "per_head", "per_layer_per_head"}:
+        return _unavailable(f"unsupported_pruning_mode:{mode}")
+    try:
+        from .. import _lib
+        _lib.load()
+    except Exception as exc:
+        raise RuntimeError(f"{MARK}:import_failed:{type(exc).__name__}") from exc
+
+    semantics = config.per_head_selection_semantics
+    model_path = getattr(config, "model_path", None)
+    if model_path is None and base_runner is not None:
+        for owner in (getattr(base_runner, "model_config", None),
+                      getattr(getattr(base_runner, "vllm_config", None), "model_config", None)):
+            cand = getattr(owner, "model", None)
+            if isinstance(cand, Path) or (isinstance(cand, str) and cand.strip()):
+                model_path = Path(cand)
+                break
+
+    holder: dict = {}
+
+    def _stats() -> _DeviceStats:
+        if "s" not in holder:
+            holder["s"] = _DeviceStats(config, stats_path, model_path)
+        return holder["s"]
+
+    def _recent_count(total_tokens: int) -> int:
+        if total_tokens <= 0 or config.window_size <= 0:
+            return 0
+        return min(config.window_size, total_tokens)
+
+    def _head_layout(runtime_heads: int):
+        """(heads scored per layer, group reduce): all file heads with a max (or the
+        configured per-layer reduce) when the file is per query head, else stats pooled
+        down to the runtime heads (selector_hf.py:242-297)."""
+        st = _stats()
+        group_max = st.stats_heads != runtime_heads and (
+            (mode == "per_head" and semantics == "hf_aligned_global_per_head") or mode == "per_layer_per_head")
+        if group_max:
+            if runtime_heads <= 0 or st.stats_heads % runtime_heads:
+                raise RuntimeError(f"{MARK}:incompatible_head_mapping:source={st.stats_heads},target={runtime_heads}")
+            return st.stats_heads, (config.layer_perhead_aggregation if mode == "per_layer_per_head" else "max")
+        return runtime_heads, "max"
+
+    def _paged_kv(caches):
+        hints = {kv_axis_hint(c) for c in caches}
+        return ops.PagedKV.from_kv_caches(caches, rope_style=_stats().rope_style,
+                                          kv_axis=hints.pop() if len(hints) == 1 else None)
+
+    def _score_and_select(kv: ops.PagedKV, layer_ids: tuple, block_ids, total_tokens: int, prefill_len: int,
+                          protect_prefill: bool, round_start: int, k: int, layer_reduce, group_reduce: str,
+                          score_heads: int, shared: bool) -> torch.Tensor:
+        st = _stats()
+        omega, offsets = st.vectors(kv.device)
+        sc = ops.ScoreConfig(st.folded(layer_ids, score_heads, kv.device), omega, offsets,
+                             config.sparse_score_aggregation)
+        tables = None if block_ids is None else [
+            block_ids.flatten().tolist() if isinstance(block_ids, torch.Tensor) else [int(x) for x in block_ids]]
+        batch = ops.StepBatch(kv.device, [total_tokens], round_start=[round_start], budgets=[k],
+                              block_tables=tables, prefill_lens=[prefill_len])
+        try:
+            raw, ws = ops.score_paged(kv, batch, sc)
+        except Exception as exc:
+            raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
+        sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
+                               protect_prefill=bool(protect_prefill and prefill_len > 0),
+                               group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared)
+        keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+        return keep.to(torch.long)
+
+    def _select_keep_indices(*, keys_dense: torch.Tensor | None = None, kv_cache: torch.Tensor | None = None,
+                             block_ids=None, block_size: int | None = None, total_tokens: int, prefill_len: int,
+                             protect_prefill: bool, layer_idx: int, round_start: int, budget_total: int):
+        """One layer (selector_hf.py:679-747, paged streaming :473-677)."""
+        if total_tokens <= budget_total:
+            return {"mode": "shared", "indices": list(range(total_tokens))}
+        if protect_prefill and config.include_prefill_in_budget and prefill_len > budget_total:
+            return None
+        if keys_dense is not None:
+            if keys_dense.shape[0] != 1:
+                raise RuntimeError("selector expects keys_dense of shape [1, H, T, D]")
+            kv = ops.PagedKV.from_dense_keys(keys_dense[..., :total_tokens, :], rope_style=_stats().rope_style)
+            tables = None
+        elif kv_cache is not None and block_ids is not None and block_size is not None:
+            kv = _paged_kv([kv_cache])
+            tables = block_ids
+        else:
+            raise RuntimeError("missing scoring inputs for selector")
+        k = min(int(budget_total), int(total_tokens))
+        if k <= 0:
+            return {"mode": "shared", "indices": []}
+        score_heads, group_reduce = _head_layout(kv.num_kv_heads)
+        per_head = mode in {"per_head", "per_layer_per_head"}
+        keep = _score_and_select(kv, (int(layer_idx),), tables, total_tokens, prefill_len, protect_prefill,
+                                 round_start, k, None, group_reduce, score_heads, shared=not per_head)
+        if per_head:
+            return {"mode": "per_head", "indices": keep.contiguous()}
+        return {"mode": "shared", "indices": keep[0].contiguous()}
+
+    def _select_keep_indices_for_group_per_head(*, layer_inputs=None,
+                                                layer_input_iter: Callable[[], Iterable] | None = None,
+                                                layer_kv_iter: Callable[[], Iterable] | None = None,
+                                                total_tokens: int, prefill_len: int, protect_prefill: bool,
+                                                round_start: int, budget_total: int):
+        """One keep set for every layer of a KV-cache group (selector_hf.py:749-1079)."""
+        if mode != "per_head" or semantics != "hf_aligned_global_per_head":
+            return None
+        if layer_kv_iter is not None:
+            entries = list(layer_kv_iter())
+            paged = True
+        else:
+            entries = list(layer_input_iter()) if layer_input_iter is not None else list(layer_inputs or [])
+            paged = False
+        if total_tokens <= budget_total:
+            if not entries:
+                return {"mode": "per_head", "indices": []}
+            first = entries[0][1]
+            heads = int(first.shape[3] if paged else first.shape[1])
+            ident = torch.arange(total_tokens, dtype=torch.long, device=first.device)
+            return {"mode": "per_head", "indices": ident.unsqueeze(0).expand(heads, -1).contiguous()}
+        if protect_prefill and config.include_prefill_in_budget and prefill_len > budget_total:
+            return None
+        if not entries:
+            return None
+        k = min(budget_total, total_tokens)
+        if k <= 0:
+            return {"mode": "per_head", "indices": []}
+        layer_ids = tuple(int(e[0]) for e in entries)
+        if paged:
+            agg = os.environ.get("TRIATTN_RUNTIME_DEBUG_GROUP_PERHEAD_AGG_MODE", "mean").strip().lower()
+            if agg not in {"mean", "max"}:
+                agg = "mean"
+            if len({int(e[3]) for e in entries}) != 1:
+                raise RuntimeError("layers of one KV-cache group must share one block size")
+            kv = _paged_kv([e[1] for e in entries])
+            tables = entries[0][2]
+        else:
+            agg = "mean"
+            kv = ops.PagedKV([e[1][..., :total_tokens, :].permute(0, 2, 1, 3) for e in entries], None,
+                             _stats().rope_style)
+            tables = None
+        score_heads, group_reduce = _head_layout(kv.num_kv_heads)
+        keep = _score_and_select(kv, layer_ids, tables, total_tokens, prefill_len, protect_prefill, round_start,
+                                 k, agg, "max", score_heads, shared=False)
+        return {"mode": "per_head", "indices": keep.contiguous(), "semantic": "hf_aligned_global_per_head",
+                "group_agg_mode": agg, "debug_group_layer_indices": list(layer_ids),
+                "debug_recent_count": _recent_count(total_tokens)}
+
+    setattr(_select_keep_indices, "_supports_paged", True)
+    setattr(_select_keep_indices_for_group_per_head, "_supports_paged_group", True)
+    return _select_keep_indices, _select_keep_indices_for_group_per_head, "enabled"
