@@ -16,6 +16,7 @@ namespace {
 
 constexpr int kCompactThreads = 256;
 constexpr int kChunksPerThread = 4;                                  // 16-byte chunks held per thread
+static_assert(kChunksPerThread == 4, "compact_kernel spells out four chunk registers");
 constexpr int kTileChunks = kCompactThreads * kChunksPerThread;      // 16 KiB per tile
 constexpr int kSegSlots = 1024;                                      // slots whose addresses are staged in LDS
 
@@ -99,28 +100,32 @@ __global__ __launch_bounds__(kCompactThreads) void compact_kernel(CompactArgs a)
       // A slot wider than a tile is moved in several passes; every pass is read
       // completely before it is written, and passes of one slot never overlap.
       for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
-        uint4 regs[kChunksPerThread];
-        int64_t dsts[kChunksPerThread];
+        // Branch-free loads: idle chunks re-read the tile's first source row (a cache
+        // hit) and only their store is masked.
+        int64_t so[kChunksPerThread], dsto[kChunksPerThread];
         bool live[kChunksPerThread];
 #pragma unroll
         for (int c = 0; c < kChunksPerThread; ++c) {
           const int ci = c0 + c * kCompactThreads + threadIdx.x;
           live[c] = ci < nchunks;
-          if (live[c]) {
-            const int sl = t0 + ci / chunks_per_slot;
-            const int within = ci % chunks_per_slot;
-            const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
-            const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
-            const int64_t so = src_off[sl] + inner;
-            dsts[c] = dst_off[sl] + inner;
-            live[c] = so != dsts[c];            // row already in place
-            if (live[c]) regs[c] = *reinterpret_cast<const uint4*>(base + so);
-          }
+          const int cic = live[c] ? ci : c0;
+          const int sl = t0 + cic / chunks_per_slot;
+          const int within = cic % chunks_per_slot;
+          const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+          const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
+          so[c] = src_off[sl] + inner;
+          dsto[c] = dst_off[sl] + inner;
+          live[c] = live[c] && so[c] != dsto[c];     // row already in place
         }
+        uint4 r0 = *reinterpret_cast<const uint4*>(base + so[0]);
+        uint4 r1 = *reinterpret_cast<const uint4*>(base + so[1]);
+        uint4 r2 = *reinterpret_cast<const uint4*>(base + so[2]);
+        uint4 r3 = *reinterpret_cast<const uint4*>(base + so[3]);
         __syncthreads();   // every read of this tile is ordered before any write of it
-#pragma unroll
-        for (int c = 0; c < kChunksPerThread; ++c)
-          if (live[c]) *reinterpret_cast<uint4*>(base + dsts[c]) = regs[c];
+        if (live[0]) *reinterpret_cast<uint4*>(base + dsto[0]) = r0;
+        if (live[1]) *reinterpret_cast<uint4*>(base + dsto[1]) = r1;
+        if (live[2]) *reinterpret_cast<uint4*>(base + dsto[2]) = r2;
+        if (live[3]) *reinterpret_cast<uint4*>(base + dsto[3]) = r3;
       }
     }
   }
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactAr
 #pragma unroll
     for (int c = 0; c < kChunksPerThread; ++c) {
       live[c] = live[c] && src[c] >= k;
-      const int sc = live[c] ? src[c] : jj[c];           // idle chunk: read its own destination row
+      const int sc = live[c] ? src[c] : j0;              // idle chunk: re-read one row of the tile (cache hit)
       so[c] = slot_units(a, bt, sc) + inner[c];
       dsto[c] = slot_units(a, bt, jj[c]) + inner[c];
     }
