@@ -26,6 +26,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 
+# HBM bytes one score_mean_kernel launch moves on the C1 workload, from two rocprofv3 --pmc
+# runs of this script (FETCH_SIZE 9,717,510 KiB-units x 2.0, WRITE_SIZE 1,184,256 x 1.0; the
+# factors are what the same counters read for the 1 GiB copies of --copy-calibration).
+MEASURED_SCORE_TRAFFIC_BYTES = {"c1_qwen3_8b_36l_b16_16k": 9_717_510 * 1024 * 2 + 1_184_256 * 1024}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -198,7 +203,8 @@ def main() -> int:
         "timed_region_wall_s": wall_s,
         "setup_s": setup_s,
         "roofline": {"kernel": "score_mean_kernel", "bound": "hbm", "achieved": score_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS, "traffic": None},
+                     "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_SCORE_TRAFFIC_BYTES.get(w.name)},
     }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)

@@ -262,13 +262,8 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
           const uint32_t soff = (uint32_t)(min(base + p * 2 + r, last_tok) - t0) * tok_bytes;
-#ifdef TRI_EXP_NOLOAD
-          buf[p][r].lo = uint4{soff + lane, 0x3f803f80u, lane_off_bytes, 0x40004000u};
-          buf[p][r].hi = uint4{0x3f003f00u, soff, 0x3f803f80u, lane_off_bytes};
-#else
           buf[p][r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
           buf[p][r].hi = buffer_load16(rsrc, lane_off_bytes + (IL ? 16 : LPH * 16), soff);
-#endif
         }
       }
     } else {
@@ -282,9 +277,6 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
   };
 
   auto score_row = [&](const RowData& d) -> float {
-#ifdef TRI_EXP_NOCOMPUTE
-    return __uint_as_float((d.lo.x ^ d.lo.y ^ d.lo.z ^ d.lo.w ^ d.hi.x ^ d.hi.y ^ d.hi.z ^ d.hi.w) & 0x3fffffffu) * P[0][0];
-#endif
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
