@@ -13,12 +13,14 @@ from triattention_amd import ops, synth
 def build_inputs(w: synth.Workload, kv_axis: int = 0):
     """CPU-generated, seeded inputs of a workload."""
     tables = synth.make_block_tables(w)
-    caches = synth.make_kv_pool(w, tables, "cpu", kv_axis)
+    pool = synth.make_kv_pool(w, tables, "cpu", kv_axis)
+    caches, k_scales, v_scales = pool if w.kv_dtype == "fp8" else (pool, None, None)
     qc, qa = synth.make_stats(w, "cpu")
     omega = synth.rope_inv_freq(w)
     offsets = synth.geometric_offsets()
     fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2)
-    return dict(tables=tables, caches=caches, qc=qc, qa=qa, omega=omega, offsets=offsets, fs=fs, kv_axis=kv_axis)
+    return dict(tables=tables, caches=caches, qc=qc, qa=qa, omega=omega, offsets=offsets, fs=fs, kv_axis=kv_axis,
+                k_scales=k_scales, v_scales=v_scales)
 
 
 def oracle_raw(w, inp, b, round_start, aggregation="mean", disable_mlr=False, disable_trig=False):
@@ -27,6 +29,9 @@ def oracle_raw(w, inp, b, round_start, aggregation="mean", disable_mlr=False, di
     out = []
     for l in range(w.num_layers):
         kc, _ = ocp.split_kv(inp["caches"][l], inp["kv_axis"])
+        if inp.get("k_scales") is not None:      # fp8: dequantise the pool, then proceed as for bf16
+            nb, bs, h, d = kc.shape
+            kc = osc.dequant_fp8(kc.reshape(nb * bs, h, d), inp["k_scales"][l]).view(nb, bs, h, d)
         keys = ocp.gather_dense(kc, inp["tables"][b], w.block_size, 0, w.seq_lens[b])[0]      # [Hkv, T, D]
         keys = keys.float().repeat_interleave(g, dim=0)
         out.append(osc.raw_scores(keys, inp["qc"][l], inp["qa"][l], inp["omega"], inp["offsets"], inp["fs"][l],
@@ -37,7 +42,14 @@ def oracle_raw(w, inp, b, round_start, aggregation="mean", disable_mlr=False, di
 def device_objects(w, inp, device, round_start=None, budgets=None, prefill_lens=None, aggregation="mean",
                    disable_mlr=False, disable_trig=False):
     caches = [c.to(device) for c in inp["caches"]]
-    kv = ops.PagedKV.from_kv_caches(caches, w.rope_style, kv_axis=inp["kv_axis"])
+    if inp.get("k_scales") is not None:
+        ks = [t.to(device) for t in inp["k_scales"]]
+        vs = [t.to(device) for t in inp["v_scales"]]
+        ax = inp["kv_axis"]
+        kv = ops.PagedKV([c[0] if ax == 0 else c[:, 0] for c in caches],
+                         [c[1] if ax == 0 else c[:, 1] for c in caches], w.rope_style, ks, vs)
+    else:
+        kv = ops.PagedKV.from_kv_caches(caches, w.rope_style, kv_axis=inp["kv_axis"])
     batch = ops.StepBatch(device, w.seq_lens, round_start=round_start,
                           budgets=budgets if budgets is not None else w.budget,
                           block_tables=inp["tables"], prefill_lens=prefill_lens)

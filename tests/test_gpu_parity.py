@@ -54,6 +54,15 @@ SCORE_CASES = {
     "no_trig": dict(w=small(), disable_trig=True),
     "no_trig_max": dict(w=small(), disable_trig=True, aggregation="max"),
     "late_round": dict(w=small(), round_start=[70000]),
+    # fp8 e4m3 keys with per-(token, head) scales: no reference counterpart, oracle = dequantise then score
+    "fp8": dict(w=small(kv_dtype="fp8", seq_lens=(300, 45))),
+    "fp8_hkv8_llama3": dict(w=small(kv_dtype="fp8", num_q_heads=32, num_kv_heads=8, rope_theta=5e5,
+                                    rope_scaling="llama3", seq_lens=(530,))),
+    "fp8_interleaved": dict(w=small(kv_dtype="fp8", rope_style="interleaved")),
+    "fp8_d64": dict(w=small(kv_dtype="fp8", head_dim=64, num_q_heads=16, num_kv_heads=8, seq_lens=(270,))),
+    "fp8_d256_hkv2": dict(w=small(kv_dtype="fp8", head_dim=256, num_q_heads=4, num_kv_heads=2, seq_lens=(140,))),
+    "fp8_block24": dict(w=small(kv_dtype="fp8", block_size=24, seq_lens=(301,))),
+    "fp8_max_agg": dict(w=small(kv_dtype="fp8", seq_lens=(200,)), aggregation="max"),
 }
 
 
@@ -365,6 +374,79 @@ def test_end_to_end_c0_against_oracle():
     blk, off = ocp.token_slots(inp["tables"][0], w.block_size, torch.arange(k))
     dev = caches[0].cpu()
     assert torch.equal(dev[:, blk, off].view(torch.int16), ref[:, blk, off].view(torch.int16))
+
+
+def test_fp8_every_code_decodes_like_torch():
+    """All 254 finite e4m3 codes through the scorer: with one non-zero coefficient the
+    score is code_value * scale * coefficient, which pins the decoder against torch's
+    float8_e4m3fn conversion (no reference counterpart: the reference has no fp8 code)."""
+    codes = torch.tensor([c for c in range(256) if c & 0x7f != 0x7f], dtype=torch.uint8)     # 254 finite codes
+    h, d, bs = 2, 128, 16
+    t = codes.numel()
+    nb = (t + bs - 1) // bs
+    g = torch.Generator().manual_seed(5)
+    for style in ("half", "interleaved"):
+        k = torch.zeros(nb * bs, h, d, dtype=torch.uint8)
+        for pos in (0, 5, 63, 64, 77, 127):                      # element positions carrying the code
+            k[:t, :, pos] = codes.unsqueeze(1)
+        scales = 0.25 + torch.rand(nb * bs, h, generator=g)
+        kf8 = k.view(torch.float8_e4m3fn).view(nb, bs, h, d)
+        qc = torch.randn(1, h, d // 2, 2, generator=g)
+        qa = qc.pow(2).sum(-1).sqrt() + torch.rand(1, h, d // 2, generator=g)
+        fs = torch.ones(1, h, d // 2)
+        omega, offs = synth.rope_inv_freq(small()), synth.geometric_offsets()
+        kd, sd = kf8.to(DEV), scales.to(DEV)
+        kv = ops.PagedKV([kd], None, style, [sd], None)
+        batch = ops.StepBatch(DEV, [t], round_start=[900], block_tables=[list(range(nb))])
+        sc = ops.ScoreConfig(ops.fold_stats(qc.to(DEV), qa.to(DEV), fs.to(DEV)), omega.to(DEV), offs.to(DEV))
+        raw, _ = ops.score_paged(kv, batch, sc, head_major=True)
+        torch.cuda.synchronize()
+        keys = osc.dequant_fp8(kf8.view(nb * bs, h, d), scales)[:t].permute(1, 0, 2)          # [H, T, D]
+        want = osc.raw_scores(keys, qc[0], qa[0], omega, offs, fs[0], 900, rope_style=style)
+        got = raw[0, 0, :, :t].cpu()
+        assert bool(((got - want).abs() <= score_tolerance(want)).all()), style
+
+
+def test_fp8_step_scores_selects_and_compacts():
+    """fp8 cache end to end: kept set against the oracle on dequantised keys, then codes
+    and scales of K and V compacted bit-exactly."""
+    w = small(kv_dtype="fp8", seq_lens=(700, 150, 60), num_layers=3, num_q_heads=16, num_kv_heads=4, budget=128)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    keep, _ = ops.compress_step(kv, batch, sc, sel)
+    torch.cuda.synchronize()
+    got = keep.cpu().long()
+    h = w.num_kv_heads
+    ks_dev, vs_dev = kv._keep[2], kv._keep[3]
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        rows = got[b * h:(b + 1) * h, :k]
+        if t > w.budget:
+            oraw = oracle_raw(w, inp, b, t)
+            want, ofin = osel.group_keep_per_head(oraw, h, k, window_size=w.window_size,
+                                                  chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
+            scale = float(ofin[torch.isfinite(ofin)].abs().max())
+            assert_keep_matches(rows, want, ofin, k, tie_tol=2e-3 * scale)
+        else:
+            assert torch.equal(rows, torch.arange(t).expand(h, t))
+    for l in range(w.num_layers):
+        ref = inp["caches"][l].clone().view(torch.uint8)
+        nb = ref.shape[1]
+        ref_s = torch.stack([inp["k_scales"][l].view(nb, w.block_size, h, 1),
+                             inp["v_scales"][l].view(nb, w.block_size, h, 1)]).clone()
+        dev_c = caches[l].cpu().view(torch.uint8)
+        dev_s = torch.stack([ks_dev[l].cpu().view(nb, w.block_size, h, 1), vs_dev[l].cpu().view(nb, w.block_size, h, 1)])
+        for b, t in enumerate(w.seq_lens):
+            k = min(w.budget, t)
+            if k >= t:
+                continue
+            rows = got[b * h:(b + 1) * h, :k]
+            ocp.compact_per_head(ref, inp["tables"][b], w.block_size, rows, t, full_permutation=False)
+            ocp.compact_per_head(ref_s, inp["tables"][b], w.block_size, rows, t, full_permutation=False)
+            blk, off = ocp.token_slots(inp["tables"][b], w.block_size, torch.arange(k))
+            assert torch.equal(dev_c[:, blk, off], ref[:, blk, off]), (l, b)
+            assert torch.equal(dev_s[:, blk, off], ref_s[:, blk, off]), (l, b)
 
 
 def test_invalid_arguments_raise():

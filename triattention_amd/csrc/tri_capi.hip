@@ -101,7 +101,6 @@ T* at(void* ws, int64_t off) { return reinterpret_cast<T*>(reinterpret_cast<char
 int do_score(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp, float* raw,
              int64_t rs_layer, int64_t rs_token, int64_t rs_head, void* ws, const tri::Workspace& w,
              hipStream_t s) {
-  if (kv->kv_dtype == TRI_KV_FP8_E4M3) return fail(TRI_ERR_UNSUPPORTED, "fp8 keys: scorer not built yet");
   const int F = kv->head_dim / 2;
   hipError_t e = tri::launch_prepare(sp->folded, sp->omega, sp->offsets, sp->num_offsets, batch->round_start,
                                      batch->num_seqs, kv->num_layers, sp->num_score_heads, F, sp->aggregation,

@@ -68,6 +68,15 @@ __device__ __forceinline__ float elem_hi<TRI_KV_FP16>(uint32_t w) {
   return (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
 }
 
+// fp8 e4m3 (OCP encoding on gfx950): byte SEL of a 32-bit word.
+template <int SEL>
+__device__ __forceinline__ float fp8_byte(uint32_t w) {
+  return __builtin_amdgcn_cvt_f32_fp8((int)w, SEL);
+}
+
+template <int DT>
+constexpr int elem_size() { return DT == TRI_KV_FP8_E4M3 ? 1 : 2; }
+
 // Pointers fetched from the per-layer pointer table are generic to the compiler;
 // the casts below tell it they are global memory, so it emits global (not flat) loads
 // and can keep a wave-uniform base in scalar registers.
@@ -75,9 +84,18 @@ typedef const __attribute__((address_space(1))) char* GlobalBytes;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) u32x4* GlobalU4;
 
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(1))) u32x2* GlobalU2;
+typedef const __attribute__((address_space(1))) float* GlobalF32;
+
+// 2-byte elements: lo/hi are 16 bytes each.  fp8: "half" uses lo.xy (8 real parts) and
+// hi.xy (8 imaginary parts), "interleaved" uses the 16 bytes of lo; `scale` is the
+// row's dequantisation scale (the score is homogeneous of degree one in the key, so
+// the scale multiplies the reduced score once).
 struct RowData {
   uint4 lo;  // half: 8 real parts          interleaved: pairs 0-3
   uint4 hi;  // half: 8 imaginary parts     interleaved: pairs 4-7
+  float scale;
 };
 
 // Real and imaginary part of this lane's pair p (0..7).
@@ -85,7 +103,21 @@ template <int DT, bool IL>
 __device__ __forceinline__ void unpack_pair(const RowData& d, int p, float& kr, float& ki) {
   const uint32_t* lo = reinterpret_cast<const uint32_t*>(&d.lo);
   const uint32_t* hi = reinterpret_cast<const uint32_t*>(&d.hi);
-  if (IL) {
+  if constexpr (DT == TRI_KV_FP8_E4M3) {
+    if (IL) {
+      const uint32_t w = lo[p >> 1];
+      kr = (p & 1) ? fp8_byte<2>(w) : fp8_byte<0>(w);
+      ki = (p & 1) ? fp8_byte<3>(w) : fp8_byte<1>(w);
+    } else {
+      const uint32_t wr = lo[p >> 2], wi = hi[p >> 2];
+      switch (p & 3) {
+        case 0: kr = fp8_byte<0>(wr); ki = fp8_byte<0>(wi); break;
+        case 1: kr = fp8_byte<1>(wr); ki = fp8_byte<1>(wi); break;
+        case 2: kr = fp8_byte<2>(wr); ki = fp8_byte<2>(wi); break;
+        default: kr = fp8_byte<3>(wr); ki = fp8_byte<3>(wi); break;
+      }
+    }
+  } else if (IL) {
     const uint32_t w = (p < 4) ? lo[p] : hi[p - 4];
     kr = elem_lo<DT>(w);
     ki = elem_hi<DT>(w);
@@ -98,6 +130,7 @@ __device__ __forceinline__ void unpack_pair(const RowData& d, int p, float& kr, 
 
 struct ScoreArgs {
   const void* const* k_layers;
+  const float* const* k_scale_layers;   // fp8 only
   const int32_t* block_table;
   const int32_t* seq_lens;
   const float* coef;
@@ -139,9 +172,9 @@ struct LaneMap {
 };
 
 template <int LPH, int DT, bool IL>
-__device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbase, int b, int tok,
-                                            int last_tok, const int* lds_blk, int lb0,
-                                            int64_t lane_off_elems) {
+__device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbase, const float* kscale,
+                                            int head, int b, int tok, int last_tok, const int* lds_blk,
+                                            int lb0, int64_t lane_off_elems) {
   // Rows past the tile are clamped to its last token (loaded, never stored), so
   // every address stays inside the blocks whose ids were staged in LDS.
   const int t = min(tok, last_tok);
@@ -154,12 +187,27 @@ __device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbas
     in_off = t - lb * a.block_size;
   }
   const int64_t e = phys * a.stride_block + in_off * a.stride_token + lane_off_elems;
-  GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + e * 2;
+  GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + e * elem_size<DT>();
   RowData d;
-  const u32x4 lo = *(GlobalU4)(p);
-  const u32x4 hi = *(GlobalU4)(p + (IL ? 16 : LPH * 16));
-  d.lo = uint4{lo.x, lo.y, lo.z, lo.w};
-  d.hi = uint4{hi.x, hi.y, hi.z, hi.w};
+  d.scale = 1.f;
+  if constexpr (DT == TRI_KV_FP8_E4M3) {
+    if (IL) {
+      const u32x4 lo = *(GlobalU4)(p);
+      d.lo = uint4{lo.x, lo.y, lo.z, lo.w};
+      d.hi = uint4{0, 0, 0, 0};
+    } else {
+      const u32x2 lo = *(GlobalU2)(p);
+      const u32x2 hi = *(GlobalU2)(p + LPH * 8);
+      d.lo = uint4{lo.x, lo.y, 0, 0};
+      d.hi = uint4{hi.x, hi.y, 0, 0};
+    }
+    d.scale = ((GlobalF32)(uintptr_t)kscale)[(phys * a.block_size + in_off) * a.Hkv + head];
+  } else {
+    const u32x4 lo = *(GlobalU4)(p);
+    const u32x4 hi = *(GlobalU4)(p + (IL ? 16 : LPH * 16));
+    d.lo = uint4{lo.x, lo.y, lo.z, lo.w};
+    d.hi = uint4{hi.x, hi.y, hi.z, hi.w};
+  }
   return d;
 }
 
@@ -168,6 +216,14 @@ __device__ __forceinline__ RowData load_row(const ScoreArgs& a, const char* kbas
 __device__ __forceinline__ uint4 buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t sgpr_off) {
   const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, (int)sgpr_off, 0);
   return uint4{v.x, v.y, v.z, v.w};
+}
+
+__device__ __forceinline__ uint4 buffer_load8(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t sgpr_off) {
+  const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_off, (int)sgpr_off, 0);
+  return uint4{v.x, v.y, 0, 0};
+}
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t sgpr_off) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_off, (int)sgpr_off, 0));
 }
 
 // ------------------------------------------------------------------ mean
@@ -220,9 +276,12 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
     }
   }
 
+  constexpr bool FP8 = DT == TRI_KV_FP8_E4M3;
+  constexpr int ES = elem_size<DT>();
   const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
+  const float* kscale = FP8 ? a.k_scale_layers[l] : nullptr;
   const int64_t lane_off = (int64_t)head_c * a.stride_head + (IL ? lm.m * 16 : lm.m * 8);
-  const uint32_t lane_off_bytes = (uint32_t)(lane_off * 2);
+  const uint32_t lane_off_bytes = (uint32_t)(lane_off * ES);
 
   // This wave's tokens: a quarter of the tile, walked in stages of SP token pairs.
   constexpr int TW = kScoreTileTokens / 4;
@@ -242,36 +301,54 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
   float s1 = 0.f, s2 = 0.f;
 
   const int last_tok = n1 - 1;
-  const uint32_t tok_bytes = (uint32_t)(a.stride_token * 2);
+  const uint32_t tok_bytes = (uint32_t)(a.stride_token * ES);
+  const uint32_t scale_tok_bytes = (uint32_t)a.Hkv * 4u;
   auto load_stage = [&](RowData (&buf)[SP][2], int base) {
     if (UNI) {
       // Rows past the tile are clamped to its last token (loaded, never stored).
       const int t0 = min(base, last_tok);
-      int64_t row_elems;
+      int64_t row_elems, slot;
       if (a.block_table_pitch < 0) {
         row_elems = (int64_t)b * a.stride_block + (int64_t)t0 * a.stride_token;
+        slot = (int64_t)b * a.block_size + t0;
       } else {
         const int lb = t0 >> a.bs_shift;
         const int64_t phys = __builtin_amdgcn_readfirstlane(lds_blk[lb - lb0]);
         row_elems = phys * a.stride_block + (int64_t)(t0 - (lb << a.bs_shift)) * a.stride_token;
+        slot = phys * a.block_size + (t0 - (lb << a.bs_shift));
       }
       const __amdgpu_buffer_rsrc_t rsrc =
-          __builtin_amdgcn_make_buffer_rsrc((void*)(kbase + row_elems * 2), 0, 0x7fffffff, 0x00020000);
+          __builtin_amdgcn_make_buffer_rsrc((void*)(kbase + row_elems * ES), 0, 0x7fffffff, 0x00020000);
+      __amdgpu_buffer_rsrc_t srsrc = rsrc;
+      if constexpr (FP8)
+        srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(kscale + slot * a.Hkv), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
       for (int p = 0; p < SP; ++p) {
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-          const uint32_t soff = (uint32_t)(min(base + p * 2 + r, last_tok) - t0) * tok_bytes;
-          buf[p][r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
-          buf[p][r].hi = buffer_load16(rsrc, lane_off_bytes + (IL ? 16 : LPH * 16), soff);
+          const uint32_t dt = (uint32_t)(min(base + p * 2 + r, last_tok) - t0);
+          const uint32_t soff = dt * tok_bytes;
+          if constexpr (FP8) {
+            if (IL) {
+              buf[p][r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
+              buf[p][r].hi = uint4{0, 0, 0, 0};
+            } else {
+              buf[p][r].lo = buffer_load8(rsrc, lane_off_bytes, soff);
+              buf[p][r].hi = buffer_load8(rsrc, lane_off_bytes + LPH * 8, soff);
+            }
+            buf[p][r].scale = buffer_load_f32(srsrc, (uint32_t)head_c * 4u, dt * scale_tok_bytes);
+          } else {
+            buf[p][r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
+            buf[p][r].hi = buffer_load16(rsrc, lane_off_bytes + (IL ? 16 : LPH * 16), soff);
+          }
         }
       }
     } else {
 #pragma unroll
       for (int p = 0; p < SP; ++p) {
         const int ta = base + p * tok_per_pair + lm.tsub;
-        buf[p][0] = load_row<LPH, DT, IL>(a, kbase, b, ta, last_tok, lds_blk, lb0, lane_off);
-        buf[p][1] = load_row<LPH, DT, IL>(a, kbase, b, ta + lm.tpi, last_tok, lds_blk, lb0, lane_off);
+        buf[p][0] = load_row<LPH, DT, IL>(a, kbase, kscale, head_c, b, ta, last_tok, lds_blk, lb0, lane_off);
+        buf[p][1] = load_row<LPH, DT, IL>(a, kbase, kscale, head_c, b, ta + lm.tpi, last_tok, lds_blk, lb0, lane_off);
       }
     }
   };
@@ -290,7 +367,8 @@ __global__ __launch_bounds__(kScoreThreads) void score_mean_kernel(ScoreArgs a) 
         acc[q] = fmaf(mag, E[q][p], acc[q]);
       }
     }
-    return reduce_row<LPH>(acc, lm.b0, lm.b1);
+    const float r = reduce_row<LPH>(acc, lm.b0, lm.b1);
+    return FP8 ? r * d.scale : r;
   };
 
   auto compute_stage = [&](const RowData (&buf)[SP][2], int base) {
@@ -441,7 +519,9 @@ __global__ __launch_bounds__(kScoreThreads) void score_max_kernel(ScoreArgs a) {
     }
   }
 
+  constexpr bool FP8 = DT == TRI_KV_FP8_E4M3;
   const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
+  const float* kscale = FP8 ? a.k_scale_layers[l] : nullptr;
   const int64_t lane_off = (int64_t)head_c * a.stride_head + (IL ? lm.m * 16 : lm.m * 8);
   constexpr int TW = kScoreTileTokens / 4;
   const int wstart = n0 + wave * TW;
@@ -478,14 +558,14 @@ __global__ __launch_bounds__(kScoreThreads) void score_max_kernel(ScoreArgs a) {
       }
       best = fmaxf(best, reduce_row<LPH>(acc, lm.b0, lm.b1));
     }
-    return best + extra;
+    return FP8 ? (best + extra) * d.scale : best + extra;
   };
 
   const int step = 2 * lm.tpi;
   for (int base = wstart; base < wend; base += step) {
     const int ta = base + lm.tsub, tb = ta + lm.tpi;
-    const RowData da = load_row<LPH, DT, IL>(a, kbase, b, ta, n1 - 1, lds_blk, lb0, lane_off);
-    const RowData db = load_row<LPH, DT, IL>(a, kbase, b, tb, n1 - 1, lds_blk, lb0, lane_off);
+    const RowData da = load_row<LPH, DT, IL>(a, kbase, kscale, head_c, b, ta, n1 - 1, lds_blk, lb0, lane_off);
+    const RowData db = load_row<LPH, DT, IL>(a, kbase, kscale, head_c, b, tb, n1 - 1, lds_blk, lb0, lane_off);
     const float ra = score_row(da);
     const float rb = score_row(db);
     if (LPH >= 8) {
@@ -618,6 +698,9 @@ hipError_t launch_score_lph(const ScoreArgs& args, dim3 grid, int dt, int il, in
   if (dt == TRI_KV_FP16)
     return il ? launch_score_t<LPH, TRI_KV_FP16, true>(args, grid, aggregation, s)
               : launch_score_t<LPH, TRI_KV_FP16, false>(args, grid, aggregation, s);
+  if (dt == TRI_KV_FP8_E4M3)
+    return il ? launch_score_t<LPH, TRI_KV_FP8_E4M3, true>(args, grid, aggregation, s)
+              : launch_score_t<LPH, TRI_KV_FP8_E4M3, false>(args, grid, aggregation, s);
   return hipErrorInvalidValue;
 }
 
@@ -650,6 +733,7 @@ hipError_t launch_prepare(const float* folded, const float* omega, const float* 
 hipError_t launch_score(const ScoreLaunch& a, hipStream_t s) {
   ScoreArgs k{};
   k.k_layers = a.k_layers;
+  k.k_scale_layers = a.k_scale_layers;
   k.block_table = a.block_table;
   k.seq_lens = a.seq_lens;
   k.coef = a.coef;
