@@ -26,10 +26,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 
-# HBM bytes one score_mean_kernel launch moves on the C1 workload, from two rocprofv3 --pmc
-# runs of this script (FETCH_SIZE 9,717,510 KiB-units x 2.0, WRITE_SIZE 1,184,256 x 1.0; the
-# factors are what the same counters read for the 1 GiB copies of --copy-calibration).
-MEASURED_SCORE_TRAFFIC_BYTES = {"c1_qwen3_8b_36l_b16_16k": 9_717_510 * 1024 * 2 + 1_184_256 * 1024}
+# HBM bytes one launch of the dominant kernel moves on the C1 workload, from two rocprofv3
+# --pmc runs of this script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB; the factors are what
+# the same counters read for the 1 GiB copies of --copy-calibration).  Keyed by
+# (workload, two_pass); absent = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    ("c1_qwen3_8b_36l_b16_16k", True): 9_717_510 * 1024 * 2 + 1_184_256 * 1024,   # score_mean_kernel
+}
 
 
 def parse_args():
@@ -40,6 +43,8 @@ def parse_args():
     ap.add_argument("--config", type=int, default=1, help="BASELINE.json config index (default 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=36, help="layers of one sequence the CPU baseline scores")
+    ap.add_argument("--two-pass", action="store_true",
+                    help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (reference point for HBM byte counters)")
     return ap.parse_args()
@@ -131,20 +136,35 @@ def main() -> int:
                 k_scales[i][slot] = saved_scales[i][0]
                 v_scales[i][slot] = saved_scales[i][1]
 
+    # Stage boundaries (events): 0 | scores of every key -> selection scores | 1 | top-k | 2 | compaction | 3.
+    # Default: select_paged (one resident kernel when the shape has one, raw scores stay in
+    # LDS).  --two-pass: score_paged writes the raw scores, select normalises and reduces.
+    rows = w.num_seqs * w.num_kv_heads
+    fin_buf = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=dev)
+    two_pass = args.two_pass or ops.select_path(kv, batch, sc, sel) != "resident"
+    raw_buf = None
+    if two_pass:
+        raw_buf = torch.empty(w.num_seqs, w.num_layers, batch.max_seq_len, w.num_q_heads, dtype=torch.float32,
+                              device=dev)
+
     def step(events=None):
         if events is not None:
             events[0].record()
-        raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
-        if events is not None:
-            events[1].record()
-        ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
+        if two_pass:
+            raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
+            if events is not None:
+                events[1].record()
+            ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
+        else:
+            ops.select_paged(kv, batch, sc, sel, ws, scores_out=fin_buf, want_keep=False)
+            if events is not None:
+                events[1].record()
+            ops.topk_batch(fin_buf, batch, w.num_kv_heads, keep)
         if events is not None:
             events[2].record()
         ops.compact(kv, batch, keep)
         if events is not None:
             events[3].record()
-
-    raw_buf = torch.empty(w.num_seqs, w.num_layers, batch.max_seq_len, w.num_q_heads, dtype=torch.float32, device=dev)
 
     for _ in range(args.warmup):
         step()
@@ -197,14 +217,16 @@ def main() -> int:
         "achieved_gbs": step_gbs,
         "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "algorithmic_bytes": algo,
-        "stage_ms": {"score": mean(score_ms), "select": mean(select_ms), "compact": mean(compact_ms)},
+        "stage_ms": {"score": mean(score_ms), "select" if two_pass else "topk": mean(select_ms),
+                     "compact": mean(compact_ms)},
         "stage_gbs": {"score": score_gbs, "compact": compact_gbs},
         "key_vectors_per_s": total_keys * w.num_layers * w.num_kv_heads / (ms_per_step * 1e-3),
         "timed_region_wall_s": wall_s,
         "setup_s": setup_s,
-        "roofline": {"kernel": "score_mean_kernel", "bound": "hbm", "achieved": score_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_SCORE_TRAFFIC_BYTES.get(w.name)},
+        "path": "two_pass" if two_pass else "resident",
+        "roofline": {"kernel": "score_mean_kernel" if two_pass else "fused_select_kernel", "bound": "hbm",
+                     "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, two_pass))},
     }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)

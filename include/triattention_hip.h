@@ -112,6 +112,14 @@ int tri_fold_stats(const float* q_mean_real, const float* q_mean_imag, const flo
 uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
                              const tri_score_params* sp);
 
+/* Byte offset inside the workspace of a 32-bit status word: tri_select_paged and
+ * tri_compress_step clear it and the resident kernel sets it to non-zero if one of its
+ * bounded waits on another workgroup expired (results are then invalid).  The caller
+ * may read it after synchronising the stream.  Host-only; no counterpart in the
+ * reference. */
+uint64_t tri_workspace_status_offset(const tri_kv_layout* kv, const tri_batch* batch,
+                                     const tri_score_params* sp);
+
 /* Raw scores of every cached key of every sequence and layer, straight from the
  * paged blocks; replaces gather_request_k_dense_range + repeat_interleave +
  * compute_scores_triton per (layer, chunk) (runtime/selector_hf.py:860-894,
@@ -135,6 +143,25 @@ int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_
                const tri_select_params* sel, const float* raw, int64_t raw_stride_layer,
                int64_t raw_stride_token, int64_t raw_stride_head, float* final_scores,
                int32_t* keep, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* tri_score_paged + tri_select in one call, without the raw scores ever being handed to
+ * the caller: the device side of _select_keep_indices_for_group_per_head's paged branch
+ * (runtime/selector_hf.py:813-1033) and of the per-layer selector (:473-677).  When the
+ * shape allows (head_dim 128, at most four query heads per KV head, mean aggregation
+ * over offsets, power-of-two block size >= 4, layer_reduce >= 0, not shared, every
+ * sequence fits the GPU's LDS) one resident kernel keeps each layer's raw scores in LDS
+ * and they never reach memory; otherwise the two calls above run back to back on the
+ * workspace.  Outputs as tri_select; keep may be NULL when only final_scores is wanted
+ * (tri_topk_rows then turns them into keep rows). */
+int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                     const tri_select_params* sel, float* final_scores, int32_t* keep, void* workspace,
+                     uint64_t workspace_bytes, void* stream);
+
+/* Which path tri_select_paged / tri_compress_step take for these arguments on the
+ * current device: 1 = resident kernel, 0 = score then select, -1 = invalid arguments.
+ * Host-only.  No counterpart in the reference (it has a single path). */
+int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                    const tri_select_params* sel);
 
 /* Top-k of arbitrary fp32 rows (core/compressor.py:388-409): keep[r][0..k_r) =
  * ascending indices of the k_r largest of scores[r][0..len_r). */

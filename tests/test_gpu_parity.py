@@ -376,6 +376,77 @@ def test_end_to_end_c0_against_oracle():
     assert torch.equal(dev[:, blk, off].view(torch.int16), ref[:, blk, off].view(torch.int16))
 
 
+RESIDENT_CASES = {
+    "gqa4": dict(w=small()),
+    "ragged": dict(w=small(seq_lens=(300, 17, 1000, 256, 513, 1), num_layers=3)),
+    "hkv8": dict(w=small(num_q_heads=32, num_kv_heads=8, seq_lens=(700, 90), num_layers=4)),
+    "hkv5_g3": dict(w=small(num_q_heads=15, num_kv_heads=5, seq_lens=(333, 130))),
+    "hkv16": dict(w=small(num_q_heads=32, num_kv_heads=16, seq_lens=(450,))),
+    "hkv32_g1": dict(w=small(num_q_heads=32, num_kv_heads=32, seq_lens=(200, 77))),
+    "g1": dict(w=small(num_q_heads=2, num_kv_heads=2, seq_lens=(129,))),
+    "interleaved": dict(w=small(rope_style="interleaved")),
+    "fp16": dict(w=small(kv_dtype="fp16")),
+    "fp8": dict(w=small(kv_dtype="fp8", seq_lens=(300, 45))),
+    "block4": dict(w=small(block_size=4, seq_lens=(301,))),
+    "block64": dict(w=small(block_size=64, seq_lens=(500, 31))),
+    "kv_axis1": dict(w=small(seq_lens=(290, 64)), kv_axis=1),
+    "one_layer": dict(w=small(num_layers=1)),
+    "layer_max_group_mean": dict(w=small(num_layers=3), sel=dict(layer_reduce="max", group_reduce="mean")),
+    "no_normalize": dict(w=small(), sel=dict(normalize=False)),
+    "prefill_guard": dict(w=small(seq_lens=(400, 90)), sel=dict(protect_prefill=True), prefill_lens=[37, 5]),
+    "tw64": dict(w=small(seq_lens=(9000,) * 20, budget=512, num_layers=2)),
+    "tw128": dict(w=small(seq_lens=(40000, 3000, 25001), budget=2048, num_layers=2)),
+    "two_launches": dict(w=small(seq_lens=(70000, 100, 66000, 69000), budget=1024, num_layers=2)),
+}
+
+
+@pytest.mark.parametrize("name", list(RESIDENT_CASES))
+def test_resident_selection_matches_two_pass(name):
+    """The single resident kernel (raw scores kept in LDS) against score_paged + select:
+    same selection scores up to the rounding of differently grouped fp32 sums in the
+    statistics (the reference's streaming variance sumsq - n*mean^2 amplifies that
+    rounding by mean^2/var), same kept sets away from ties."""
+    case = dict(RESIDENT_CASES[name])
+    w = case["w"]
+    inp = build_inputs(w, case.get("kv_axis", 0))
+    print(f"case={name} workload={w}", flush=True)
+    caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=case.get("prefill_lens"))
+    selkw = dict(window_size=w.window_size)
+    selkw.update(case.get("sel", {}))
+    sel = ops.SelectConfig(**selkw)
+    assert ops.select_path(kv, batch, sc, sel) == "resident"
+    keep_r, fin_r, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    raw, ws2 = ops.score_paged(kv, batch, sc)
+    keep_t, fin_t = ops.select(kv, batch, sc, sel, raw, ws2, want_scores=True)
+    torch.cuda.synchronize()
+    assert ws.status() == 0
+    h = w.num_kv_heads
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        fr, ft = fin_r[b * h:(b + 1) * h, :t].cpu(), fin_t[b * h:(b + 1) * h, :t].cpu()
+        assert torch.equal(torch.isinf(fr), torch.isinf(ft))
+        finite = torch.isfinite(ft)
+        scale = float(ft[finite].abs().max()) if bool(finite.any()) else 1.0
+        assert float((fr[finite] - ft[finite]).abs().max() if bool(finite.any()) else 0.0) <= 5e-4 * scale, (name, b)
+        assert_keep_matches(keep_r[b * h:(b + 1) * h, :k].cpu().long(), keep_t[b * h:(b + 1) * h, :k].cpu().long(),
+                            ft, k, tie_tol=2e-3 * scale)
+
+
+def test_resident_path_falls_back_when_shape_has_no_kernel():
+    for kw, selkw in ((dict(num_q_heads=64, num_kv_heads=8), {}), (dict(head_dim=64), {}),
+                      (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
+        w = small(**kw)
+        inp = build_inputs(w)
+        caches, kv, batch, sc = device_objects(w, inp, DEV)
+        sel = ops.SelectConfig(window_size=w.window_size, **selkw)
+        assert ops.select_path(kv, batch, sc, sel) == "two_pass", (kw, selkw)
+        keep_a, fin_a, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+        raw, ws2 = ops.score_paged(kv, batch, sc)
+        keep_b, fin_b = ops.select(kv, batch, sc, sel, raw, ws2, want_scores=True)
+        torch.cuda.synchronize()
+        assert torch.equal(keep_a, keep_b) and torch.equal(fin_a[:, :300], fin_b[:, :300])
+
+
 def test_fp8_every_code_decodes_like_torch():
     """All 254 finite e4m3 codes through the scorer: with one non-zero coefficient the
     score is code_value * scale * coefficient, which pins the decoder against torch's

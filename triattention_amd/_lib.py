@@ -24,8 +24,9 @@ ROPE_HALF, ROPE_INTERLEAVED = 0, 1
 REDUCE_MEAN, REDUCE_MAX, REDUCE_NONE = 0, 1, -1
 
 EXPORTS = (
-    "tri_abi_version", "tri_last_error", "tri_fold_stats", "tri_workspace_bytes", "tri_score_paged",
-    "tri_select", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
+    "tri_abi_version", "tri_last_error", "tri_fold_stats", "tri_workspace_bytes", "tri_workspace_status_offset",
+    "tri_score_paged",
+    "tri_select", "tri_select_paged", "tri_select_path", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
     "tri_compact_paged_full", "tri_compress_step",
 )
 
@@ -88,10 +89,16 @@ def load() -> C.CDLL:
     lib.tri_fold_stats.argtypes = [P, P, P, P, I32, I32, I32, I32, I32, P, P]
     lib.tri_workspace_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams)]
     lib.tri_workspace_bytes.restype = U64
+    lib.tri_workspace_status_offset.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams)]
+    lib.tri_workspace_status_offset.restype = U64
     lib.tri_score_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
                                     P, I64, I64, I64, P, U64, P]
     lib.tri_select.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
                                C.POINTER(SelectParams), P, I64, I64, I64, P, P, P, U64, P]
+    lib.tri_select_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                     C.POINTER(SelectParams), P, P, P, U64, P]
+    lib.tri_select_path.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                    C.POINTER(SelectParams)]
     lib.tri_topk_rows.argtypes = [P, I64, I32, P, P, I32, I32, P, I32, P]
     lib.tri_compact_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), P, I32, I32, P]
     lib.tri_compact_full_staging_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch)]

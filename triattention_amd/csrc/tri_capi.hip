@@ -83,8 +83,12 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
 }
 
 tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
+  const tri::FusedPlan fused =
+      tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, sp->num_score_heads / kv->num_kv_heads,
+                      kv->block_size, b->block_table != nullptr, sp->aggregation, b->max_seq_len,
+                      tri::fused_resident_workgroups());
   return tri::plan_workspace(b->num_seqs, kv->num_layers, sp->num_score_heads, kv->head_dim / 2, sp->num_offsets,
-                             kv->num_kv_heads, b->max_seq_len);
+                             kv->num_kv_heads, b->max_seq_len, fused);
 }
 
 int check_workspace(const tri::Workspace& w, void* ws, uint64_t bytes) {
@@ -148,6 +152,48 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
   return launch_status(tri::launch_select(a, s), "select");
 }
 
+// Selection straight from the paged keys: the resident kernel when the shape has one,
+// else score into the workspace and select from there.
+int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                    const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
+                    hipStream_t s) {
+  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared;
+  if (!fused) {
+    float* raw = at<float>(ws, w.raw);
+    const int64_t A = sp->num_score_heads;
+    const int64_t rs_layer = (int64_t)batch->max_seq_len * A;
+    const int rc = do_score(kv, batch, sp, raw, rs_layer, A, 1, ws, w, s);
+    if (rc) return rc;
+    return do_select(kv, batch, sp, sel, raw, rs_layer, A, 1, fin, keep, ws, w, s);
+  }
+  const int F = kv->head_dim / 2;
+  hipError_t e = tri::launch_prepare(sp->folded, sp->omega, sp->offsets, sp->num_offsets, batch->round_start,
+                                     batch->num_seqs, kv->num_layers, sp->num_score_heads, F, sp->aggregation,
+                                     at<float>(ws, w.coef), at<float>(ws, w.trig), s);
+  if (e != hipSuccess) return launch_status(e, "prepare");
+  tri::FusedLaunch a{};
+  a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
+  a.block_size = kv->block_size; a.kv_dtype = kv->kv_dtype; a.rope_style = kv->rope_style;
+  a.A = sp->num_score_heads; a.G = sp->num_score_heads / kv->num_kv_heads; a.Tmax = batch->max_seq_len;
+  a.normalize = sel->normalize; a.window_size = sel->window_size; a.protect_prefill = sel->protect_prefill;
+  a.group_reduce = sel->group_reduce; a.layer_reduce = sel->layer_reduce;
+  a.stride_block = kv->stride_block; a.stride_token = kv->stride_token; a.stride_head = kv->stride_head;
+  a.k_layers = kv->k_layers; a.k_scale_layers = kv->k_scale_layers;
+  a.block_table = batch->block_table; a.block_table_pitch = batch->block_table_pitch;
+  a.seq_lens = batch->seq_lens; a.prefill_lens = batch->prefill_lens;
+  a.coef = at<float>(ws, w.coef);
+  a.xchg = at<unsigned long long>(ws, w.xchg);
+  a.status = at<uint32_t>(ws, w.status);
+  a.fin = fin ? fin : at<float>(ws, w.fin);
+  a.plan = w.fused;
+  e = tri::launch_fused_select(a, s);
+  if (e != hipSuccess) return launch_status(e, "fused_select");
+  if (!keep) return TRI_OK;   // selection scores only
+  return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, keep,
+                                             batch->max_budget, s),
+                       "topk_rows");
+}
+
 int fill_compact(const tri_kv_layout* kv, const tri_batch* batch, const int32_t* keep, int keep_per_layer,
                  int shared, tri::CompactLaunch& a) {
   int rc = check_layout(kv, true);
@@ -199,6 +245,14 @@ uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch, co
   return (uint64_t)plan(kv, batch, sp).total;
 }
 
+uint64_t tri_workspace_status_offset(const tri_kv_layout* kv, const tri_batch* batch,
+                                     const tri_score_params* sp) {
+  if (check_layout(kv, false) || check_batch(batch, false) || !sp || sp->num_score_heads <= 0 ||
+      sp->num_offsets <= 0)
+    return 0;
+  return (uint64_t)plan(kv, batch, sp).status;
+}
+
 int tri_score_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     float* raw, int64_t raw_stride_layer, int64_t raw_stride_token,
                     int64_t raw_stride_head, void* workspace, uint64_t workspace_bytes, void* stream) {
@@ -235,6 +289,32 @@ int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_
   if (rc) return rc;
   return do_select(kv, batch, sp, sel, raw, raw_stride_layer, raw_stride_token, raw_stride_head, final_scores,
                    keep, workspace, w, (hipStream_t)stream);
+}
+
+int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                     const tri_select_params* sel, float* final_scores, int32_t* keep, void* workspace,
+                     uint64_t workspace_bytes, void* stream) {
+  int rc = check_layout(kv, false);
+  if (rc) return rc;
+  rc = check_batch(batch, true);
+  if (rc) return rc;
+  rc = check_score(kv, sp);
+  if (rc) return rc;
+  rc = check_select(sel);
+  if (rc) return rc;
+  if (!batch->round_start) return fail(TRI_ERR_INVALID_ARGUMENT, "round_start is NULL");
+  if (!keep && !final_scores) return fail(TRI_ERR_INVALID_ARGUMENT, "keep and final_scores are both NULL");
+  const tri::Workspace w = plan(kv, batch, sp);
+  rc = check_workspace(w, workspace, workspace_bytes);
+  if (rc) return rc;
+  return do_select_paged(kv, batch, sp, sel, final_scores, keep, workspace, w, (hipStream_t)stream);
+}
+
+int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                    const tri_select_params* sel) {
+  if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
+  const tri::Workspace w = plan(kv, batch, sp);
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared) ? 1 : 0;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,
@@ -296,12 +376,7 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
   rc = check_workspace(w, workspace, workspace_bytes);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  float* raw = at<float>(workspace, w.raw);
-  const int64_t A = sp->num_score_heads;
-  const int64_t rs_layer = (int64_t)batch->max_seq_len * A;
-  rc = do_score(kv, batch, sp, raw, rs_layer, A, 1, workspace, w, s);
-  if (rc) return rc;
-  rc = do_select(kv, batch, sp, sel, raw, rs_layer, A, 1, nullptr, keep, workspace, w, s);
+  rc = do_select_paged(kv, batch, sp, sel, nullptr, keep, workspace, w, s);
   if (rc) return rc;
   tri::CompactLaunch c{};
   rc = fill_compact(kv, batch, keep, sel->layer_reduce < 0, sel->shared, c);

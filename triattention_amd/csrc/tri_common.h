@@ -14,9 +14,28 @@ constexpr int kScoreTileTokens = 512;   // tokens of one (sequence, layer) per s
 constexpr int kQPerPass = 4;            // query heads scored per wave pass
 constexpr int kPairsPerLane = 8;        // frequency pairs held by one lane
 constexpr int kMaxOffsets = 32;
+constexpr int kFusedWaves = 8;          // waves of a resident-scorer workgroup
+constexpr int kFusedThreads = kFusedWaves * kWave;
 
 inline __host__ __device__ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 inline __host__ __device__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline __host__ __device__ int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Geometry of the resident (single-kernel) score + reduce path; eligible == 0 when the
+// shape has no such kernel and the two-kernel path is used.
+struct FusedPlan {
+  int eligible;
+  int tw;               // tokens per wave
+  int HC;               // chunks of 8 KV heads; waves of a workgroup are split over them
+  int tile_tokens;      // tokens per workgroup
+  int tiles_per_seq;    // workgroups per sequence (by max_seq_len)
+  int seqs_per_launch;  // whole sequences per cooperative launch
+  int bs_shift;
+};
+// Workgroups of the resident kernel the current device can hold at once (0: none).
+int fused_resident_workgroups();
+FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
+                     int resident);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {
@@ -26,12 +45,16 @@ struct Workspace {
   int64_t mustd;     // [B][L][A][2] fp32 mean / safe std
   int64_t raw;       // [B][L][Tmax][A] fp32 raw scores (tri_compress_step)
   int64_t fin;       // [B*L*Hkv][Tmax] fp32 selection scores (worst case: per-layer selection)
+  int64_t xchg;      // [B][L][tiles_per_seq][A][2] tagged sums exchanged by the resident kernel
+  int64_t status;    // one word: non-zero when a bounded wait of the resident kernel expired
   int64_t total;
   int32_t num_tiles; // NT
+  FusedPlan fused;
 };
 
-inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int Tmax) {
+inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int Tmax, const FusedPlan& fused) {
   Workspace w{};
+  w.fused = fused;
   int64_t off = 0;
   auto take = [&](int64_t bytes) { int64_t o = off; off = align_up(off + bytes, 256); return o; };
   w.num_tiles = ceil_div(Tmax > 0 ? Tmax : 1, kScoreTileTokens);
@@ -41,6 +64,8 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.mustd = take((int64_t)B * L * A * 2 * 4);
   w.raw = take((int64_t)B * L * Tmax * A * 4);
   w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
+  w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
+  w.status = take(256);
   w.total = off;
   return w;
 }
@@ -89,6 +114,24 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
 hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
                             const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry,
                             int32_t* keep, int keep_pitch, hipStream_t s);
+
+struct FusedLaunch {
+  int B, L, Hkv, D, block_size, kv_dtype, rope_style, A, G, Tmax;
+  int normalize, window_size, protect_prefill, group_reduce, layer_reduce;
+  int64_t stride_block, stride_token, stride_head;
+  const void* const* k_layers;
+  const float* const* k_scale_layers;
+  const int32_t* block_table;
+  int block_table_pitch;
+  const int32_t* seq_lens;
+  const int32_t* prefill_lens;
+  const float* coef;             // workspace
+  unsigned long long* xchg;      // workspace
+  uint32_t* status;              // workspace
+  float* fin;                    // [B*Hkv][Tmax]
+  FusedPlan plan;
+};
+hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s);
 
 struct CompactLaunch {
   int B, L, Hkv, D, block_size, elem_bytes, max_budget;

@@ -312,6 +312,7 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   e = hipGetLastError();
   if (e != hipSuccess) return e;
 
+  if (!a.keep) return hipSuccess;   // selection scores only
   const int rows_per_entry = c.rows_per_seq * (per_layer ? a.L : 1);
   return launch_topk_rows(a.fin, a.Tmax, a.B * rows_per_entry, a.seq_lens, a.budgets, rows_per_entry, a.keep,
                           a.max_budget, s);

@@ -240,6 +240,13 @@ class Workspace:
         self.buf = torch.empty(self.bytes + 256, dtype=torch.uint8, device=kv.device)
         off = (-self.buf.data_ptr()) % 256
         self.ptr = self.buf.data_ptr() + off
+        self._status_at = off + int(lib.tri_workspace_status_offset(C.byref(kv.struct), C.byref(batch.struct),
+                                                                    C.byref(sp)))
+
+    def status(self) -> int:
+        """Synchronises, then returns the resident kernel's status word (0 = fine)."""
+        torch.cuda.synchronize(self.buf.device)
+        return int(self.buf[self._status_at:self._status_at + 4].view(torch.int32).item())
 
     def fits(self, kv, batch, sc) -> bool:
         sp = sc.struct()
@@ -304,6 +311,50 @@ def select(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, ra
     return keep, fin
 
 
+def select_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig,
+                 ws: Workspace | None = None, want_scores: bool = False, keep: torch.Tensor | None = None,
+                 scores_out: torch.Tensor | None = None, want_keep: bool = True):
+    """Score and select in one call; the raw scores stay on the device side (in LDS when
+    the shape has a resident kernel).  Returns (keep, selection scores or None, ws);
+    with want_keep=False only the selection scores are produced (see topk_batch)."""
+    lib = _lib.load()
+    _check_devices(kv, sc)
+    if batch.budgets is None:
+        raise ValueError("batch has no budgets")
+    batch.check_capacity(kv.block_size)
+    ws = ws if ws is not None and ws.fits(kv, batch, sc) else Workspace(kv, batch, sc)
+    rows = batch.num_seqs * (kv.num_layers if sel.layer_reduce is None else 1) * (1 if sel.shared else kv.num_kv_heads)
+    if not want_keep:
+        keep, want_scores = None, True
+    elif keep is None:
+        keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+    elif (keep.numel() != rows * batch.max_budget or keep.dtype != torch.int32 or not keep.is_contiguous()
+          or keep.device != kv.device):
+        raise ValueError(f"keep must be a contiguous int32 tensor with {rows} x {batch.max_budget} entries")
+    fin = None
+    if scores_out is not None:
+        if (tuple(scores_out.shape) != (rows, batch.max_seq_len) or scores_out.dtype != torch.float32
+                or not scores_out.is_contiguous() or scores_out.device != kv.device):
+            raise ValueError(f"scores_out must be a contiguous fp32 [{rows}, {batch.max_seq_len}] device tensor")
+        fin = scores_out
+    elif want_scores:
+        fin = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=kv.device)
+    sp, ss = sc.struct(), sel.struct()
+    _lib.check(lib.tri_select_paged(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss),
+                                    _ptr(fin), _ptr(keep), ws.ptr, ws.bytes, _stream()))
+    return keep, fin, ws
+
+
+def select_path(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig) -> str:
+    """'resident' when select_paged / compress_step run the single resident kernel for
+    these arguments on the current device, else 'two_pass'."""
+    sp, ss = sc.struct(), sel.struct()
+    rc = int(_lib.load().tri_select_path(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss)))
+    if rc < 0:
+        raise ValueError("invalid arguments: " + _lib.load().tri_last_error().decode("utf-8", "replace"))
+    return "resident" if rc == 1 else "two_pass"
+
+
 def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] | None = None) -> torch.Tensor:
     """Ascending int32 indices of the k largest entries of every row of a 2-D fp32 tensor."""
     lib = _lib.load()
@@ -319,6 +370,23 @@ def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] 
     lens_t, ks_t = _i32(ls, scores.device), _i32(ks, scores.device)
     _lib.check(lib.tri_topk_rows(_ptr(scores), int(scores.stride(0)), R, _ptr(lens_t), _ptr(ks_t), 1, T,
                                  _ptr(keep), kmax, _stream()))
+    return keep
+
+
+def topk_batch(scores: torch.Tensor, batch: StepBatch, rows_per_seq: int, keep: torch.Tensor | None = None):
+    """keep rows (ascending int32 [rows, max_budget]) from selection scores [rows, Tmax] with
+    the batch's own device-side lengths and budgets; rows_per_seq rows belong to a sequence."""
+    lib = _lib.load()
+    if batch.budgets is None:
+        raise ValueError("batch has no budgets")
+    rows, T = (int(x) for x in scores.shape)
+    if (rows != batch.num_seqs * rows_per_seq or T != batch.max_seq_len or scores.dtype != torch.float32
+            or not scores.is_contiguous()):
+        raise ValueError("scores must be the contiguous fp32 [rows, max_seq_len] tensor of select_paged")
+    if keep is None:
+        keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=scores.device)
+    _lib.check(lib.tri_topk_rows(_ptr(scores), T, rows, _ptr(batch.seq_lens), _ptr(batch.budgets), rows_per_seq, T,
+                                 _ptr(keep), batch.max_budget, _stream()))
     return keep
 
 
