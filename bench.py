@@ -29,9 +29,9 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # HBM bytes one launch of the dominant kernel moves on the C1 workload, from two rocprofv3
 # --pmc runs of this script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB; the factors are what
 # the same counters read for the 1 GiB copies of --copy-calibration).  Keyed by
-# (workload, two_pass); absent = not measured.
+# (workload, path); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_qwen3_8b_36l_b16_16k", True): 9_717_510 * 1024 * 2 + 1_184_256 * 1024,   # score_mean_kernel
+    ("c1_qwen3_8b_36l_b16_16k", "two_pass"): 9_717_510 * 1024 * 2 + 1_184_256 * 1024,   # score_mean_kernel
 }
 
 
@@ -141,7 +141,8 @@ def main() -> int:
     # LDS).  --two-pass: score_paged writes the raw scores, select normalises and reduces.
     rows = w.num_seqs * w.num_kv_heads
     fin_buf = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=dev)
-    two_pass = args.two_pass or ops.select_path(kv, batch, sc, sel) != "resident"
+    path = "two_pass" if args.two_pass else ops.select_path(kv, batch, sc, sel)
+    two_pass = path == "two_pass"
     raw_buf = None
     if two_pass:
         raw_buf = torch.empty(w.num_seqs, w.num_layers, batch.max_seq_len, w.num_q_heads, dtype=torch.float32,
@@ -223,10 +224,11 @@ def main() -> int:
         "key_vectors_per_s": total_keys * w.num_layers * w.num_kv_heads / (ms_per_step * 1e-3),
         "timed_region_wall_s": wall_s,
         "setup_s": setup_s,
-        "path": "two_pass" if two_pass else "resident",
-        "roofline": {"kernel": "score_mean_kernel" if two_pass else "fused_select_kernel", "bound": "hbm",
+        "path": path,
+        "roofline": {"kernel": {"two_pass": "score_mean_kernel", "resident_valu": "fused_select_kernel",
+                                "resident_mfma": "fused_mfma_kernel"}[path], "bound": "hbm",
                      "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, two_pass))},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, path))},
     }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)

@@ -148,7 +148,7 @@ int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_
  * the caller: the device side of _select_keep_indices_for_group_per_head's paged branch
  * (runtime/selector_hf.py:813-1033) and of the per-layer selector (:473-677).  When the
  * shape allows (head_dim 128, at most four query heads per KV head, mean aggregation
- * over offsets, power-of-two block size >= 4, layer_reduce >= 0, not shared, every
+ * over offsets, power-of-two block size, layer_reduce >= 0, not shared, every
  * sequence fits the GPU's LDS) one resident kernel keeps each layer's raw scores in LDS
  * and they never reach memory; otherwise the two calls above run back to back on the
  * workspace.  Outputs as tri_select; keep may be NULL when only final_scores is wanted
@@ -158,7 +158,8 @@ int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_
                      uint64_t workspace_bytes, void* stream);
 
 /* Which path tri_select_paged / tri_compress_step take for these arguments on the
- * current device: 1 = resident kernel, 0 = score then select, -1 = invalid arguments.
+ * current device: 2 = resident kernel scoring on the matrix cores (bf16 keys), 1 = resident
+ * kernel scoring on the vector unit, 0 = score then select, -1 = invalid arguments.
  * Host-only.  No counterpart in the reference (it has a single path). */
 int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel);

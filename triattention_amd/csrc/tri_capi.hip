@@ -2,6 +2,7 @@
 // then kernel launches on the caller's stream.  Nothing here allocates or waits.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "tri_common.h"
@@ -83,10 +84,20 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
 }
 
 tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
-  const tri::FusedPlan fused =
-      tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, sp->num_score_heads / kv->num_kv_heads,
-                      kv->block_size, b->block_table != nullptr, sp->aggregation, b->max_seq_len,
-                      tri::fused_resident_workgroups());
+  // bf16 keys go to the matrix-core kernel, other types to the vector-unit one;
+  // TRIATTN_RESIDENT_KERNEL=valu forces the vector-unit kernel (for comparison runs).
+  const char* force = getenv("TRIATTN_RESIDENT_KERNEL");
+  const bool want_mfma = kv->kv_dtype == TRI_KV_BF16 && !(force && strcmp(force, "valu") == 0);
+  const int G = sp->num_score_heads / kv->num_kv_heads;
+  const bool paged = b->block_table != nullptr;
+  const int resident = tri::fused_resident_workgroups();
+  tri::FusedPlan fused{};
+  if (want_mfma)
+    fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
+                                 sp->aggregation, b->max_seq_len, resident);
+  if (!fused.eligible)
+    fused = tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged, sp->aggregation,
+                            b->max_seq_len, resident);
   return tri::plan_workspace(b->num_seqs, kv->num_layers, sp->num_score_heads, kv->head_dim / 2, sp->num_offsets,
                              kv->num_kv_heads, b->max_seq_len, fused);
 }
@@ -186,7 +197,8 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.status = at<uint32_t>(ws, w.status);
   a.fin = fin ? fin : at<float>(ws, w.fin);
   a.plan = w.fused;
-  e = tri::launch_fused_select(a, s);
+  a.bmat = at<char>(ws, w.bmat);
+  e = w.fused.eligible == 2 ? tri::launch_fused_mfma(a, s) : tri::launch_fused_select(a, s);
   if (e != hipSuccess) return launch_status(e, "fused_select");
   if (!keep) return TRI_OK;   // selection scores only
   return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, keep,
@@ -314,7 +326,7 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared) ? 1 : 0;
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared) ? w.fused.eligible : 0;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,

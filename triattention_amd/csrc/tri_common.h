@@ -24,18 +24,20 @@ inline __host__ __device__ int64_t ceil_div64(int64_t a, int64_t b) { return (a 
 // Geometry of the resident (single-kernel) score + reduce path; eligible == 0 when the
 // shape has no such kernel and the two-kernel path is used.
 struct FusedPlan {
-  int eligible;
+  int eligible;         // 0: none, 1: vector-unit kernel, 2: matrix-core kernel
   int tw;               // tokens per wave
   int HC;               // chunks of 8 KV heads; waves of a workgroup are split over them
   int tile_tokens;      // tokens per workgroup
   int tiles_per_seq;    // workgroups per sequence (by max_seq_len)
-  int seqs_per_launch;  // whole sequences per cooperative launch
+  int seqs_per_launch;  // whole sequences per launch
   int bs_shift;
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                      int resident);
+FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
+                          int resident);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {
@@ -47,6 +49,7 @@ struct Workspace {
   int64_t fin;       // [B*L*Hkv][Tmax] fp32 selection scores (worst case: per-layer selection)
   int64_t xchg;      // [B][L][tiles_per_seq][A][2] tagged sums exchanged by the resident kernel
   int64_t status;    // one word: non-zero when a bounded wait of the resident kernel expired
+  int64_t bmat;      // [B][L][Hkv][6][64][8] bf16 coefficient slabs of the matrix-core kernel
   int64_t total;
   int32_t num_tiles; // NT
   FusedPlan fused;
@@ -66,6 +69,7 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
   w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
   w.status = take(256);
+  w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * 6 * 64 * 16 : 0);
   w.total = off;
   return w;
 }
@@ -128,10 +132,12 @@ struct FusedLaunch {
   const float* coef;             // workspace
   unsigned long long* xchg;      // workspace
   uint32_t* status;              // workspace
+  void* bmat;                    // workspace (matrix-core kernel)
   float* fin;                    // [B*Hkv][Tmax]
   FusedPlan plan;
 };
 hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s);
+hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s);
 
 struct CompactLaunch {
   int B, L, Hkv, D, block_size, elem_bytes, max_budget;

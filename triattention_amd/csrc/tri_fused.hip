@@ -7,8 +7,8 @@
 // consumed once every token of that layer has been scored.  The two-kernel path writes
 // them to memory (128 bytes per token and layer); here they stay in LDS instead:
 //
-//  * one workgroup per tile of a sequence, all tiles of the launch resident at once
-//    (cooperative launch, one workgroup per CU); a wave owns TW tokens and keeps their
+//  * one workgroup per tile of a sequence and at most one workgroup per CU in a launch, so
+//    all tiles of the launch are resident at once; a wave owns TW tokens and keeps their
 //    raw scores of one layer in a ring of TW + SL slots in LDS;
 //  * after a layer, each workgroup publishes its per-head sum / sum of squares as 8-byte
 //    words (value, layer tag) with device-scope atomic stores; consumers poll the tagged
@@ -21,58 +21,16 @@
 //  * the key loads are one continuous double-buffered stream across layer boundaries.
 //
 // Each wave waits only on data other workgroups publish unconditionally, so progress
-// needs nothing but co-residency, which the cooperative launch guarantees; every wait is
+// needs nothing but every workgroup of the launch getting a CU, which holds because a
+// launch never has more workgroups than the device has CUs (workgroups that must queue
+// behind another stream's kernels start late, they are never starved).  Every wait is
 // also bounded in time and raises a status word instead of spinning forever.
 #include "tri_common.h"
 #include "tri_score_device.h"
+#include "tri_fused_device.h"
 
 namespace tri {
 namespace {
-
-constexpr int kFusedLdsLimit = 160 * 1024;
-
-struct FusedArgs {
-  const void* const* k_layers;
-  const float* const* k_scale_layers;
-  const int32_t* block_table;
-  const int32_t* seq_lens;
-  const int32_t* prefill_lens;
-  const float* coef;              // [B][L][A][3][F]
-  unsigned long long* xchg;       // [B][L][tiles_per_seq][A][2]: (tag << 32) | float bits
-  float* fin;                     // [B * Hkv][Tmax]
-  uint32_t* status;
-  int64_t stride_block, stride_token, stride_head;
-  int L, Hkv, A, G, HC;
-  int block_size, bs_shift, block_table_pitch;
-  int tiles_per_seq, tile_tokens, seq_base, num_seqs, Tmax;
-  int normalize, window_size, protect_prefill, group_reduce, layer_reduce;
-  long long spin_ticks;
-};
-
-__device__ __forceinline__ unsigned long long xchg_load(const unsigned long long* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void xchg_store(unsigned long long* p, unsigned long long v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Entry l of a device-resident table of pointers, read through the constant address space:
-// a scalar load (tracked by its own counter), where a vector load would make the wave
-// wait for every key load issued before it.  The tables are never written by a kernel.
-__device__ __forceinline__ const char* table_entry(const void* const* table, int l) {
-  typedef const __attribute__((address_space(4))) uint64_t* ConstU64;
-  return reinterpret_cast<const char*>(((ConstU64)(uintptr_t)table)[l]);
-}
-
-// A wave-uniform address, pinned to scalar registers: 64-bit address arithmetic may be
-// done on the vector unit, and a buffer descriptor built from vector registers costs a
-// readfirstlane loop around every load that uses it.
-__device__ __forceinline__ void* uniform_ptr(const void* p) {
-  const uint64_t v = reinterpret_cast<uint64_t>(p);
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
-}
 
 template <int DT, bool IL, int TW, int SL>
 __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a) {
@@ -280,56 +238,6 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
     }
   };
 
-  // mean / safe std of layer l for every score head of the sequence -> stats[l & 1].
-  auto gather_stats = [&](int l) __attribute__((always_inline)) {
-    float* st = stats + (l & 1) * a.A * 2;
-    const unsigned long long* in = a.xchg + (int64_t)(b * a.L + l) * a.tiles_per_seq * a.A * 2;
-    const uint32_t want = (uint32_t)(l + 1);
-    const long long t_begin = wall_clock64();
-    const int items = a.A * 2;
-    for (int base = 0; base < items; base += 64) {
-      const int item = base + lane;
-      const bool live = item < items;
-      double acc = 0.0;
-      for (int t0 = 0; t0 < seq_tiles; t0 += 8) {
-        unsigned long long w[8];
-        for (;;) {
-          bool ok = true;
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int t = min(t0 + u, seq_tiles - 1);
-            w[u] = live ? xchg_load(in + (int64_t)t * a.A * 2 + item) : ((unsigned long long)want << 32);
-            ok = ok && (uint32_t)(w[u] >> 32) == want;
-          }
-          if (__all(ok) || aborted) break;
-          if (wall_clock64() - t_begin > a.spin_ticks ||
-              __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-            aborted = true;
-            if (lane == 0) atomicExch(a.status, 1u);
-          }
-          __builtin_amdgcn_s_sleep(4);
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (t0 + u < seq_tiles) acc += (double)__uint_as_float((uint32_t)w[u]);
-      }
-      // Lanes 2i / 2i+1 hold the sum and the sum of squares of score head (base/2 + i);
-      // the reference's streaming formula on fp32 sums (runtime/selector_hf.py:902-909).
-      const float mine = (float)acc;
-      const float other = __shfl_xor(mine, 1);
-      const float sum = (lane & 1) ? other : mine;
-      const float sumsq = (lane & 1) ? mine : other;
-      const float cnt = (float)T;
-      const float mean = __fdiv_rn(sum, cnt);
-      float var = 0.f;
-      if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(mean, mean))), (float)(T - 1));
-      var = fmaxf(var, 0.f);
-      float sd = __fsqrt_rn(var);
-      if (sd < 1e-8f) sd = 1.f;
-      if (live) st[item] = (lane & 1) ? sd : mean;
-    }
-  };
-
   float fin[TW / 8];
 #pragma unroll
   for (int k = 0; k < TW / 8; ++k) fin[k] = 0.f;
@@ -353,7 +261,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
       }
       won = __builtin_amdgcn_readfirstlane(won);
       if (won) {
-        gather_stats(l);
+        gather_layer_stats(a, b, l, seq_tiles, T, 0, a.A * 2, stats + (l & 1) * a.A * 2, lane, aborted);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0) __hip_atomic_store(ready, (uint32_t)(l + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
       } else {
@@ -458,12 +366,6 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
   }
 }
 
-__global__ void fused_clear_kernel(unsigned long long* xchg, int64_t words, uint32_t* status) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < words) xchg[i] = 0ull;
-  if (i == 0) *status = 0u;
-}
-
 template <int TW, int SL>
 size_t fused_lds_bytes(int A, int tile_tokens, int bs_shift, bool paged) {
   const int blocks = paged ? (tile_tokens >> bs_shift) + 2 : 0;
@@ -480,8 +382,9 @@ hipError_t launch_fused_t(FusedArgs& k, int seqs_per_launch, int B, hipStream_t 
   for (int base = 0; base < B; base += seqs_per_launch) {
     k.seq_base = base;
     const int n = min(seqs_per_launch, B - base);
-    void* params[] = {&k};
-    e = hipLaunchCooperativeKernel(fn, dim3(n * k.tiles_per_seq), dim3(kFusedThreads), params, (unsigned)lds, s);
+    hipLaunchKernelGGL((fused_select_kernel<DT, IL, TW, SL>), dim3(n * k.tiles_per_seq), dim3(kFusedThreads), lds, s,
+                       k);
+    e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
@@ -505,10 +408,9 @@ int fused_resident_workgroups() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
   if (cached[dev] == 0) {
-    int cus = 0, coop = 0;
+    int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
-    if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess) coop = 0;
-    cached[dev] = (coop && cus > 0) ? cus : -1;
+    cached[dev] = cus > 0 ? cus : -1;
   }
   return cached[dev] > 0 ? cached[dev] : 0;
 }

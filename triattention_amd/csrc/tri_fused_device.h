@@ -1,0 +1,117 @@
+// Pieces shared by the two resident score + reduce kernels (tri_fused.hip: vector-unit
+// scoring; tri_fused_mfma.hip: matrix-core scoring): kernel arguments, the tagged-word
+// exchange between workgroups, and scalar-register helpers.
+#pragma once
+
+#include "tri_common.h"
+
+namespace tri {
+namespace {
+
+constexpr int kFusedLdsLimit = 160 * 1024;
+
+struct FusedArgs {
+  const void* const* k_layers;
+  const float* const* k_scale_layers;
+  const int32_t* block_table;
+  const int32_t* seq_lens;
+  const int32_t* prefill_lens;
+  const float* coef;              // [B][L][A][3][F]
+  unsigned long long* xchg;       // [B][L][tiles_per_seq][A][2]: (tag << 32) | float bits
+  float* fin;                     // [B * Hkv][Tmax]
+  uint32_t* status;
+  int64_t stride_block, stride_token, stride_head;
+  int L, Hkv, A, G, HC;
+  int block_size, bs_shift, block_table_pitch;
+  int tiles_per_seq, tile_tokens, seq_base, num_seqs, Tmax;
+  int normalize, window_size, protect_prefill, group_reduce, layer_reduce;
+  long long spin_ticks;
+};
+
+__device__ __forceinline__ unsigned long long xchg_load(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void xchg_store(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Entry l of a device-resident table of pointers, read through the constant address space:
+// a scalar load (tracked by its own counter), where a vector load would make the wave
+// wait for every key load issued before it.  The tables are never written by a kernel.
+__device__ __forceinline__ const char* table_entry(const void* const* table, int l) {
+  typedef const __attribute__((address_space(4))) uint64_t* ConstU64;
+  return reinterpret_cast<const char*>(((ConstU64)(uintptr_t)table)[l]);
+}
+
+// A wave-uniform address, pinned to scalar registers: 64-bit address arithmetic may be
+// done on the vector unit, and a buffer descriptor built from vector registers costs a
+// readfirstlane loop around every load that uses it.
+__device__ __forceinline__ void* uniform_ptr(const void* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+}
+
+// Clears the exchange words and the status word before a launch sequence.
+__global__ void fused_clear_kernel(unsigned long long* xchg, int64_t words, uint32_t* status) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < words) xchg[i] = 0ull;
+  if (i == 0) *status = 0u;
+}
+
+// Mean and safe standard deviation, over all tokens of sequence b, of layer l's raw scores
+// for `items / 2` consecutive score heads starting at head ah0: waits (bounded) until every
+// tile of the sequence has published its tagged sums, adds them in tile order in double,
+// then applies the reference's streaming formula on the fp32 sums
+// (runtime/selector_hf.py:902-909).  st[2*i] = mean, st[2*i + 1] = std of head ah0 + i.
+// Called by one whole wave.
+__device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, int l, int seq_tiles, int T, int ah0,
+                                                   int items, float* st, int lane, bool& aborted) {
+  const unsigned long long* in = a.xchg + ((int64_t)(b * a.L + l) * a.tiles_per_seq * a.A + ah0) * 2;
+  const uint32_t want = (uint32_t)(l + 1);
+  const long long t_begin = wall_clock64();
+  for (int base = 0; base < items; base += 64) {
+    const int item = base + lane;
+    const bool live = item < items;
+    double acc = 0.0;
+    for (int t0 = 0; t0 < seq_tiles; t0 += 8) {
+      unsigned long long w[8];
+      for (;;) {
+        bool ok = true;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = min(t0 + u, seq_tiles - 1);
+          w[u] = live ? xchg_load(in + (int64_t)t * a.A * 2 + item) : ((unsigned long long)want << 32);
+          ok = ok && (uint32_t)(w[u] >> 32) == want;
+        }
+        if (__all(ok) || aborted) break;
+        if (wall_clock64() - t_begin > a.spin_ticks ||
+            __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+          aborted = true;
+          if (lane == 0) atomicExch(a.status, 1u);
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (t0 + u < seq_tiles) acc += (double)__uint_as_float((uint32_t)w[u]);
+    }
+    // Lanes 2i / 2i+1 hold the sum and the sum of squares of head ah0 + base/2 + i.
+    const float mine = (float)acc;
+    const float other = __shfl_xor(mine, 1);
+    const float sum = (lane & 1) ? other : mine;
+    const float sumsq = (lane & 1) ? mine : other;
+    const float cnt = (float)T;
+    const float mean = __fdiv_rn(sum, cnt);
+    float var = 0.f;
+    if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(mean, mean))), (float)(T - 1));
+    var = fmaxf(var, 0.f);
+    float sd = __fsqrt_rn(var);
+    if (sd < 1e-8f) sd = 1.f;
+    if (live) st[item] = (lane & 1) ? sd : mean;
+  }
+}
+
+}  // namespace
+}  // namespace tri

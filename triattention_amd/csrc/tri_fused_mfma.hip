@@ -1,0 +1,490 @@
+// Resident score + normalise + reduce kernel with the contraction on the matrix cores
+// (gfx950, v_mfma_f32_16x16x32_bf16).  Same structure as tri_fused.hip (raw scores of a
+// layer stay in LDS, per-layer statistics exchanged through tagged words, one continuous
+// stream of key loads), different mapping of the arithmetic:
+//
+//   raw[n][q] = sum_e k[n][e] * C[e][q]  +  sum_f |k_f[n]| * E[f][q]
+//
+// with k[n][.] the 128 cached elements of one KV head of token n (bf16, exact), C the P / R
+// coefficients laid out per element, E the magnitude coefficients.  One wave owns one KV
+// head.  An MFMA multiplies a 16-token x 32-element slab of keys, taken straight from the
+// 16-byte loads (no unpacking), with a 32 x 16 coefficient slab whose columns are
+// (query head, split): every fp32 coefficient is carried as three bf16 pieces
+// c = c1 + c2 + c3, so the products are exact and the sum is an fp32 accumulation of the
+// same terms the vector-unit kernel adds.  The magnitudes are evaluated on the vector unit
+// in fp32 (sqrt(k_r^2 + k_i^2)), cut into two bf16 pieces and contracted the same way.
+// The three column groups of a query head are added with row rotations, which leaves every
+// token's four scores spread over the lanes exactly as the ring in LDS wants them.
+//
+// Per 16 tokens of a head: 8 MFMAs, and vector work only for the magnitudes (about 40 %
+// of the vector-unit kernel's instruction count), so the kernel is bound by the key stream.
+#include "tri_common.h"
+#include "tri_score_device.h"
+#include "tri_fused_device.h"
+
+namespace tri {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kDppRor4 = 0x124;   // row_ror:4
+constexpr int kDppRor8m = 0x128;  // row_ror:8
+
+// Four 16-byte chunks of one (token, head) row per lane: chunk 4*s + kb for s = 0..3, where
+// kb = lane / 16 and the token is lane % 16 of the step.
+struct StepData {
+  uint4 c[4];
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(const uint4& v) { return __builtin_bit_cast(bf16x8, v); }
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Two fp32 values -> packed bf16 (round to nearest even) and the fp32 remainders.
+__device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, float& r1) {
+  const f32x2 x = {x0, x1};
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+  r0 = x0 - bf16_lo(packed);
+  r1 = x1 - bf16_hi(packed);
+  return packed;
+}
+
+// Coefficient slabs of one (sequence, layer, head) in MFMA B-operand order:
+// bmat[((b*L + l)*Hkv + head)*6 + o][lane][8] bf16.  Operand o: 0..3 the key chunks
+// 4*o + kb, 4 and 5 the magnitudes of pair sets 0 and 1.  Lane (j = lane % 16, kb):
+// column j = (query head j % 4, split j / 4); element e = k index kb*8 + e of the slab.
+template <bool IL>
+__global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int64_t n_heads_total, uint4* bmat) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (head instance, operand, lane)
+  if (idx >= n_heads_total * 6 * 64) return;
+  const int lane = (int)(idx % 64);
+  const int o = (int)((idx / 64) % 6);
+  const int64_t hi = idx / (64 * 6);                 // (b*L + l)*Hkv + head
+  const int head = (int)(hi % Hkv);
+  const int64_t bl = hi / Hkv;
+  const int j = lane & 15, kb = lane >> 4;
+  const int q = j & 3, sp = j >> 2;
+  uint32_t out[4] = {0, 0, 0, 0};
+  if (q < G && sp < 3) {
+    const float* c = coef + ((bl * A + (int64_t)head * G + q) * 3) * 64;   // [P | R | E][64]
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      int which, pair;   // which: 0 = P, 1 = R, 2 = E
+      if (o < 4) {
+        const int chunk = 4 * o + kb;
+        if (IL) { which = e & 1; pair = chunk * 4 + (e >> 1); }
+        else { which = chunk >= 8 ? 1 : 0; pair = (chunk & 7) * 8 + e; }
+      } else {
+        which = 2;
+        const int set = o - 4;
+        if (IL) pair = (4 * (2 * set + (e >> 2)) + kb) * 4 + (e & 3);   // chunks of steps 2*set, 2*set+1
+        else pair = (4 * set + kb) * 8 + e;                               // real chunk 4*set + kb
+      }
+      float x = c[which * 64 + pair];
+      // piece sp of x = x1 + x2 + x3 (each bf16, round to nearest even)
+      for (int s = 0; s < sp; ++s) x = x - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x) << 16);
+      v[e] = x;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const f32x2 x = {v[2 * e], v[2 * e + 1]};
+      out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    }
+  }
+  bmat[idx] = uint4{out[0], out[1], out[2], out[3]};
+}
+
+template <int DT, bool IL, int TW, int SL>
+__global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
+  constexpr int RING = TW + SL;
+  extern __shared__ __align__(16) float lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int chunk = blockIdx.x % a.HC;
+  const int tile = (blockIdx.x / a.HC) % a.tiles_per_seq;
+  const int b = a.seq_base + blockIdx.x / (a.HC * a.tiles_per_seq);
+  if (b >= a.num_seqs) return;
+  const int T = a.seq_lens[b];
+  const int n0 = tile * a.tile_tokens;
+  if (n0 >= T) return;
+  const int n1 = min(n0 + a.tile_tokens, T);
+  const int ntok = n1 - n0;
+  const int last_tok = n1 - 1;
+  const int seq_tiles = ceil_div(T, a.tile_tokens);
+  const int heads_here = min(8, a.Hkv - chunk * 8);
+
+  float* ring = lds + wave * (RING * 4);                       // [RING][4 query heads]
+  float* part = lds + kFusedWaves * (RING * 4);                // [waves][64][2]
+  float* stats = part + kFusedWaves * 128;                     // [2][32 score heads][2]
+  uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128);    // arrive count, claimed, ready
+  int* lds_blk = reinterpret_cast<int*>(ctl + 8);
+
+  for (int i = threadIdx.x; i < kFusedWaves * 128; i += kFusedThreads) part[i] = 0.f;
+  if (threadIdx.x < 8) ctl[threadIdx.x] = 0;
+  int lb0 = 0;
+  if (a.block_table_pitch >= 0) {
+    lb0 = n0 >> a.bs_shift;
+    const int lb1 = last_tok >> a.bs_shift;
+    for (int i = threadIdx.x; i <= lb1 - lb0; i += kFusedThreads)
+      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
+  }
+  __syncthreads();
+  // From here on the waves of the workgroup run independently.
+  if (wave >= heads_here) return;
+  const int head = chunk * 8 + wave;
+
+  const int j = lane & 15, kb = lane >> 4;       // MFMA column / k block; also output row block
+  const int q = j & 3, rsel = j >> 2;
+  const bool q_ok = q < a.G;
+
+  // Coefficient slabs of the current layer.
+  uint4 B[6];
+  auto load_coefs = [&](int l) __attribute__((always_inline)) {
+    const uint4* p = bmat + (((int64_t)(b * a.L + l) * a.Hkv + head) * 6) * 64 + lane;
+#pragma unroll
+    for (int o = 0; o < 6; ++o) B[o] = p[o * 64];
+  };
+
+  // Element offset of this lane inside a (token, head) row and of its head inside a token.
+  const int64_t lane_elems = (int64_t)head * a.stride_head + kb * 8;
+
+  // Sixteen tokens of layer l starting at local token t (t % 16 == 0): lane's token is
+  // t + lane % 16, clamped to the tile's last token (loaded, never stored).
+  auto load_step = [&](StepData& d, int l, int t) __attribute__((always_inline)) {
+    const char* kbase = table_entry(a.k_layers, l);
+    const int n = min(n0 + t + j, last_tok);
+    int64_t row;
+    if (a.block_table_pitch < 0) {
+      row = (int64_t)b * a.stride_block + (int64_t)n * a.stride_token;
+    } else {
+      const int lb = n >> a.bs_shift;
+      row = (int64_t)lds_blk[lb - lb0] * a.stride_block + (int64_t)(n - (lb << a.bs_shift)) * a.stride_token;
+    }
+    GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + (row + lane_elems) * 2;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const u32x4 v = *(GlobalU4)(p + s * 64);
+      d.c[s] = uint4{v.x, v.y, v.z, v.w};
+    }
+  };
+
+  float s1 = 0.f, s2 = 0.f;
+  // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
+  // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
+  auto compute_step = [&](const StepData& d, int l, int t) __attribute__((always_inline)) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(d.c[s]), as_bf16x8(B[s]), acc, 0, 0, 0);
+    f32x4 acc_e = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int set = 0; set < 2; ++set) {
+      float mag[8];
+      if (IL) {
+        // chunks 2*set and 2*set + 1 hold four (real, imaginary) pairs each
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint4& cc = d.c[2 * set + (e >> 2)];
+          const uint32_t w = (&cc.x)[e & 3];
+          const float kr = bf16_lo(w), ki = bf16_hi(w);
+          mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
+        }
+      } else {
+        // real parts in chunk `set`, imaginary parts in chunk `set + 2`
+        const uint4& cr = d.c[set];
+        const uint4& ci = d.c[set + 2];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t wr = (&cr.x)[e >> 1], wi = (&ci.x)[e >> 1];
+          const float kr = (e & 1) ? bf16_hi(wr) : bf16_lo(wr);
+          const float ki = (e & 1) ? bf16_hi(wi) : bf16_lo(wi);
+          mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
+        }
+      }
+      uint4 hi, lo;
+      float r[8];
+      hi.x = split_pair(mag[0], mag[1], r[0], r[1]);
+      hi.y = split_pair(mag[2], mag[3], r[2], r[3]);
+      hi.z = split_pair(mag[4], mag[5], r[4], r[5]);
+      hi.w = split_pair(mag[6], mag[7], r[6], r[7]);
+      float unused0, unused1;
+      lo.x = split_pair(r[0], r[1], unused0, unused1);
+      lo.y = split_pair(r[2], r[3], unused0, unused1);
+      lo.z = split_pair(r[4], r[5], unused0, unused1);
+      lo.w = split_pair(r[6], r[7], unused0, unused1);
+      acc_e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(hi), as_bf16x8(B[4 + set]), acc_e, 0, 0, 0);
+      acc_e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(lo), as_bf16x8(B[4 + set]), acc_e, 0, 0, 0);
+    }
+    float v = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = acc[r] + acc_e[r];
+      x += dpp<kDppRor8m>(x);
+      x += dpp<kDppRor4>(x);
+      v = (rsel == r) ? x : v;
+    }
+    const int tl = t + 4 * kb + rsel;
+    if (q_ok && tl < ntok) {
+      ring[((uint32_t)(l * TW + tl) % RING) * 4 + q] = v;
+      s1 += v;
+      s2 = fmaf(v, v, s2);
+    }
+  };
+
+  bool aborted = false;
+  uint32_t* arrive_cnt = ctl;
+  uint32_t* claimed = ctl + 1;
+  uint32_t* ready = ctl + 2;
+  const int items = heads_here * a.G * 2;        // (score head, sum | sum of squares) of this workgroup
+  const int ah0 = chunk * 8 * a.G;
+
+  // Deposit this wave's sums of layer l; the last wave of the workgroup to do so adds the
+  // lanes in a fixed order and publishes the tile's sums.  Every wave deposits layer l
+  // before any wave deposits layer l + 1 (a wave consumes layer l, which needs every
+  // deposit of layer l, before it finishes layer l + 1), so the counter never mixes layers.
+  auto arrive = [&](int l) __attribute__((always_inline)) {
+    part[(wave * 64 + lane) * 2] = s1;
+    part[(wave * 64 + lane) * 2 + 1] = s2;
+    s1 = 0.f;
+    s2 = 0.f;
+    uint32_t prev = 0;
+    if (lane == 0) prev = __hip_atomic_fetch_add(arrive_cnt, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+    prev = __builtin_amdgcn_readfirstlane(prev);
+    if (prev + 1 != (uint32_t)(l + 1) * (uint32_t)heads_here) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (lane < items) {
+      const int ahl = lane >> 1, which = lane & 1;
+      const int w = ahl / a.G, qq = ahl - w * a.G;
+      float t = 0.f;
+      for (int i = 0; i < 16; ++i) t += part[(w * 64 + (i >> 2) * 16 + (i & 3) * 4 + qq) * 2 + which];
+      unsigned long long* out = a.xchg + (((int64_t)(b * a.L + l) * a.tiles_per_seq + tile) * a.A + ah0) * 2;
+      xchg_store(out + lane, ((unsigned long long)(uint32_t)(l + 1) << 32) | __float_as_uint(t));
+    }
+  };
+
+  float fin[TW / 64];
+#pragma unroll
+  for (int k = 0; k < TW / 64; ++k) fin[k] = 0.f;
+  const int prefill = (a.protect_prefill && a.prefill_lens) ? a.prefill_lens[b] : 0;
+  const int window_from = a.window_size > 0 ? T - min(a.window_size, T) : T;
+
+  // Turn layer l's ring entries into selection-score contributions (lane = token).
+  auto consume = [&](int l) __attribute__((always_inline)) {
+    float mean[4] = {0.f, 0.f, 0.f, 0.f}, sd[4] = {1.f, 1.f, 1.f, 1.f};
+    if (a.normalize) {
+      uint32_t won = 0;
+      if (lane == 0) {
+        uint32_t expect = (uint32_t)l;
+        won = __hip_atomic_compare_exchange_strong(claimed, &expect, (uint32_t)(l + 1), __ATOMIC_ACQ_REL,
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) ? 1u : 0u;
+      }
+      won = __builtin_amdgcn_readfirstlane(won);
+      if (won) {
+        gather_layer_stats(a, b, l, seq_tiles, T, ah0, items, stats + (l & 1) * 64, lane, aborted);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0) __hip_atomic_store(ready, (uint32_t)(l + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      } else {
+        // The claiming wave always finishes (its own waits are bounded).
+        while (__hip_atomic_load(ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)(l + 1))
+          __builtin_amdgcn_s_sleep(2);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      const float* st = stats + (l & 1) * 64;
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq)
+        if (qq < a.G) {
+          mean[qq] = st[(wave * a.G + qq) * 2];
+          sd[qq] = st[(wave * a.G + qq) * 2 + 1];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < TW / 64; ++k) {
+      const int tl = lane + 64 * k;
+      if (tl >= ntok) continue;
+      const float4 x = *reinterpret_cast<const float4*>(&ring[((uint32_t)(l * TW + tl) % RING) * 4]);
+      const float xs[4] = {x.x, x.y, x.z, x.w};
+      float v;
+      if (a.group_reduce == TRI_REDUCE_MAX) {
+        v = -INFINITY;
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq)
+          if (qq < a.G) v = fmaxf(v, __fdiv_rn(__fsub_rn(xs[qq], mean[qq]), sd[qq]));
+      } else {
+        v = 0.f;
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq)
+          if (qq < a.G) v = __fadd_rn(v, __fdiv_rn(__fsub_rn(xs[qq], mean[qq]), sd[qq]));
+        v = __fdiv_rn(v, (float)a.G);
+      }
+      const int n = n0 + tl;
+      if (n >= window_from || n < prefill) v = INFINITY;
+      if (l == 0) fin[k] = v;
+      else fin[k] = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(fin[k], v) : __fadd_rn(fin[k], v);
+    }
+  };
+
+  // ---- one continuous stream of key rows over (layer, step of 16 tokens).  Four step
+  // buffers rotate; a buffer is refilled as soon as it has been scored.  A layer is padded to
+  // whole rotations (padding steps re-read the last row and are not scored); the rotations
+  // form inner loops that contain nothing but key loads and scoring, and the work at layer
+  // boundaries sits between them.
+  const int nsteps = (ntok + 15) >> 4;
+  const int rotations = (nsteps + 3) >> 2;
+  const int rot_before_consume = min(SL / 64, rotations);
+  int ld_l = 0, ld_slot = 0;
+  auto fetch = [&](StepData& d) __attribute__((always_inline)) {
+    const int l = __builtin_amdgcn_readfirstlane(min(ld_l, a.L - 1));
+    const int t = __builtin_amdgcn_readfirstlane(min(ld_slot, nsteps - 1) * 16);
+    load_step(d, l, t);
+    if (++ld_slot >= rotations * 4) { ld_slot = 0; ++ld_l; }
+  };
+  auto score = [&](const StepData& d, int l, int slot) __attribute__((always_inline)) {
+    if (slot < nsteps) compute_step(d, l, slot * 16);
+  };
+  StepData buf0, buf1, buf2, buf3;
+  auto rotate = [&](int l, int r0, int r1) __attribute__((always_inline)) {
+    for (int r = r0; r < r1; ++r) {
+      score(buf0, l, r * 4 + 0);
+      fetch(buf0);
+      score(buf1, l, r * 4 + 1);
+      fetch(buf1);
+      score(buf2, l, r * 4 + 2);
+      fetch(buf2);
+      score(buf3, l, r * 4 + 3);
+      fetch(buf3);
+    }
+  };
+  auto settle = [&]() __attribute__((always_inline)) { __builtin_amdgcn_s_waitcnt(0x0F70); };
+
+  load_coefs(0);
+  fetch(buf0);
+  fetch(buf1);
+  fetch(buf2);
+  fetch(buf3);
+  for (int l = 0; l < a.L; ++l) {
+    settle();
+    rotate(l, 0, rot_before_consume);
+    if (l > 0) consume(l - 1);
+    rotate(l, rot_before_consume, rotations);
+    if (a.normalize) arrive(l);
+    if (l + 1 < a.L) load_coefs(l + 1);
+  }
+  consume(a.L - 1);
+
+  float* out = a.fin + ((int64_t)b * a.Hkv + head) * a.Tmax + n0;
+#pragma unroll
+  for (int k = 0; k < TW / 64; ++k) {
+    const int tl = lane + 64 * k;
+    if (tl < ntok) out[tl] = (a.layer_reduce == TRI_REDUCE_MEAN) ? __fdiv_rn(fin[k], (float)a.L) : fin[k];
+  }
+}
+
+template <int TW, int SL>
+size_t mfma_lds_bytes(int tile_tokens, int bs_shift, bool paged) {
+  const int blocks = paged ? (tile_tokens >> bs_shift) + 2 : 0;
+  return ((size_t)kFusedWaves * (TW + SL) * 4 + kFusedWaves * 128 + 128 + 8 + blocks) * 4;
+}
+
+template <int DT, bool IL, int TW, int SL>
+hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int B, hipStream_t s) {
+  const size_t lds = mfma_lds_bytes<TW, SL>(k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
+  if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  for (int base = 0; base < B; base += seqs_per_launch) {
+    k.seq_base = base;
+    const int n = min(seqs_per_launch, B - base);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads),
+                       lds, s, k, bmat);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+template <int DT, bool IL>
+hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int B, hipStream_t s) {
+  switch (tw) {
+    case 1024: return launch_mfma_t<DT, IL, 1024, 64>(k, bmat, seqs_per_launch, B, s);
+    case 512: return launch_mfma_t<DT, IL, 512, 64>(k, bmat, seqs_per_launch, B, s);
+    case 256: return launch_mfma_t<DT, IL, 256, 64>(k, bmat, seqs_per_launch, B, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
+                          int resident) {
+  FusedPlan p{};
+  if (resident <= 0 || D != 128 || G < 1 || G > 4 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
+    return p;
+  int bs_shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == block_size) bs_shift = sft;
+  if (paged && bs_shift < 0) return p;
+  const int HC = ceil_div(Hkv, 8);
+  const int tws[3] = {256, 512, 1024};
+  int tw = 1024;
+  for (int i = 0; i < 3; ++i)
+    if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
+  const int tiles = ceil_div(Tmax, tw);
+  if ((int64_t)tiles * HC > resident) return p;
+  p.eligible = 2;
+  p.tw = tw;
+  p.HC = HC;
+  p.tile_tokens = tw;
+  p.tiles_per_seq = tiles;
+  p.seqs_per_launch = resident / (tiles * HC);
+  p.bs_shift = bs_shift;
+  return p;
+}
+
+hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
+  FusedArgs k{};
+  k.k_layers = a.k_layers;
+  k.k_scale_layers = a.k_scale_layers;
+  k.block_table = a.block_table;
+  k.seq_lens = a.seq_lens;
+  k.prefill_lens = a.prefill_lens;
+  k.coef = a.coef;
+  k.xchg = a.xchg;
+  k.fin = a.fin;
+  k.status = a.status;
+  k.stride_block = a.stride_block; k.stride_token = a.stride_token; k.stride_head = a.stride_head;
+  k.L = a.L; k.Hkv = a.Hkv; k.A = a.A; k.G = a.G; k.HC = a.plan.HC;
+  k.block_size = a.block_size; k.bs_shift = a.plan.bs_shift;
+  k.block_table_pitch = a.block_table ? a.block_table_pitch : -1;
+  k.tiles_per_seq = a.plan.tiles_per_seq; k.tile_tokens = a.plan.tile_tokens;
+  k.seq_base = 0; k.num_seqs = a.B; k.Tmax = a.Tmax;
+  k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
+  k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
+  k.spin_ticks = 200000000LL;   // 2 s of the 100 MHz wall clock
+  const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
+  hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div64(words, 256)), dim3(256), 0, s, a.xchg, words,
+                     a.status);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
+  const int64_t heads_total = (int64_t)a.B * a.L * a.Hkv;
+  uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
+  const unsigned cgrid = (unsigned)ceil_div64(heads_total * 6 * 64, 256);
+  if (il)
+    hipLaunchKernelGGL(coef_mfma_kernel<true>, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
+  else
+    hipLaunchKernelGGL(coef_mfma_kernel<false>, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (a.kv_dtype != TRI_KV_BF16) return hipErrorInvalidValue;
+  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
+            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
+}
+
+}  // namespace tri

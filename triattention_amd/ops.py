@@ -346,13 +346,14 @@ def select_paged(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConf
 
 
 def select_path(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig) -> str:
-    """'resident' when select_paged / compress_step run the single resident kernel for
-    these arguments on the current device, else 'two_pass'."""
+    """'resident_mfma' / 'resident_valu' when select_paged / compress_step run the single
+    resident kernel (scoring on the matrix cores / on the vector unit) for these arguments
+    on the current device, else 'two_pass'."""
     sp, ss = sc.struct(), sel.struct()
     rc = int(_lib.load().tri_select_path(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss)))
     if rc < 0:
         raise ValueError("invalid arguments: " + _lib.load().tri_last_error().decode("utf-8", "replace"))
-    return "resident" if rc == 1 else "two_pass"
+    return {2: "resident_mfma", 1: "resident_valu"}.get(rc, "two_pass")
 
 
 def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] | None = None) -> torch.Tensor:
