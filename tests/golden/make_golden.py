@@ -106,79 +106,83 @@ def main() -> int:
     torch.save(out, HERE / "scoring_pytorch.pt")
 
     # ------------------------------------------------------ selector (paged)
-    layers, hq, hkv, d, t, bs = 3, 8, 2, 64, 300, 16
-    f = d // 2
-    omega = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
-    qc, qa = synth_stats(21, layers, hq, f)
-    keys, vals = synth_keys(22, layers, hkv, t, d, omega)
-    nblk_req = (t + bs - 1) // bs
-    pool = nblk_req + 5
-    g = torch.Generator().manual_seed(23)
-    block_ids = torch.randperm(pool, generator=g)[:nblk_req].tolist()
-    kv_caches = []
-    for l in range(layers):
-        kv = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
-        for n in range(t):
-            kv[0, block_ids[n // bs], n % bs] = keys[l, :, n]
-            kv[1, block_ids[n // bs], n % bs] = vals[l, :, n]
-        kv_caches.append(kv)
+    def selector_case(out_name, layers, hq, hkv, d, t, bs, seed):
+        f = d // 2
+        omega = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        qc, qa = synth_stats(seed, layers, hq, f)
+        keys, vals = synth_keys(seed + 1, layers, hkv, t, d, omega)
+        nblk_req = (t + bs - 1) // bs
+        pool = nblk_req + 5
+        g = torch.Generator().manual_seed(seed + 2)
+        block_ids = torch.randperm(pool, generator=g)[:nblk_req].tolist()
+        kv_caches = []
+        for l in range(layers):
+            kv = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
+            for n in range(t):
+                kv[0, block_ids[n // bs], n % bs] = keys[l, :, n]
+                kv[1, block_ids[n // bs], n % bs] = vals[l, :, n]
+            kv_caches.append(kv)
 
-    # The selector calls compute_scores_triton; bind it to the PyTorch scorer.
-    def _torch_scorer(key_states, cache_positions, head_stats, omega, offsets, freq_scale_sq,
-                      config, round_start=None, trig_cache=None):
-        return ref_scoring.compute_scores_pytorch(
-            key_states=key_states.float(), cache_positions=cache_positions, head_stats=head_stats,
-            omega=omega, offsets=offsets, freq_scale_sq=freq_scale_sq, config=config,
-            round_start=round_start)
-    ref_scoring.compute_scores_triton = _torch_scorer
-    # The selector builds its TriAttentionConfig with the default device ("cuda");
-    # there is no GPU here, so pin the device argument to CPU.
-    import functools
-    from triattention.vllm.core import config as ref_core_config
-    ref_core_config.TriAttentionConfig = functools.partial(TriAttentionConfig, device=cpu)
+        # The selector calls compute_scores_triton; bind it to the PyTorch scorer.
+        def _torch_scorer(key_states, cache_positions, head_stats, omega, offsets, freq_scale_sq,
+                          config, round_start=None, trig_cache=None):
+            return ref_scoring.compute_scores_pytorch(
+                key_states=key_states.float(), cache_positions=cache_positions, head_stats=head_stats,
+                omega=omega, offsets=offsets, freq_scale_sq=freq_scale_sq, config=config,
+                round_start=round_start)
+        ref_scoring.compute_scores_triton = _torch_scorer
+        # The selector builds its TriAttentionConfig with the default device ("cuda");
+        # there is no GPU here, so pin the device argument to CPU.
+        import functools
+        from triattention.vllm.core import config as ref_core_config
+        ref_core_config.TriAttentionConfig = functools.partial(TriAttentionConfig, device=cpu)
 
-    sel_out = {"keys": keys, "values": vals, "q_mean_complex": qc, "q_abs_mean": qa, "omega": omega,
-               "block_ids": torch.tensor(block_ids), "block_size": torch.tensor(bs),
-               "pool_blocks": torch.tensor(pool)}
-    with tempfile.TemporaryDirectory() as tmp:
-        sp = Path(tmp) / "stats.pt"
-        write_stats_file(sp, qc, qa, omega, d)
-        meta, head_stats = load_frequency_stats(sp, device=cpu, dtype=torch.float32, num_kv_heads=None)
-        sel_out["loader_q_mean_complex"] = torch.stack([head_stats[l]["q_mean_complex"] for l in range(layers)])
-        sel_out["loader_q_abs_mean"] = torch.stack([head_stats[l]["q_abs_mean"] for l in range(layers)])
-        sel_out["loader_freq_scale_sq"] = torch.stack([head_stats[l]["freq_scale_sq"] for l in range(layers)])
-        meta8, hs8 = load_frequency_stats(sp, device=cpu, dtype=torch.float32, num_kv_heads=hkv)
-        sel_out["loader_pooled_q_mean_complex"] = torch.stack([hs8[l]["q_mean_complex"] for l in range(layers)])
-        sel_out["loader_pooled_q_abs_mean"] = torch.stack([hs8[l]["q_abs_mean"] for l in range(layers)])
+        sel_out = {"keys": keys, "values": vals, "q_mean_complex": qc, "q_abs_mean": qa, "omega": omega,
+                   "block_ids": torch.tensor(block_ids), "block_size": torch.tensor(bs),
+                   "pool_blocks": torch.tensor(pool)}
+        with tempfile.TemporaryDirectory() as tmp:
+            sp = Path(tmp) / "stats.pt"
+            write_stats_file(sp, qc, qa, omega, d)
+            meta, head_stats = load_frequency_stats(sp, device=cpu, dtype=torch.float32, num_kv_heads=None)
+            sel_out["loader_q_mean_complex"] = torch.stack([head_stats[l]["q_mean_complex"] for l in range(layers)])
+            sel_out["loader_q_abs_mean"] = torch.stack([head_stats[l]["q_abs_mean"] for l in range(layers)])
+            sel_out["loader_freq_scale_sq"] = torch.stack([head_stats[l]["freq_scale_sq"] for l in range(layers)])
+            meta8, hs8 = load_frequency_stats(sp, device=cpu, dtype=torch.float32, num_kv_heads=hkv)
+            sel_out["loader_pooled_q_mean_complex"] = torch.stack([hs8[l]["q_mean_complex"] for l in range(layers)])
+            sel_out["loader_pooled_q_abs_mean"] = torch.stack([hs8[l]["q_abs_mean"] for l in range(layers)])
 
-        for tag, kw in {
-            "default": dict(),
-            "chunk64_prefill": dict(score_chunk_max_tokens=64, protect_prefill=True),
-            "nonorm": dict(sparse_normalize_scores=False),
-            "aggmax": dict(sparse_score_aggregation="max"),
-        }.items():
-            rc = TriAttentionRuntimeConfig(kv_budget=96, divide_length=16, window_size=12,
-                                           sparse_stats_path=sp, **kw)
-            os.environ.pop("TRIATTN_RUNTIME_DEBUG_GROUP_PERHEAD_AGG_MODE", None)
-            sel_layer, sel_group, status = ref_sel.build_triattention_selector(rc, base_runner=None)
-            assert status == "enabled"
-            prefill = 20
-            res = sel_group(layer_inputs=None, layer_input_iter=None,
-                            layer_kv_iter=lambda: [(l, kv_caches[l], block_ids, bs) for l in range(layers)],
-                            total_tokens=t, prefill_len=prefill, protect_prefill=rc.protect_prefill,
-                            round_start=t + 3, budget_total=96)
-            sel_out[f"group_{tag}_keep"] = res["indices"].clone()
-            res_l = sel_layer(keys_dense=None, kv_cache=kv_caches[1], block_ids=torch.tensor(block_ids),
-                              block_size=bs, total_tokens=t, prefill_len=prefill,
-                              protect_prefill=rc.protect_prefill, layer_idx=1, round_start=t + 3,
-                              budget_total=96)
-            assert res_l["mode"] == "per_head"
-            sel_out[f"layer1_{tag}_keep"] = res_l["indices"].clone()
-        sel_out["prefill_len"] = torch.tensor(20)
-        sel_out["round_start"] = torch.tensor(t + 3)
-        sel_out["budget"] = torch.tensor(96)
-        sel_out["window"] = torch.tensor(12)
-    torch.save(sel_out, HERE / "selector_group.pt")
+            for tag, kw in {
+                "default": dict(),
+                "chunk64_prefill": dict(score_chunk_max_tokens=64, protect_prefill=True),
+                "nonorm": dict(sparse_normalize_scores=False),
+                "aggmax": dict(sparse_score_aggregation="max"),
+            }.items():
+                rc = TriAttentionRuntimeConfig(kv_budget=96, divide_length=16, window_size=12,
+                                               sparse_stats_path=sp, **kw)
+                os.environ.pop("TRIATTN_RUNTIME_DEBUG_GROUP_PERHEAD_AGG_MODE", None)
+                sel_layer, sel_group, status = ref_sel.build_triattention_selector(rc, base_runner=None)
+                assert status == "enabled"
+                prefill = 20
+                res = sel_group(layer_inputs=None, layer_input_iter=None,
+                                layer_kv_iter=lambda: [(l, kv_caches[l], block_ids, bs) for l in range(layers)],
+                                total_tokens=t, prefill_len=prefill, protect_prefill=rc.protect_prefill,
+                                round_start=t + 3, budget_total=96)
+                sel_out[f"group_{tag}_keep"] = res["indices"].clone()
+                res_l = sel_layer(keys_dense=None, kv_cache=kv_caches[1], block_ids=torch.tensor(block_ids),
+                                  block_size=bs, total_tokens=t, prefill_len=prefill,
+                                  protect_prefill=rc.protect_prefill, layer_idx=1, round_start=t + 3,
+                                  budget_total=96)
+                assert res_l["mode"] == "per_head"
+                sel_out[f"layer1_{tag}_keep"] = res_l["indices"].clone()
+            sel_out["prefill_len"] = torch.tensor(20)
+            sel_out["round_start"] = torch.tensor(t + 3)
+            sel_out["budget"] = torch.tensor(96)
+            sel_out["window"] = torch.tensor(12)
+        torch.save(sel_out, HERE / out_name)
+
+    selector_case("selector_group.pt", 3, 8, 2, 64, 300, 16, 21)
+    # head_dim 128: the shape the resident kernels of the HIP path take
+    selector_case("selector_group_d128.pt", 3, 8, 2, 128, 700, 16, 41)
 
     # ------------------------------------------------------------ compaction
     comp = {}

@@ -177,9 +177,14 @@ def test_group_selection_matches_oracle(name):
     ("nonorm", dict(normalize=False)),
     ("aggmax", dict(aggregation="max")),
 ])
-def test_group_selection_matches_reference_golden(tag, kw):
-    """Keep sets written by the reference's own selector (paged group branch)."""
-    gold = load_golden("selector_group.pt")
+@pytest.mark.parametrize("path", ["two_pass", "resident_mfma", "resident_valu"])
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
+def test_group_selection_matches_reference_golden(tag, kw, path, fixture, monkeypatch):
+    """Keep sets written by the reference's own selector (paged group branch), through the
+    two-pass path and through both resident kernels."""
+    if path == "resident_valu":
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+    gold = load_golden(fixture)
     layers, hkv, t, d = gold["keys"].shape
     hq = gold["q_mean_complex"].shape[1]
     bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])
@@ -202,8 +207,14 @@ def test_group_selection_matches_reference_golden(tag, kw):
                          kw.get("aggregation", "mean"))
     sel = ops.SelectConfig(normalize=kw.get("normalize", True), window_size=int(gold["window"]),
                            protect_prefill=kw.get("protect_prefill", False))
-    raw, ws = ops.score_paged(kv, batch, sc)
-    keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+    if path == "two_pass":
+        raw, ws = ops.score_paged(kv, batch, sc)
+        keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+    else:
+        if ops.select_path(kv, batch, sc, sel) != path:
+            pytest.skip(f"this setting runs {ops.select_path(kv, batch, sc, sel)}")
+        keep, _, ws = ops.select_paged(kv, batch, sc, sel)
+        assert ws.status() == 0
     torch.cuda.synchronize()
     want = gold[f"group_{tag}_keep"]
     got = keep.cpu().long()
@@ -212,10 +223,11 @@ def test_group_selection_matches_reference_golden(tag, kw):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
 @pytest.mark.parametrize("tag,kw", [("default", dict()), ("nonorm", dict(normalize=False))])
-def test_layer_selection_matches_reference_golden(tag, kw):
+def test_layer_selection_matches_reference_golden(tag, kw, fixture):
     """Per-layer selection (runtime/selector_hf.py:473-677) against the reference's output for layer 1."""
-    gold = load_golden("selector_group.pt")
+    gold = load_golden(fixture)
     layers, hkv, t, d = gold["keys"].shape
     hq = gold["q_mean_complex"].shape[1]
     bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])

@@ -52,8 +52,9 @@ def _golden_caches(gold):
 @pytest.mark.parametrize("tag,kw", [("default", {}), ("nonorm", {"sparse_normalize_scores": False}),
                                     ("aggmax", {"sparse_score_aggregation": "max"}),
                                     ("chunk64_prefill", {"score_chunk_max_tokens": 64, "protect_prefill": True})])
-def test_selector_api_matches_reference_outputs(tmp_path, tag, kw):
-    gold = load_golden("selector_group.pt")
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
+def test_selector_api_matches_reference_outputs(tmp_path, tag, kw, fixture):
+    gold = load_golden(fixture)
     layers, hkv, t, d = gold["keys"].shape
     _write_stats(tmp_path / "s.pt", gold["q_mean_complex"], gold["q_abs_mean"], gold["omega"], d)
     cfg = TriAttentionRuntimeConfig(kv_budget=96, divide_length=16, window_size=12, sparse_stats_path=tmp_path / "s.pt", **kw)

@@ -43,9 +43,10 @@ def _sets_equal_off_ties(keep, want, fin, k):
             assert fin[h, idx] == thr, (h, idx, float(fin[h, idx]), float(thr))
 
 
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
 @pytest.mark.parametrize("tag", list(CASES))
-def test_group_selection_matches_reference(tag):
-    gold = load_golden("selector_group.pt")
+def test_group_selection_matches_reference(tag, fixture):
+    gold = load_golden(fixture)
     raw, hkv = _golden_raw(gold, "max" if tag == "aggmax" else "mean")
     kw = dict(window_size=int(gold["window"]), prefill_len=int(gold["prefill_len"]))
     kw.update(CASES[tag])
@@ -57,9 +58,10 @@ def test_group_selection_matches_reference(tag):
     assert torch.equal(keep, want)          # no ties at the threshold in this fixture
 
 
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
 @pytest.mark.parametrize("tag", list(CASES))
-def test_layer_selection_matches_reference(tag):
-    gold = load_golden("selector_group.pt")
+def test_layer_selection_matches_reference(tag, fixture):
+    gold = load_golden(fixture)
     raw, hkv = _golden_raw(gold, "max" if tag == "aggmax" else "mean")
     kw = dict(window_size=int(gold["window"]), prefill_len=int(gold["prefill_len"]))
     kw.update(CASES[tag])

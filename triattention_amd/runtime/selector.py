@@ -4,7 +4,8 @@ keyword signatures, result dictionaries and failure markers, executed by the HIP
 the combine kernel and the radix top-k.
 
 Nothing is chunked and K is neither gathered nor repeated per query head: the scorer
-reads the paged blocks of every layer once.  Ties at the budget keep the lowest token
+reads the paged blocks of every layer once and, for shapes that have a resident kernel,
+keeps the raw scores on chip (``ops.select_paged``).  Ties at the budget keep the lowest token
 index (the reference's ``torch.topk`` leaves them undefined).
 """
 from __future__ import annotations
@@ -150,14 +151,13 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
             block_ids.flatten().tolist() if isinstance(block_ids, torch.Tensor) else [int(x) for x in block_ids]]
         batch = ops.StepBatch(kv.device, [total_tokens], round_start=[round_start], budgets=[k],
                               block_tables=tables, prefill_lens=[prefill_len])
-        try:
-            raw, ws = ops.score_paged(kv, batch, sc)
-        except Exception as exc:
-            raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
         sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
                                protect_prefill=bool(protect_prefill and prefill_len > 0),
                                group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared)
-        keep, _ = ops.select(kv, batch, sc, sel, raw, ws)
+        try:
+            keep, _, _ = ops.select_paged(kv, batch, sc, sel)
+        except Exception as exc:
+            raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
         return keep.to(torch.long)
 
     def _select_keep_indices(*, keys_dense: torch.Tensor | None = None, kv_cache: torch.Tensor | None = None,
