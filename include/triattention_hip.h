@@ -158,7 +158,7 @@ int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_
                      uint64_t workspace_bytes, void* stream);
 
 /* Which path tri_select_paged / tri_compress_step take for these arguments on the
- * current device: 2 = resident kernel scoring on the matrix cores (bf16 keys), 1 = resident
+ * current device: 2 = resident kernel scoring on the matrix cores (bf16 and fp8 keys), 1 = resident
  * kernel scoring on the vector unit, 0 = score then select, -1 = invalid arguments.
  * Host-only.  No counterpart in the reference (it has a single path). */
 int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,

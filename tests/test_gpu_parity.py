@@ -399,6 +399,8 @@ RESIDENT_CASES = {
     "interleaved": dict(w=small(rope_style="interleaved")),
     "fp16": dict(w=small(kv_dtype="fp16")),
     "fp8": dict(w=small(kv_dtype="fp8", seq_lens=(300, 45))),
+    "fp8_interleaved_hkv8": dict(w=small(kv_dtype="fp8", rope_style="interleaved", num_q_heads=32, num_kv_heads=8,
+                                         seq_lens=(530, 64))),
     "block4": dict(w=small(block_size=4, seq_lens=(301,))),
     "block64": dict(w=small(block_size=64, seq_lens=(500, 31))),
     "kv_axis1": dict(w=small(seq_lens=(290, 64)), kv_axis=1),
@@ -421,8 +423,8 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     rounding by mean^2/var), same kept sets away from ties."""
     case = dict(RESIDENT_CASES[name])
     w = case["w"]
-    if kernel == "mfma" and w.kv_dtype != "bf16":
-        pytest.skip("the matrix-core kernel takes bf16 keys; other types run the vector-unit kernel")
+    if kernel == "mfma" and w.kv_dtype == "fp16":
+        pytest.skip("the matrix-core kernel takes bf16 and fp8 keys; fp16 runs the vector-unit kernel")
     if kernel == "valu":
         monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
     inp = build_inputs(w, case.get("kv_axis", 0))

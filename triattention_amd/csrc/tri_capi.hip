@@ -84,10 +84,11 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
 }
 
 tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
-  // bf16 keys go to the matrix-core kernel, other types to the vector-unit one;
+  // bf16 and fp8 keys go to the matrix-core kernel, fp16 to the vector-unit one;
   // TRIATTN_RESIDENT_KERNEL=valu forces the vector-unit kernel (for comparison runs).
   const char* force = getenv("TRIATTN_RESIDENT_KERNEL");
-  const bool want_mfma = kv->kv_dtype == TRI_KV_BF16 && !(force && strcmp(force, "valu") == 0);
+  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) &&
+                         !(force && strcmp(force, "valu") == 0);
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;
   const int resident = tri::fused_resident_workgroups();

@@ -18,6 +18,8 @@
 //
 // Per 16 tokens of a head: 8 MFMAs, and vector work only for the magnitudes (about 40 %
 // of the vector-unit kernel's instruction count), so the kernel is bound by the key stream.
+// fp8 e4m3 keys are widened to bf16 (exact) in registers and take the same route; the
+// per-(token, head) scale multiplies the finished score.
 #include "tri_common.h"
 #include "tri_score_device.h"
 #include "tri_fused_device.h"
@@ -33,11 +35,30 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 constexpr int kDppRor4 = 0x124;   // row_ror:4
 constexpr int kDppRor8m = 0x128;  // row_ror:8
 
-// Four 16-byte chunks of one (token, head) row per lane: chunk 4*s + kb for s = 0..3, where
-// kb = lane / 16 and the token is lane % 16 of the step.
+// What a lane loads of one (token, head) row per step; the token is lane % 16 of the step,
+// kb = lane / 16.  Two-byte keys: the 16-byte chunks 4*s + kb, s = 0..3 (8 elements each,
+// MFMA s takes chunk s).  fp8 keys: the 16-byte chunks kb and 4 + kb (16 elements each;
+// MFMA s takes half s % 2 of chunk s / 2) and the dequantisation scale of the token this
+// lane will store.
+template <int DT>
 struct StepData {
-  uint4 c[4];
+  uint4 c[DT == TRI_KV_FP8_E4M3 ? 2 : 4];
+  float scale;
 };
+
+// Index, inside the 128 elements of a head row, of element e of lane block kb in MFMA s.
+template <int DT>
+__host__ __device__ constexpr int slab_elem(int s, int kb, int e) {
+  return DT == TRI_KV_FP8_E4M3 ? (kb + 4 * (s >> 1)) * 16 + (s & 1) * 8 + e : (4 * s + kb) * 8 + e;
+}
+
+// Four fp8 e4m3 bytes -> four bf16 (exact: e4m3 has 3 mantissa bits).
+__device__ __forceinline__ void fp8x4_to_bf16x4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+  const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+  const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, bf16x2));
+  hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, bf16x2));
+}
 
 __device__ __forceinline__ bf16x8 as_bf16x8(const uint4& v) { return __builtin_bit_cast(bf16x8, v); }
 
@@ -54,10 +75,10 @@ __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, fl
 }
 
 // Coefficient slabs of one (sequence, layer, head) in MFMA B-operand order:
-// bmat[((b*L + l)*Hkv + head)*6 + o][lane][8] bf16.  Operand o: 0..3 the key chunks
-// 4*o + kb, 4 and 5 the magnitudes of pair sets 0 and 1.  Lane (j = lane % 16, kb):
+// bmat[((b*L + l)*Hkv + head)*6 + o][lane][8] bf16.  Operand o: 0..3 the key slabs of
+// MFMA o, 4 and 5 the magnitudes of pair sets 0 and 1.  Lane (j = lane % 16, kb):
 // column j = (query head j % 4, split j / 4); element e = k index kb*8 + e of the slab.
-template <bool IL>
+template <int DT, bool IL>
 __global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int64_t n_heads_total, uint4* bmat) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (head instance, operand, lane)
   if (idx >= n_heads_total * 6 * 64) return;
@@ -76,14 +97,15 @@ __global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int64
     for (int e = 0; e < 8; ++e) {
       int which, pair;   // which: 0 = P, 1 = R, 2 = E
       if (o < 4) {
-        const int chunk = 4 * o + kb;
-        if (IL) { which = e & 1; pair = chunk * 4 + (e >> 1); }
-        else { which = chunk >= 8 ? 1 : 0; pair = (chunk & 7) * 8 + e; }
+        const int el = slab_elem<DT>(o, kb, e);
+        if (IL) { which = el & 1; pair = el >> 1; }
+        else { which = el >= 64 ? 1 : 0; pair = el & 63; }
       } else {
         which = 2;
         const int set = o - 4;
-        if (IL) pair = (4 * (2 * set + (e >> 2)) + kb) * 4 + (e & 3);   // chunks of steps 2*set, 2*set+1
-        else pair = (4 * set + kb) * 8 + e;                               // real chunk 4*set + kb
+        // interleaved: pairs of MFMAs 2*set and 2*set + 1; half: real parts of MFMA `set`
+        if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
+        else pair = slab_elem<DT>(set, kb, e) & 63;
       }
       float x = c[which * 64 + pair];
       // piece sp of x = x1 + x2 + x3 (each bf16, round to nearest even)
@@ -152,11 +174,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   };
 
   // Element offset of this lane inside a (token, head) row and of its head inside a token.
-  const int64_t lane_elems = (int64_t)head * a.stride_head + kb * 8;
+  const int64_t lane_elems = (int64_t)head * a.stride_head + kb * (DT == TRI_KV_FP8_E4M3 ? 16 : 8);
 
   // Sixteen tokens of layer l starting at local token t (t % 16 == 0): lane's token is
   // t + lane % 16, clamped to the tile's last token (loaded, never stored).
-  auto load_step = [&](StepData& d, int l, int t) __attribute__((always_inline)) {
+  constexpr bool FP8 = DT == TRI_KV_FP8_E4M3;
+  constexpr int ES = FP8 ? 1 : 2;
+  auto load_step = [&](StepData<DT>& d, int l, int t) __attribute__((always_inline)) {
     const char* kbase = table_entry(a.k_layers, l);
     const int n = min(n0 + t + j, last_tok);
     int64_t row;
@@ -166,18 +190,53 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       const int lb = n >> a.bs_shift;
       row = (int64_t)lds_blk[lb - lb0] * a.stride_block + (int64_t)(n - (lb << a.bs_shift)) * a.stride_token;
     }
-    GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + (row + lane_elems) * 2;
+    GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + (row + lane_elems) * ES;
+    d.scale = 1.f;
+    if constexpr (FP8) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const u32x4 v = *(GlobalU4)(p + s * 64);
-      d.c[s] = uint4{v.x, v.y, v.z, v.w};
+      for (int s = 0; s < 2; ++s) {
+        const u32x4 v = *(GlobalU4)(p + s * 64);
+        d.c[s] = uint4{v.x, v.y, v.z, v.w};
+      }
+      // scale of the token this lane stores: local token t + 4*kb + rsel
+      const int ns = min(n0 + t + 4 * kb + rsel, last_tok);
+      int64_t slot;
+      if (a.block_table_pitch < 0) {
+        slot = (int64_t)b * a.block_size + ns;
+      } else {
+        const int lb = ns >> a.bs_shift;
+        slot = (int64_t)lds_blk[lb - lb0] * a.block_size + (ns - (lb << a.bs_shift));
+      }
+      const float* sc = reinterpret_cast<const float*>(
+          table_entry(reinterpret_cast<const void* const*>(a.k_scale_layers), l));
+      d.scale = ((GlobalF32)(uintptr_t)sc)[slot * a.Hkv + head];
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 v = *(GlobalU4)(p + s * 64);
+        d.c[s] = uint4{v.x, v.y, v.z, v.w};
+      }
     }
   };
 
   float s1 = 0.f, s2 = 0.f;
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
-  auto compute_step = [&](const StepData& d, int l, int t) __attribute__((always_inline)) {
+  auto compute_step = [&](const StepData<DT>& raw, int l, int t) __attribute__((always_inline)) {
+    // The four bf16 A operands of the step.
+    struct { uint4 c[4]; } d;
+    if constexpr (FP8) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        fp8x4_to_bf16x4(raw.c[s].x, d.c[2 * s].x, d.c[2 * s].y);
+        fp8x4_to_bf16x4(raw.c[s].y, d.c[2 * s].z, d.c[2 * s].w);
+        fp8x4_to_bf16x4(raw.c[s].z, d.c[2 * s + 1].x, d.c[2 * s + 1].y);
+        fp8x4_to_bf16x4(raw.c[s].w, d.c[2 * s + 1].z, d.c[2 * s + 1].w);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) d.c[s] = raw.c[s];
+    }
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s)
@@ -229,6 +288,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       x += dpp<kDppRor4>(x);
       v = (rsel == r) ? x : v;
     }
+    if (FP8) v *= raw.scale;
     const int tl = t + 4 * kb + rsel;
     if (q_ok && tl < ntok) {
       ring[((uint32_t)(l * TW + tl) % RING) * 4 + q] = v;
@@ -338,16 +398,16 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   const int rotations = (nsteps + 3) >> 2;
   const int rot_before_consume = min(SL / 64, rotations);
   int ld_l = 0, ld_slot = 0;
-  auto fetch = [&](StepData& d) __attribute__((always_inline)) {
+  auto fetch = [&](StepData<DT>& d) __attribute__((always_inline)) {
     const int l = __builtin_amdgcn_readfirstlane(min(ld_l, a.L - 1));
     const int t = __builtin_amdgcn_readfirstlane(min(ld_slot, nsteps - 1) * 16);
     load_step(d, l, t);
     if (++ld_slot >= rotations * 4) { ld_slot = 0; ++ld_l; }
   };
-  auto score = [&](const StepData& d, int l, int slot) __attribute__((always_inline)) {
+  auto score = [&](const StepData<DT>& d, int l, int slot) __attribute__((always_inline)) {
     if (slot < nsteps) compute_step(d, l, slot * 16);
   };
-  StepData buf0, buf1, buf2, buf3;
+  StepData<DT> buf0, buf1, buf2, buf3;
   auto rotate = [&](int l, int r0, int r1) __attribute__((always_inline)) {
     for (int r = r0; r < r1; ++r) {
       score(buf0, l, r * 4 + 0);
@@ -476,13 +536,23 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   const int64_t heads_total = (int64_t)a.B * a.L * a.Hkv;
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
   const unsigned cgrid = (unsigned)ceil_div64(heads_total * 6 * 64, 256);
-  if (il)
-    hipLaunchKernelGGL(coef_mfma_kernel<true>, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
-  else
-    hipLaunchKernelGGL(coef_mfma_kernel<false>, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
+  const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
+  if (a.kv_dtype != TRI_KV_BF16 && !fp8) return hipErrorInvalidValue;
+  auto coef_launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
+  };
+  if (fp8) {
+    if (il) coef_launch(coef_mfma_kernel<TRI_KV_FP8_E4M3, true>);
+    else coef_launch(coef_mfma_kernel<TRI_KV_FP8_E4M3, false>);
+  } else {
+    if (il) coef_launch(coef_mfma_kernel<TRI_KV_BF16, true>);
+    else coef_launch(coef_mfma_kernel<TRI_KV_BF16, false>);
+  }
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  if (a.kv_dtype != TRI_KV_BF16) return hipErrorInvalidValue;
+  if (fp8)
+    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
   return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
             : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
 }
