@@ -154,21 +154,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
         }
         buf[r].scale = buffer_load_f32(srsrc, (uint32_t)head_c * 4u, dt * scale_tok_bytes);
       } else {
-#ifdef TRI_EXP_NOLOAD
-        buf[r].lo = uint4{soff + lane, 0x3f803f80u, lane_off_bytes, 0x40004000u};
-        buf[r].hi = uint4{0x3f003f00u, soff, 0x3f803f80u, lane_off_bytes};
-#else
         buf[r].lo = buffer_load16(rsrc, lane_off_bytes, soff);
         buf[r].hi = buffer_load16(rsrc, lane_off_bytes + (IL ? 16 : LPH * 16), soff);
-#endif
       }
     }
   };
 
   auto score_row = [&](const RowData& d) __attribute__((always_inline)) -> float {
-#ifdef TRI_EXP_NOCOMPUTE
-    return __uint_as_float((d.lo.x ^ d.lo.y ^ d.lo.z ^ d.lo.w ^ d.hi.x ^ d.hi.y ^ d.hi.z ^ d.hi.w) & 0x3fffffffu) * P[0][0];
-#endif
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
