@@ -396,6 +396,9 @@ RESIDENT_CASES = {
     "hkv16": dict(w=small(num_q_heads=32, num_kv_heads=16, seq_lens=(450,))),
     "hkv32_g1": dict(w=small(num_q_heads=32, num_kv_heads=32, seq_lens=(200, 77))),
     "g1": dict(w=small(num_q_heads=2, num_kv_heads=2, seq_lens=(129,))),
+    "g8": dict(w=small(num_q_heads=64, num_kv_heads=8, seq_lens=(700, 90), num_layers=3)),
+    "g6_hkv3": dict(w=small(num_q_heads=18, num_kv_heads=3, seq_lens=(333, 130))),
+    "g8_fp8_long": dict(w=small(kv_dtype="fp8", num_q_heads=16, num_kv_heads=2, seq_lens=(9000, 2500), budget=512)),
     "interleaved": dict(w=small(rope_style="interleaved")),
     "fp16": dict(w=small(kv_dtype="fp16")),
     "fp8": dict(w=small(kv_dtype="fp8", seq_lens=(300, 45))),
@@ -425,6 +428,8 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     w = case["w"]
     if kernel == "mfma" and w.kv_dtype == "fp16":
         pytest.skip("the matrix-core kernel takes bf16 and fp8 keys; fp16 runs the vector-unit kernel")
+    if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
+        pytest.skip("the vector-unit kernel holds four query heads per KV head")
     if kernel == "valu":
         monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
     inp = build_inputs(w, case.get("kv_axis", 0))
@@ -452,7 +457,7 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
 
 
 def test_resident_path_falls_back_when_shape_has_no_kernel():
-    for kw, selkw in ((dict(num_q_heads=64, num_kv_heads=8), {}), (dict(head_dim=64), {}),
+    for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=64), {}),
                       (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
         w = small(**kw)
         inp = build_inputs(w)

@@ -49,7 +49,7 @@ struct Workspace {
   int64_t fin;       // [B*L*Hkv][Tmax] fp32 selection scores (worst case: per-layer selection)
   int64_t xchg;      // [B][L][tiles_per_seq][A][2] tagged sums exchanged by the resident kernel
   int64_t status;    // one word: non-zero when a bounded wait of the resident kernel expired
-  int64_t bmat;      // [B][L][Hkv][6][64][8] bf16 coefficient slabs of the matrix-core kernel
+  int64_t bmat;      // [B][L][Hkv][groups of 4 query heads][6][64][8] bf16 coefficient slabs (matrix-core kernel)
   int64_t total;
   int32_t num_tiles; // NT
   FusedPlan fused;
@@ -69,7 +69,7 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
   w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
   w.status = take(256);
-  w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * 6 * 64 * 16 : 0);
+  w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * (A / Hkv > 4 ? 2 : 1) * 6 * 64 * 16 : 0);
   w.total = off;
   return w;
 }

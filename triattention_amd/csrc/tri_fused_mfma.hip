@@ -75,20 +75,23 @@ __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, fl
 }
 
 // Coefficient slabs of one (sequence, layer, head) in MFMA B-operand order:
-// bmat[((b*L + l)*Hkv + head)*6 + o][lane][8] bf16.  Operand o: 0..3 the key slabs of
-// MFMA o, 4 and 5 the magnitudes of pair sets 0 and 1.  Lane (j = lane % 16, kb):
-// column j = (query head j % 4, split j / 4); element e = k index kb*8 + e of the slab.
+// bmat[(((b*L + l)*Hkv + head)*QG + g)*6 + o][lane][8] bf16.  Group g holds query heads
+// 4g..4g+3 of the KV head.  Operand o: 0..3 the key slabs of MFMA o, 4 and 5 the magnitudes
+// of pair sets 0 and 1.  Lane (j = lane % 16, kb): column j = (query head 4g + j % 4, split
+// j / 4); element e = k index kb*8 + e of the slab.
 template <int DT, bool IL>
-__global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int64_t n_heads_total, uint4* bmat) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (head instance, operand, lane)
-  if (idx >= n_heads_total * 6 * 64) return;
+__global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int QG, int64_t n_heads_total,
+                                 uint4* bmat) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (head instance, group, operand, lane)
+  if (idx >= n_heads_total * QG * 6 * 64) return;
   const int lane = (int)(idx % 64);
   const int o = (int)((idx / 64) % 6);
-  const int64_t hi = idx / (64 * 6);                 // (b*L + l)*Hkv + head
+  const int g = (int)((idx / (64 * 6)) % QG);
+  const int64_t hi = idx / (64 * 6 * QG);            // (b*L + l)*Hkv + head
   const int head = (int)(hi % Hkv);
   const int64_t bl = hi / Hkv;
   const int j = lane & 15, kb = lane >> 4;
-  const int q = j & 3, sp = j >> 2;
+  const int q = 4 * g + (j & 3), sp = j >> 2;
   uint32_t out[4] = {0, 0, 0, 0};
   if (q < G && sp < 3) {
     const float* c = coef + ((bl * A + (int64_t)head * G + q) * 3) * 64;   // [P | R | E][64]
@@ -121,9 +124,11 @@ __global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int64
   bmat[idx] = uint4{out[0], out[1], out[2], out[3]};
 }
 
-template <int DT, bool IL, int TW, int SL>
+// QG: groups of four query heads per KV head (1 or 2).
+template <int DT, bool IL, int TW, int SL, int QG>
 __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   constexpr int RING = TW + SL;
+  constexpr int RQ = 4 * QG;                                   // ring floats per token
   extern __shared__ __align__(16) float lds[];
 
   const int lane = threadIdx.x & 63;
@@ -141,13 +146,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   const int seq_tiles = ceil_div(T, a.tile_tokens);
   const int heads_here = min(8, a.Hkv - chunk * 8);
 
-  float* ring = lds + wave * (RING * 4);                       // [RING][4 query heads]
-  float* part = lds + kFusedWaves * (RING * 4);                // [waves][64][2]
-  float* stats = part + kFusedWaves * 128;                     // [2][32 score heads][2]
-  uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128);    // arrive count, claimed, ready
+  float* ring = lds + wave * (RING * RQ);                      // [RING][query heads of the KV head]
+  float* part = lds + kFusedWaves * (RING * RQ);               // [waves][64][QG][2]
+  float* stats = part + kFusedWaves * 128 * QG;                // [2][32*QG score heads][2]
+  uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128 * QG);  // arrive count, claimed, ready
   int* lds_blk = reinterpret_cast<int*>(ctl + 8);
 
-  for (int i = threadIdx.x; i < kFusedWaves * 128; i += kFusedThreads) part[i] = 0.f;
+  for (int i = threadIdx.x; i < kFusedWaves * 128 * QG; i += kFusedThreads) part[i] = 0.f;
   if (threadIdx.x < 8) ctl[threadIdx.x] = 0;
   int lb0 = 0;
   if (a.block_table_pitch >= 0) {
@@ -163,14 +168,15 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 
   const int j = lane & 15, kb = lane >> 4;       // MFMA column / k block; also output row block
   const int q = j & 3, rsel = j >> 2;
-  const bool q_ok = q < a.G;
 
   // Coefficient slabs of the current layer.
-  uint4 B[6];
+  uint4 B[QG][6];
   auto load_coefs = [&](int l) __attribute__((always_inline)) {
-    const uint4* p = bmat + (((int64_t)(b * a.L + l) * a.Hkv + head) * 6) * 64 + lane;
+    const uint4* p = bmat + (((int64_t)(b * a.L + l) * a.Hkv + head) * QG * 6) * 64 + lane;
 #pragma unroll
-    for (int o = 0; o < 6; ++o) B[o] = p[o * 64];
+    for (int g = 0; g < QG; ++g)
+#pragma unroll
+      for (int o = 0; o < 6; ++o) B[g][o] = p[(g * 6 + o) * 64];
   };
 
   // Element offset of this lane inside a (token, head) row and of its head inside a token.
@@ -219,7 +225,9 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     }
   };
 
-  float s1 = 0.f, s2 = 0.f;
+  float s1[QG], s2[QG];
+#pragma unroll
+  for (int g = 0; g < QG; ++g) { s1[g] = 0.f; s2[g] = 0.f; }
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
   auto compute_step = [&](const StepData<DT>& raw, int l, int t) __attribute__((always_inline)) {
@@ -237,11 +245,15 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 #pragma unroll
       for (int s = 0; s < 4; ++s) d.c[s] = raw.c[s];
     }
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[QG], acc_e[QG];
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(d.c[s]), as_bf16x8(B[s]), acc, 0, 0, 0);
-    f32x4 acc_e = {0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < QG; ++g) {
+      acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+      acc_e[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(d.c[s]), as_bf16x8(B[g][s]), acc[g], 0, 0, 0);
+    }
 #pragma unroll
     for (int set = 0; set < 2; ++set) {
       float mag[8];
@@ -277,23 +289,29 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       lo.y = split_pair(r[2], r[3], unused0, unused1);
       lo.z = split_pair(r[4], r[5], unused0, unused1);
       lo.w = split_pair(r[6], r[7], unused0, unused1);
-      acc_e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(hi), as_bf16x8(B[4 + set]), acc_e, 0, 0, 0);
-      acc_e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(lo), as_bf16x8(B[4 + set]), acc_e, 0, 0, 0);
-    }
-    float v = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float x = acc[r] + acc_e[r];
-      x += dpp<kDppRor8m>(x);
-      x += dpp<kDppRor4>(x);
-      v = (rsel == r) ? x : v;
+      for (int g = 0; g < QG; ++g) {
+        acc_e[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(hi), as_bf16x8(B[g][4 + set]), acc_e[g], 0, 0, 0);
+        acc_e[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(lo), as_bf16x8(B[g][4 + set]), acc_e[g], 0, 0, 0);
+      }
     }
-    if (FP8) v *= raw.scale;
     const int tl = t + 4 * kb + rsel;
-    if (q_ok && tl < ntok) {
-      ring[((uint32_t)(l * TW + tl) % RING) * 4 + q] = v;
-      s1 += v;
-      s2 = fmaf(v, v, s2);
+#pragma unroll
+    for (int g = 0; g < QG; ++g) {
+      float v = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float x = acc[g][r] + acc_e[g][r];
+        x += dpp<kDppRor8m>(x);
+        x += dpp<kDppRor4>(x);
+        v = (rsel == r) ? x : v;
+      }
+      if (FP8) v *= raw.scale;
+      if (4 * g + q < a.G && tl < ntok) {
+        ring[((uint32_t)(l * TW + tl) % RING) * RQ + 4 * g + q] = v;
+        s1[g] += v;
+        s2[g] = fmaf(v, v, s2[g]);
+      }
     }
   };
 
@@ -309,22 +327,27 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   // before any wave deposits layer l + 1 (a wave consumes layer l, which needs every
   // deposit of layer l, before it finishes layer l + 1), so the counter never mixes layers.
   auto arrive = [&](int l) __attribute__((always_inline)) {
-    part[(wave * 64 + lane) * 2] = s1;
-    part[(wave * 64 + lane) * 2 + 1] = s2;
-    s1 = 0.f;
-    s2 = 0.f;
+#pragma unroll
+    for (int g = 0; g < QG; ++g) {
+      part[((wave * 64 + lane) * QG + g) * 2] = s1[g];
+      part[((wave * 64 + lane) * QG + g) * 2 + 1] = s2[g];
+      s1[g] = 0.f;
+      s2[g] = 0.f;
+    }
     uint32_t prev = 0;
     if (lane == 0) prev = __hip_atomic_fetch_add(arrive_cnt, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
     prev = __builtin_amdgcn_readfirstlane(prev);
     if (prev + 1 != (uint32_t)(l + 1) * (uint32_t)heads_here) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    if (lane < items) {
-      const int ahl = lane >> 1, which = lane & 1;
+    unsigned long long* out = a.xchg + (((int64_t)(b * a.L + l) * a.tiles_per_seq + tile) * a.A + ah0) * 2;
+    for (int item = lane; item < items; item += 64) {
+      const int ahl = item >> 1, which = item & 1;
       const int w = ahl / a.G, qq = ahl - w * a.G;
+      const int g = qq >> 2, q4 = qq & 3;
       float t = 0.f;
-      for (int i = 0; i < 16; ++i) t += part[(w * 64 + (i >> 2) * 16 + (i & 3) * 4 + qq) * 2 + which];
-      unsigned long long* out = a.xchg + (((int64_t)(b * a.L + l) * a.tiles_per_seq + tile) * a.A + ah0) * 2;
-      xchg_store(out + lane, ((unsigned long long)(uint32_t)(l + 1) << 32) | __float_as_uint(t));
+      for (int i = 0; i < 16; ++i)
+        t += part[((w * 64 + (i >> 2) * 16 + (i & 3) * 4 + q4) * QG + g) * 2 + which];
+      xchg_store(out + item, ((unsigned long long)(uint32_t)(l + 1) << 32) | __float_as_uint(t));
     }
   };
 
@@ -336,7 +359,9 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 
   // Turn layer l's ring entries into selection-score contributions (lane = token).
   auto consume = [&](int l) __attribute__((always_inline)) {
-    float mean[4] = {0.f, 0.f, 0.f, 0.f}, sd[4] = {1.f, 1.f, 1.f, 1.f};
+    float mean[RQ], sd[RQ];
+#pragma unroll
+    for (int qq = 0; qq < RQ; ++qq) { mean[qq] = 0.f; sd[qq] = 1.f; }
     if (a.normalize) {
       uint32_t won = 0;
       if (lane == 0) {
@@ -346,7 +371,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       }
       won = __builtin_amdgcn_readfirstlane(won);
       if (won) {
-        gather_layer_stats(a, b, l, seq_tiles, T, ah0, items, stats + (l & 1) * 64, lane, aborted);
+        gather_layer_stats(a, b, l, seq_tiles, T, ah0, items, stats + (l & 1) * 64 * QG, lane, aborted);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0) __hip_atomic_store(ready, (uint32_t)(l + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
       } else {
@@ -355,9 +380,9 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
           __builtin_amdgcn_s_sleep(2);
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-      const float* st = stats + (l & 1) * 64;
+      const float* st = stats + (l & 1) * 64 * QG;
 #pragma unroll
-      for (int qq = 0; qq < 4; ++qq)
+      for (int qq = 0; qq < RQ; ++qq)
         if (qq < a.G) {
           mean[qq] = st[(wave * a.G + qq) * 2];
           sd[qq] = st[(wave * a.G + qq) * 2 + 1];
@@ -367,18 +392,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     for (int k = 0; k < TW / 64; ++k) {
       const int tl = lane + 64 * k;
       if (tl >= ntok) continue;
-      const float4 x = *reinterpret_cast<const float4*>(&ring[((uint32_t)(l * TW + tl) % RING) * 4]);
-      const float xs[4] = {x.x, x.y, x.z, x.w};
+      float xs[RQ];
+#pragma unroll
+      for (int g = 0; g < QG; ++g) {
+        const float4 x = *reinterpret_cast<const float4*>(&ring[((uint32_t)(l * TW + tl) % RING) * RQ + 4 * g]);
+        xs[4 * g] = x.x; xs[4 * g + 1] = x.y; xs[4 * g + 2] = x.z; xs[4 * g + 3] = x.w;
+      }
       float v;
       if (a.group_reduce == TRI_REDUCE_MAX) {
         v = -INFINITY;
 #pragma unroll
-        for (int qq = 0; qq < 4; ++qq)
+        for (int qq = 0; qq < RQ; ++qq)
           if (qq < a.G) v = fmaxf(v, __fdiv_rn(__fsub_rn(xs[qq], mean[qq]), sd[qq]));
       } else {
         v = 0.f;
 #pragma unroll
-        for (int qq = 0; qq < 4; ++qq)
+        for (int qq = 0; qq < RQ; ++qq)
           if (qq < a.G) v = __fadd_rn(v, __fdiv_rn(__fsub_rn(xs[qq], mean[qq]), sd[qq]));
         v = __fdiv_rn(v, (float)a.G);
       }
@@ -445,23 +474,23 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   }
 }
 
-template <int TW, int SL>
+template <int TW, int SL, int QG>
 size_t mfma_lds_bytes(int tile_tokens, int bs_shift, bool paged) {
   const int blocks = paged ? (tile_tokens >> bs_shift) + 2 : 0;
-  return ((size_t)kFusedWaves * (TW + SL) * 4 + kFusedWaves * 128 + 128 + 8 + blocks) * 4;
+  return ((size_t)kFusedWaves * (TW + SL) * 4 * QG + kFusedWaves * 128 * QG + 128 * QG + 8 + blocks) * 4;
 }
 
-template <int DT, bool IL, int TW, int SL>
+template <int DT, bool IL, int TW, int SL, int QG>
 hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int B, hipStream_t s) {
-  const size_t lds = mfma_lds_bytes<TW, SL>(k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
+  const size_t lds = mfma_lds_bytes<TW, SL, QG>(k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
   if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
-  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL>);
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   for (int base = 0; base < B; base += seqs_per_launch) {
     k.seq_base = base;
     const int n = min(seqs_per_launch, B - base);
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads),
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads),
                        lds, s, k, bmat);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -471,10 +500,17 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
 
 template <int DT, bool IL>
 hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int B, hipStream_t s) {
+  if (k.G > 4) {
+    switch (tw) {   // eight query heads per KV head: 32 bytes of ring per token
+      case 512: return launch_mfma_t<DT, IL, 512, 64, 2>(k, bmat, seqs_per_launch, B, s);
+      case 256: return launch_mfma_t<DT, IL, 256, 64, 2>(k, bmat, seqs_per_launch, B, s);
+      default: return hipErrorInvalidValue;
+    }
+  }
   switch (tw) {
-    case 1024: return launch_mfma_t<DT, IL, 1024, 64>(k, bmat, seqs_per_launch, B, s);
-    case 512: return launch_mfma_t<DT, IL, 512, 64>(k, bmat, seqs_per_launch, B, s);
-    case 256: return launch_mfma_t<DT, IL, 256, 64>(k, bmat, seqs_per_launch, B, s);
+    case 1024: return launch_mfma_t<DT, IL, 1024, 64, 1>(k, bmat, seqs_per_launch, B, s);
+    case 512: return launch_mfma_t<DT, IL, 512, 64, 1>(k, bmat, seqs_per_launch, B, s);
+    case 256: return launch_mfma_t<DT, IL, 256, 64, 1>(k, bmat, seqs_per_launch, B, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -484,7 +520,7 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                           int resident) {
   FusedPlan p{};
-  if (resident <= 0 || D != 128 || G < 1 || G > 4 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
+  if (resident <= 0 || D != 128 || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
   int bs_shift = -1;
   for (int sft = 0; sft < 31; ++sft)
@@ -492,8 +528,9 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   if (paged && bs_shift < 0) return p;
   const int HC = ceil_div(Hkv, 8);
   const int tws[3] = {256, 512, 1024};
-  int tw = 1024;
-  for (int i = 0; i < 3; ++i)
+  const int ntw = G > 4 ? 2 : 3;          // the ring of a 1024-token tile fits LDS for four query heads only
+  int tw = tws[ntw - 1];
+  for (int i = 0; i < ntw; ++i)
     if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   const int tiles = ceil_div(Tmax, tw);
   if ((int64_t)tiles * HC > resident) return p;
@@ -535,11 +572,12 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
   const int64_t heads_total = (int64_t)a.B * a.L * a.Hkv;
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
-  const unsigned cgrid = (unsigned)ceil_div64(heads_total * 6 * 64, 256);
+  const int QG = a.G > 4 ? 2 : 1;
+  const unsigned cgrid = (unsigned)ceil_div64(heads_total * QG * 6 * 64, 256);
   const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
   if (a.kv_dtype != TRI_KV_BF16 && !fp8) return hipErrorInvalidValue;
   auto coef_launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, heads_total, bmat);
+    hipLaunchKernelGGL(kernel, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, QG, heads_total, bmat);
   };
   if (fp8) {
     if (il) coef_launch(coef_mfma_kernel<TRI_KV_FP8_E4M3, true>);
