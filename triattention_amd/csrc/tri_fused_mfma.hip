@@ -52,14 +52,6 @@ __host__ __device__ constexpr int slab_elem(int s, int kb, int e) {
   return DT == TRI_KV_FP8_E4M3 ? (kb + 4 * (s >> 1)) * 16 + (s & 1) * 8 + e : (4 * s + kb) * 8 + e;
 }
 
-// Four fp8 e4m3 bytes -> four bf16 (exact: e4m3 has 3 mantissa bits).
-__device__ __forceinline__ void fp8x4_to_bf16x4(uint32_t w, uint32_t& lo, uint32_t& hi) {
-  const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
-  const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
-  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, bf16x2));
-  hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, bf16x2));
-}
-
 __device__ __forceinline__ bf16x8 as_bf16x8(const uint4& v) { return __builtin_bit_cast(bf16x8, v); }
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
@@ -231,19 +223,36 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
   auto compute_step = [&](const StepData<DT>& raw, int l, int t) __attribute__((always_inline)) {
-    // The four bf16 A operands of the step.
+    // The four bf16 A operands of the step and the fp32 values of their elements (for the
+    // magnitudes): fp8 keys are widened once and both come out of that, bf16 keys are the
+    // loaded registers and the fp32 values are unpacked from them.
     struct { uint4 c[4]; } d;
+    float fe[4][8];
     if constexpr (FP8) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        fp8x4_to_bf16x4(raw.c[s].x, d.c[2 * s].x, d.c[2 * s].y);
-        fp8x4_to_bf16x4(raw.c[s].y, d.c[2 * s].z, d.c[2 * s].w);
-        fp8x4_to_bf16x4(raw.c[s].z, d.c[2 * s + 1].x, d.c[2 * s + 1].y);
-        fp8x4_to_bf16x4(raw.c[s].w, d.c[2 * s + 1].z, d.c[2 * s + 1].w);
+        const uint32_t w[4] = {raw.c[s].x, raw.c[s].y, raw.c[s].z, raw.c[s].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
+          const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+          float* f = &fe[2 * s + (i >> 1)][(i & 1) * 4];
+          f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
+          uint32_t* o = &(&d.c[2 * s + (i >> 1)].x)[(i & 1) * 2];
+          o[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+          o[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+        }
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) d.c[s] = raw.c[s];
+      for (int s = 0; s < 4; ++s) {
+        d.c[s] = raw.c[s];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t w = (&raw.c[s].x)[e >> 1];
+          fe[s][e] = (e & 1) ? bf16_hi(w) : bf16_lo(w);
+        }
+      }
     }
     f32x4 acc[QG], acc_e[QG];
 #pragma unroll
@@ -257,26 +266,13 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 #pragma unroll
     for (int set = 0; set < 2; ++set) {
       float mag[8];
-      if (IL) {
-        // chunks 2*set and 2*set + 1 hold four (real, imaginary) pairs each
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint4& cc = d.c[2 * set + (e >> 2)];
-          const uint32_t w = (&cc.x)[e & 3];
-          const float kr = bf16_lo(w), ki = bf16_hi(w);
-          mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
-        }
-      } else {
-        // real parts in chunk `set`, imaginary parts in chunk `set + 2`
-        const uint4& cr = d.c[set];
-        const uint4& ci = d.c[set + 2];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint32_t wr = (&cr.x)[e >> 1], wi = (&ci.x)[e >> 1];
-          const float kr = (e & 1) ? bf16_hi(wr) : bf16_lo(wr);
-          const float ki = (e & 1) ? bf16_hi(wi) : bf16_lo(wi);
-          mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
-        }
+      for (int e = 0; e < 8; ++e) {
+        // interleaved: operands 2*set and 2*set + 1 hold four (real, imaginary) pairs each;
+        // half: real parts in operand `set`, imaginary parts in operand `set + 2`
+        const float kr = IL ? fe[2 * set + (e >> 2)][2 * (e & 3)] : fe[set][e];
+        const float ki = IL ? fe[2 * set + (e >> 2)][2 * (e & 3) + 1] : fe[set + 2][e];
+        mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
       }
       uint4 hi, lo;
       float r[8];
