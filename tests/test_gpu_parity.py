@@ -182,8 +182,8 @@ def test_group_selection_matches_oracle(name):
 def test_group_selection_matches_reference_golden(tag, kw, path, fixture, monkeypatch):
     """Keep sets written by the reference's own selector (paged group branch), through the
     two-pass path and through both resident kernels."""
-    if path == "resident_valu":
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+    if path != "two_pass":
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", path.split("_")[1])
     gold = load_golden(fixture)
     layers, hkv, t, d = gold["keys"].shape
     hq = gold["q_mean_complex"].shape[1]
@@ -430,8 +430,7 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
         pytest.skip("the matrix-core kernel takes bf16 and fp8 keys; fp16 runs the vector-unit kernel")
     if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
         pytest.skip("the vector-unit kernel holds four query heads per KV head")
-    if kernel == "valu":
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)      # take that kernel however small the launch
     inp = build_inputs(w, case.get("kv_axis", 0))
     print(f"case={name} kernel={kernel} workload={w}", flush=True)
     caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=case.get("prefill_lens"))
@@ -456,7 +455,22 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
                             ft, k, tie_tol=2e-3 * scale)
 
 
-def test_resident_path_falls_back_when_shape_has_no_kernel():
+def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
+    sel = ops.SelectConfig(window_size=12)
+    for seq_lens, want in (((300,), "two_pass"), ((3072,) * 16, "resident_mfma"), ((2176,) * 16, "two_pass")):
+        w = small(seq_lens=seq_lens, num_layers=1)
+        tables = synth.make_block_tables(w)
+        cache = torch.zeros(2, w.pool_blocks, w.block_size, w.num_kv_heads, w.head_dim, dtype=torch.bfloat16, device=DEV)
+        kv = ops.PagedKV.from_kv_caches([cache])
+        batch = ops.StepBatch(DEV, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=tables)
+        qc, qa = synth.make_stats(w, DEV)
+        sc = ops.ScoreConfig(ops.fold_stats(qc, qa, torch.ones_like(qa)), synth.rope_inv_freq(w, DEV),
+                             synth.geometric_offsets(device=DEV))
+        assert ops.select_path(kv, batch, sc, sel) == want, seq_lens
+
+
+def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
     for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=64), {}),
                       (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
         w = small(**kw)

@@ -84,21 +84,25 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
 }
 
 tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
-  // bf16 and fp8 keys go to the matrix-core kernel, fp16 to the vector-unit one;
-  // TRIATTN_RESIDENT_KERNEL=valu forces the vector-unit kernel (for comparison runs).
+  // Resident kernels: bf16 and fp8 keys go to the matrix-core kernel, fp16 to the vector-unit
+  // one, and only launches that fill most of the chip take them.  TRIATTN_RESIDENT_KERNEL
+  // overrides the choice: "mfma" / "valu" take that kernel whenever the shape has it (however
+  // small the launch), "off" never takes a resident kernel.
   const char* force = getenv("TRIATTN_RESIDENT_KERNEL");
-  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) &&
-                         !(force && strcmp(force, "valu") == 0);
+  const bool f_valu = force && strcmp(force, "valu") == 0;
+  const bool f_mfma = force && strcmp(force, "mfma") == 0;
+  const bool f_off = force && strcmp(force, "off") == 0;
+  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) && !f_valu;
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;
-  const int resident = tri::fused_resident_workgroups();
+  const int resident = f_off ? 0 : tri::fused_resident_workgroups();
   tri::FusedPlan fused{};
   if (want_mfma)
     fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
-                                 sp->aggregation, b->max_seq_len, resident);
-  if (!fused.eligible)
+                                 sp->aggregation, b->max_seq_len, resident, f_mfma);
+  if (!fused.eligible && !f_mfma)
     fused = tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged, sp->aggregation,
-                            b->max_seq_len, resident);
+                            b->max_seq_len, resident, f_valu);
   return tri::plan_workspace(b->num_seqs, kv->num_layers, sp->num_score_heads, kv->head_dim / 2, sp->num_offsets,
                              kv->num_kv_heads, b->max_seq_len, fused);
 }
@@ -171,6 +175,9 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     hipStream_t s) {
   const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared;
   if (!fused) {
+    // The status word belongs to the resident kernel; on this path it just reads "fine".
+    const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
+    if (ce != hipSuccess) return launch_status(ce, "clear_status");
     float* raw = at<float>(ws, w.raw);
     const int64_t A = sp->num_score_heads;
     const int64_t rs_layer = (int64_t)batch->max_seq_len * A;

@@ -34,10 +34,11 @@ struct FusedPlan {
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();
+// any_fill: plan the resident kernel even for a launch that would leave most CUs idle.
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                     int resident);
+                     int resident, bool any_fill);
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident);
+                          int resident, bool any_fill);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {
@@ -115,6 +116,7 @@ struct SelectLaunch {
   int32_t* keep;       // [rows][max_budget]
 };
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
+hipError_t launch_clear_status(uint32_t* status, hipStream_t s);
 hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
                             const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry,
                             int32_t* keep, int keep_pitch, hipStream_t s);

@@ -408,7 +408,7 @@ int fused_resident_workgroups() {
 }
 
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                     int resident) {
+                     int resident, bool any_fill) {
   FusedPlan p{};
   if (resident <= 0 || D != 128 || G < 1 || G > 4 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
@@ -429,6 +429,8 @@ FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, i
   const int tile = tw * (kFusedWaves / HC);
   const int tiles = ceil_div(Tmax, tile);
   if (tiles > resident) return p;
+  // A launch that fills fewer than ~70 % of the CUs loses to the two-pass kernels.
+  if (!any_fill && (int64_t)B * tiles * 10 < (int64_t)resident * 7) return p;
   p.eligible = 1;
   p.tw = tw;
   p.HC = HC;

@@ -514,7 +514,7 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_
 }  // namespace
 
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident) {
+                          int resident, bool any_fill) {
   FusedPlan p{};
   if (resident <= 0 || D != 128 || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
@@ -530,6 +530,9 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
     if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   const int tiles = ceil_div(Tmax, tw);
   if ((int64_t)tiles * HC > resident) return p;
+  // A launch that fills fewer than ~70 % of the CUs loses to the two-pass kernels, which
+  // spread a small problem over the whole chip (crossover measured at B = 16: T ~ 2500).
+  if (!any_fill && (int64_t)B * tiles * HC * 10 < (int64_t)resident * 7) return p;
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;

@@ -275,6 +275,13 @@ hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows
   return hipGetLastError();
 }
 
+__global__ void clear_word_kernel(uint32_t* word) { *word = 0u; }
+
+hipError_t launch_clear_status(uint32_t* status, hipStream_t s) {
+  hipLaunchKernelGGL(clear_word_kernel, dim3(1), dim3(1), 0, s, status);
+  return hipGetLastError();
+}
+
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const int n = a.B * a.L * a.A;
   hipLaunchKernelGGL(finalize_stats_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s, a.partial, a.seq_lens,
