@@ -1,10 +1,9 @@
 // In-place, order-preserving paged K/V compaction for gfx950.
 //
 // keep[] is strictly ascending, so keep[j] >= j: destination slot j always lies at
-// or below its source.  One workgroup owns one stream -- (sequence, layer, K or V,
-// head) in per-head mode, (sequence, layer, K or V) in shared mode -- and walks the
-// destination slots in ascending tiles.  Every tile is read completely into
-// registers, the workgroup synchronises, then the tile is written: a tile's writes
+// or below its source.  One workgroup owns one (sequence, layer, K or V) and walks the
+// destination slots in ascending tiles, all heads together.  Every tile is read completely
+// into registers, the workgroup synchronises, then the tile is written: a tile's writes
 // land below the next tile's first slot while every later source lies at or above
 // it, so nothing that is still to be read is ever overwritten and no staging copy
 // of the cache is needed.  The reference gathers all T rows of K and V into
@@ -18,7 +17,23 @@ constexpr int kCompactThreads = 256;
 constexpr int kChunksPerThread = 4;                                  // 16-byte chunks held per thread
 static_assert(kChunksPerThread == 4, "compact_kernel spells out four chunk registers");
 constexpr int kTileChunks = kCompactThreads * kChunksPerThread;      // 16 KiB per tile
-constexpr int kSegSlots = 1024;                                      // slots whose addresses are staged in LDS
+constexpr int kOrderedThreads = 256;                                 // ordered pass: 4 waves, 16 KiB per tile; a whole batch of streams fits the chip at once
+constexpr int kOrderedTileChunks = kOrderedThreads * kChunksPerThread;
+constexpr int kSegEntries = 2048;                                    // (slot, list) addresses staged in LDS at a time
+
+// The per-layer pointers come out of a device-side table and are generic to the compiler;
+// these casts tell it they are global memory, so it emits global (not flat) loads and
+// stores, which complete in issue order and can be waited for individually.
+typedef unsigned int cu32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) cu32x4* GlobalChunk;
+typedef const __attribute__((address_space(1))) cu32x4* GlobalChunkIn;
+__device__ __forceinline__ uint4 load_chunk(const char* p) {
+  const cu32x4 v = *(GlobalChunkIn)(uintptr_t)p;
+  return uint4{v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ void store_chunk(char* p, const uint4& v) {
+  *(GlobalChunk)(uintptr_t)p = cu32x4{v.x, v.y, v.z, v.w};
+}
 
 struct CompactArgs {
   const void* const* k_layers;
@@ -45,13 +60,30 @@ __device__ __forceinline__ int64_t slot_offset(const CompactArgs& a, const int32
   return (int64_t)bt[lb] * a.stride_block_b + (int64_t)in_off * a.stride_token_b;
 }
 
-__global__ __launch_bounds__(kCompactThreads) void compact_kernel(CompactArgs a) {
-  __shared__ int64_t src_off[kSegSlots];
-  __shared__ int64_t dst_off[kSegSlots];
+// Offsets are kept in 16-byte units so the per-row index arithmetic stays 32-bit.
+__device__ __forceinline__ uint32_t slot_units(const CompactArgs& a, const int32_t* bt, int tok) {
+  const int lb = a.bs_shift >= 0 ? (tok >> a.bs_shift) : (tok / a.block_size);
+  const int in_off = tok - lb * a.block_size;
+  return (uint32_t)bt[lb] * a.block_units + (uint32_t)in_off * a.token_units;
+}
 
-  // stream -> (b, l, kv, row)
+constexpr uint32_t kNoSource = 0xffffffffu;
+
+// Ordered pass: the slots whose source token lies inside the kept prefix [0, k).  With keep
+// ascending they form a prefix of every list, and only they can be overwritten before they
+// are read.  One workgroup owns one (sequence, layer, K or V) and moves ALL heads of a tile
+// of destination slots together, so it writes whole token rows and reads, when little is
+// dropped (the steady-state step), from the same few rows it writes.  A tile is read
+// completely, the workgroup synchronises, the tile is written: a tile's writes land below
+// the next tile's first slot while every later source lies at or above it, for every head,
+// so nothing that is still to be read is overwritten.  Slots whose source lies at or beyond
+// k are left to compact_bulk_kernel.
+__global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a) {
+  __shared__ uint32_t src_units[kSegEntries];   // [slot][list], kNoSource: not this pass's
+  __shared__ uint32_t dst_units[kSegEntries];   // [slot]
+  __shared__ int prefix_len[256];
+
   int sidx = blockIdx.x;
-  const int row = sidx % (a.streams_per_layer / 2); sidx /= (a.streams_per_layer / 2);
   const int kv = sidx % 2; sidx /= 2;
   const int l = sidx % a.L;
   const int b = sidx / a.L;
@@ -60,87 +92,117 @@ __global__ __launch_bounds__(kCompactThreads) void compact_kernel(CompactArgs a)
   const int T = a.seq_lens[b];
   if (k > T) k = T;
   if (k <= 0) return;
-  const int rows = a.shared ? 1 : a.Hkv;
-  const int32_t* keep = a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows + row) * a.max_budget;
+  const int lists = a.shared ? 1 : a.Hkv;
+  const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * lists * a.max_budget;
   const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
   char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
-  const int head0 = a.shared ? 0 : row;
 
-  // Only slots whose source lies inside the kept prefix [0, k) can be overwritten
-  // before they are read; with keep ascending those form a prefix of the list.  The
-  // rest (source >= k) is moved by compact_bulk_kernel, which needs no ordering.
-  if (a.split_bulk) {
-    // keep is ascending: the number of entries below k is the length of that prefix.
-    __shared__ int prefix_len;
+  // Length of the prefix of every list (entries below k), and the longest one.
+  for (int h = threadIdx.x; h < lists; h += kOrderedThreads) prefix_len[h] = 0;
+  __syncthreads();
+  for (int h = 0; h < lists; ++h) {
     int below = 0;
-    for (int j = threadIdx.x; j < k; j += kCompactThreads) below += keep[j] < k;
-    if (threadIdx.x == 0) prefix_len = 0;
-    __syncthreads();
-    if (below) atomicAdd(&prefix_len, below);
-    __syncthreads();
-    k = prefix_len;
-    if (k <= 0) return;
+    for (int j = threadIdx.x; j < k; j += kOrderedThreads) below += keep[(int64_t)h * a.max_budget + j] < k;
+    if (below) atomicAdd(&prefix_len[h], below);
   }
+  __syncthreads();
+  int J = 0;
+  for (int h = 0; h < lists; ++h) J = max(J, prefix_len[h]);
+  if (J <= 0) return;
 
-  const int chunks_per_slot = a.heads_per_slot * a.chunks_per_row;
-  const int slots_per_tile = max(kTileChunks / chunks_per_slot, 1);
+  const int row_chunks = a.heads_per_slot * a.chunks_per_row;       // chunks one list moves per slot
+  const int slot_chunks = lists * row_chunks;                       // chunks of a whole token row
+  const int slots_per_tile = max(kOrderedTileChunks / slot_chunks, 1);
+  const int seg_slots = max(kSegEntries / lists / slots_per_tile, 1) * slots_per_tile;
 
-  for (int seg = 0; seg < k; seg += kSegSlots) {
-    const int nseg = min(kSegSlots, k - seg);
+  for (int seg = 0; seg < J; seg += seg_slots) {
+    const int nseg = min(seg_slots, J - seg);
     __syncthreads();   // previous segment's LDS no longer in use
-    for (int i = threadIdx.x; i < nseg; i += kCompactThreads) {
-      const int j = seg + i;
-      src_off[i] = slot_offset(a, bt, keep[j]);
-      dst_off[i] = slot_offset(a, bt, j);
+    for (int i = threadIdx.x; i < nseg * lists; i += kOrderedThreads) {
+      const int sl = i / lists, h = i - sl * lists;
+      const int j = seg + sl;
+      const int src = keep[(int64_t)h * a.max_budget + j];
+      const bool mine = j < prefix_len[h] && src != j;             // source below k, row not already in place
+      src_units[i] = mine ? slot_units(a, bt, src) : kNoSource;
+      if (h == 0) dst_units[sl] = slot_units(a, bt, j);
     }
     __syncthreads();
 
-    for (int t0 = 0; t0 < nseg; t0 += slots_per_tile) {
-      const int nchunks = min(slots_per_tile, nseg - t0) * chunks_per_slot;
-      // A slot wider than a tile is moved in several passes; every pass is read
-      // completely before it is written, and passes of one slot never overlap.
-      for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
-        // Branch-free loads: idle chunks re-read the tile's first source row (a cache
-        // hit) and only their store is masked.
-        int64_t so[kChunksPerThread], dsto[kChunksPerThread];
-        bool live[kChunksPerThread];
+    // Units of work: tiles of slots, or, when a token row is wider than a tile, the passes
+    // over one row.  The loads of unit u+1 are issued before the stores of unit u (their
+    // sources lie at or above the first slot of unit u+1, beyond everything unit u writes;
+    // passes of one row touch disjoint chunks), so a load batch and a store batch are
+    // always in flight together; a barrier between the loads of a unit and its stores
+    // orders them across the workgroup.
+    const int passes = max(ceil_div(slot_chunks, kOrderedTileChunks), 1);
+    const int tiles = ceil_div(nseg, slots_per_tile);
+    const int units = tiles * passes;
+    uint32_t dsto[kChunksPerThread];
+    bool live[kChunksPerThread];
+    uint4 r0, r1, r2, r3;
+    auto issue = [&](int u) __attribute__((always_inline)) {
+      const int t0 = (u / passes) * slots_per_tile, c0 = (u % passes) * kOrderedTileChunks;
+      const int nchunks = min(slots_per_tile, nseg - t0) * slot_chunks;
+      uint32_t so[kChunksPerThread];
 #pragma unroll
-        for (int c = 0; c < kChunksPerThread; ++c) {
-          const int ci = c0 + c * kCompactThreads + threadIdx.x;
-          live[c] = ci < nchunks;
-          const int cic = live[c] ? ci : c0;
-          const int sl = t0 + cic / chunks_per_slot;
-          const int within = cic % chunks_per_slot;
-          const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
-          const int64_t inner = (int64_t)(head0 + hh) * a.stride_head_b + (int64_t)cc * 16;
-          so[c] = src_off[sl] + inner;
-          dsto[c] = dst_off[sl] + inner;
-          live[c] = live[c] && so[c] != dsto[c];     // row already in place
-        }
-        uint4 r0 = *reinterpret_cast<const uint4*>(base + so[0]);
-        uint4 r1 = *reinterpret_cast<const uint4*>(base + so[1]);
-        uint4 r2 = *reinterpret_cast<const uint4*>(base + so[2]);
-        uint4 r3 = *reinterpret_cast<const uint4*>(base + so[3]);
-        __syncthreads();   // every read of this tile is ordered before any write of it
-        if (live[0]) *reinterpret_cast<uint4*>(base + dsto[0]) = r0;
-        if (live[1]) *reinterpret_cast<uint4*>(base + dsto[1]) = r1;
-        if (live[2]) *reinterpret_cast<uint4*>(base + dsto[2]) = r2;
-        if (live[3]) *reinterpret_cast<uint4*>(base + dsto[3]) = r3;
+      for (int c = 0; c < kChunksPerThread; ++c) {
+        // Branch-free: an idle chunk re-reads its own destination and only its store is masked.
+        const int ci = c0 + c * kOrderedThreads + threadIdx.x;
+        const bool in = ci < nchunks;
+        const int cic = in ? ci : c0;
+        const int sl = t0 + cic / slot_chunks;
+        const int within = cic % slot_chunks;
+        const int h = within / row_chunks, rem = within - h * row_chunks;
+        const int hh = rem / a.chunks_per_row, cc = rem - hh * a.chunks_per_row;
+        const uint32_t inner = (uint32_t)((a.shared ? 0 : h) + hh) * a.head_units + (uint32_t)cc;
+        const uint32_t su = src_units[sl * lists + h];
+        dsto[c] = dst_units[sl] + inner;
+        live[c] = in && su != kNoSource;
+        so[c] = live[c] ? su + inner : dsto[c];
       }
+      r0 = load_chunk(base + ((uint64_t)so[0] << 4));
+      r1 = load_chunk(base + ((uint64_t)so[1] << 4));
+      r2 = load_chunk(base + ((uint64_t)so[2] << 4));
+      r3 = load_chunk(base + ((uint64_t)so[3] << 4));
+    };
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): this thread's loads of unit 0 have arrived
+    __syncthreads();                       // ... and every other thread's
+    uint4 w0 = r0, w1 = r1, w2 = r2, w3 = r3;
+    uint32_t d0 = dsto[0], d1 = dsto[1], d2 = dsto[2], d3 = dsto[3];
+    bool l0 = live[0], l1 = live[1], l2 = live[2], l3 = live[3];
+    for (int u = 0; u + 1 < units; ++u) {
+      // Unit u is a full tile (only the last unit of a segment can be partial): every chunk
+      // stores, a chunk that is not this pass's writes back what it read from its own
+      // destination.  Exactly four stores follow the four loads of unit u+1, and vector
+      // memory operations complete in issue order, so "at most four outstanding" means the
+      // loads of unit u+1 have arrived; the wave does not wait for its stores to be
+      // acknowledged.  The loaded registers are copied right after that wait, so nothing at
+      // the top of the loop depends on a load.
+      issue(u + 1);
+      store_chunk(base + ((uint64_t)d0 << 4), w0);
+      store_chunk(base + ((uint64_t)d1 << 4), w1);
+      store_chunk(base + ((uint64_t)d2 << 4), w2);
+      store_chunk(base + ((uint64_t)d3 << 4), w3);
+      asm volatile("" ::: "memory");            // keep the compiler from moving memory operations across
+      __builtin_amdgcn_s_waitcnt(0x0074);       // vmcnt(4) lgkmcnt(0)
+      w0 = r0; w1 = r1; w2 = r2; w3 = r3;
+      d0 = dsto[0]; d1 = dsto[1]; d2 = dsto[2]; d3 = dsto[3];
+      l0 = live[0]; l1 = live[1]; l2 = live[2]; l3 = live[3];
+      __builtin_amdgcn_s_barrier();             // ... in every thread of the workgroup
+      asm volatile("" ::: "memory");
     }
+    // Last unit of the segment: its loads have arrived in every thread.
+    if (l0) store_chunk(base + ((uint64_t)d0 << 4), w0);
+    if (l1) store_chunk(base + ((uint64_t)d1 << 4), w1);
+    if (l2) store_chunk(base + ((uint64_t)d2 << 4), w2);
+    if (l3) store_chunk(base + ((uint64_t)d3 << 4), w3);
   }
 }
 
 // Slots whose source token lies at or beyond the budget: sources (>= k) and
 // destinations (< k) cannot overlap, so this is a flat gather copy.  One workgroup
 // moves a tile of destination slots for all heads, i.e. whole contiguous token rows.
-// Offsets are kept in 16-byte units so the per-row index arithmetic stays 32-bit.
-__device__ __forceinline__ uint32_t slot_units(const CompactArgs& a, const int32_t* bt, int tok) {
-  const int lb = a.bs_shift >= 0 ? (tok >> a.bs_shift) : (tok / a.block_size);
-  const int in_off = tok - lb * a.block_size;
-  return (uint32_t)bt[lb] * a.block_units + (uint32_t)in_off * a.token_units;
-}
-
 __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactArgs a) {
   int sidx = blockIdx.y;
   const int kv = sidx % 2; sidx /= 2;
@@ -189,10 +251,10 @@ __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactAr
     uint4 regs[kChunksPerThread];
 #pragma unroll
     for (int c = 0; c < kChunksPerThread; ++c)
-      regs[c] = *reinterpret_cast<const uint4*>(base + ((uint64_t)so[c] << 4));
+      regs[c] = load_chunk(base + ((uint64_t)so[c] << 4));
 #pragma unroll
     for (int c = 0; c < kChunksPerThread; ++c)
-      if (live[c]) *reinterpret_cast<uint4*>(base + ((uint64_t)dsto[c] << 4)) = regs[c];
+      if (live[c]) store_chunk(base + ((uint64_t)dsto[c] << 4), regs[c]);
   }
 }
 
@@ -291,8 +353,8 @@ __global__ __launch_bounds__(256) void permute_to_staging_kernel(FullArgs f) {
     const int sl = ci / chunks_per_slot, within = ci % chunks_per_slot;
     const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
     const int64_t so = slot_offset(a, bt, n0 + sl) + (int64_t)(head0 + hh) * a.stride_head_b + cc * 16;
-    const uint4 v = *reinterpret_cast<const uint4*>(base + so);
-    *reinterpret_cast<uint4*>(stage + ((int64_t)dest[sl] * chunks_per_slot + within) * 16) = v;
+    const uint4 v = load_chunk(base + so);
+    store_chunk(stage + ((int64_t)dest[sl] * chunks_per_slot + within) * 16, v);
   }
 }
 
@@ -318,8 +380,7 @@ __global__ __launch_bounds__(256) void staging_to_cache_kernel(FullArgs f) {
     const int sl = ci / chunks_per_slot, within = ci % chunks_per_slot;
     const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
     const int64_t d = slot_offset(a, bt, n0 + sl) + (int64_t)(head0 + hh) * a.stride_head_b + cc * 16;
-    *reinterpret_cast<uint4*>(base + d) =
-        *reinterpret_cast<const uint4*>(stage + ((int64_t)(n0 + sl) * chunks_per_slot + within) * 16);
+    store_chunk(base + d, load_chunk(stage + ((int64_t)(n0 + sl) * chunks_per_slot + within) * 16));
   }
 }
 
@@ -382,7 +443,7 @@ hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
   // Ordered pass over the slots whose sources lie inside the kept prefix, then the
   // unordered bulk pass over the rest; the first must finish reading before the second
   // writes, which stream order guarantees.
-  hipLaunchKernelGGL(compact_kernel, dim3(streams), dim3(kCompactThreads), 0, s, c);
+  hipLaunchKernelGGL(compact_kernel, dim3(a.B * a.L * 2), dim3(kOrderedThreads), 0, s, c);
   if (c.split_bulk) {
     hipError_t e0 = hipGetLastError();
     if (e0 != hipSuccess) return e0;
