@@ -235,6 +235,20 @@ def main() -> int:
                      "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, path))},
     }
+    # A plain device-to-device copy of 1 GiB on the same box, for scale: bytes read + bytes
+    # written per second (outside every timed region of the step).
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    c1.record()
+    torch.cuda.synchronize()
+    out["device_copy_gbs"] = 5 * 2 * (1 << 30) / (c0.elapsed_time(c1) * 1e-3) / 1e9
+    out["frac_of_device_copy"] = step_gbs / out["device_copy_gbs"]
+    del src, dst
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)

@@ -414,6 +414,8 @@ RESIDENT_CASES = {
     "tw64": dict(w=small(seq_lens=(9000,) * 20, budget=512, num_layers=2)),
     "tw128": dict(w=small(seq_lens=(40000, 3000, 25001), budget=2048, num_layers=2)),
     "two_launches": dict(w=small(seq_lens=(70000, 100, 66000, 69000), budget=1024, num_layers=2)),
+    "packed_ragged_launches": dict(w=small(seq_lens=(30000, 700, 61000, 9000, 45000, 1, 33000, 12000, 52000, 2100),
+                                           budget=512, num_layers=2)),
 }
 
 

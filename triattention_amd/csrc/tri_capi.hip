@@ -203,6 +203,7 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.coef = at<float>(ws, w.coef);
   a.xchg = at<unsigned long long>(ws, w.xchg);
   a.status = at<uint32_t>(ws, w.status);
+  a.pack = at<int32_t>(ws, w.pack);
   a.fin = fin ? fin : at<float>(ws, w.fin);
   a.plan = w.fused;
   a.bmat = at<char>(ws, w.bmat);

@@ -29,7 +29,8 @@ struct FusedPlan {
   int HC;               // chunks of 8 KV heads; waves of a workgroup are split over them
   int tile_tokens;      // tokens per workgroup
   int tiles_per_seq;    // workgroups per sequence (by max_seq_len)
-  int seqs_per_launch;  // whole sequences per launch
+  int seqs_per_launch;  // whole sequences of maximum length per launch
+  int resident;         // workgroups the device holds at once
   int bs_shift;
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
@@ -50,6 +51,7 @@ struct Workspace {
   int64_t fin;       // [B*L*Hkv][Tmax] fp32 selection scores (worst case: per-layer selection)
   int64_t xchg;      // [B][L][tiles_per_seq][A][2] tagged sums exchanged by the resident kernel
   int64_t status;    // one word: non-zero when a bounded wait of the resident kernel expired
+  int64_t pack;      // [2][B] int32: launch of every sequence and its first workgroup there (several launches)
   int64_t bmat;      // [B][L][Hkv][groups of 4 query heads][6][64][8] bf16 coefficient slabs (matrix-core kernel)
   int64_t total;
   int32_t num_tiles; // NT
@@ -70,6 +72,7 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
   w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
   w.status = take(256);
+  w.pack = take(fused.eligible ? (int64_t)B * 8 : 0);
   w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * (A / Hkv > 4 ? 2 : 1) * 6 * 64 * 16 : 0);
   w.total = off;
   return w;
@@ -134,6 +137,7 @@ struct FusedLaunch {
   const float* coef;             // workspace
   unsigned long long* xchg;      // workspace
   uint32_t* status;              // workspace
+  int32_t* pack;                 // workspace
   void* bmat;                    // workspace (matrix-core kernel)
   float* fin;                    // [B*Hkv][Tmax]
   FusedPlan plan;

@@ -41,9 +41,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int b = a.seq_base + blockIdx.x / a.tiles_per_seq;
-  const int tile = blockIdx.x % a.tiles_per_seq;
-  if (b >= a.num_seqs) return;
+  int b, tile;
+  if (!locate_workgroup(a, a.tiles_per_seq, 1, reinterpret_cast<int*>(lds), b, tile)) return;
   const int T = a.seq_lens[b];
   const int n0 = tile * a.tile_tokens;
   if (n0 >= T) return;
@@ -365,17 +364,31 @@ size_t fused_lds_bytes(int A, int tile_tokens, int bs_shift, bool paged) {
 }
 
 template <int DT, bool IL, int TW, int SL>
-hipError_t launch_fused_t(FusedArgs& k, int seqs_per_launch, int B, hipStream_t s) {
+hipError_t launch_fused_t(FusedArgs& k, int seqs_per_launch, int resident, int B, hipStream_t s) {
   const size_t lds = fused_lds_bytes<TW, SL>(k.A, k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
   if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
   const void* fn = reinterpret_cast<const void*>(&fused_select_kernel<DT, IL, TW, SL>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  for (int base = 0; base < B; base += seqs_per_launch) {
-    k.seq_base = base;
-    const int n = min(seqs_per_launch, B - base);
-    hipLaunchKernelGGL((fused_select_kernel<DT, IL, TW, SL>), dim3(n * k.tiles_per_seq), dim3(kFusedThreads), lds, s,
-                       k);
+  if (B <= seqs_per_launch) {
+    k.packed = 0;
+    k.seq_base = 0;
+    const int n = B;
+    hipLaunchKernelGGL((fused_select_kernel<DT, IL, TW, SL>), dim3(n * k.tiles_per_seq), dim3(kFusedThreads), lds, s, k);
+    return hipGetLastError();
+  }
+  // More workgroups than the device holds at once: whole sequences are packed into
+  // launches on the device (the host does not know the individual lengths); the host
+  // issues as many launches as the worst case needs, surplus ones find no work.
+  k.packed = 1;
+  hipLaunchKernelGGL(fused_pack_kernel, dim3(1), dim3(256), 0, s, k.seq_lens, B, k.tile_tokens, 1, resident,
+                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base));
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int launches = ceil_div(B, seqs_per_launch);
+  for (int i = 0; i < launches; ++i) {
+    k.launch_idx = i;
+    hipLaunchKernelGGL((fused_select_kernel<DT, IL, TW, SL>), dim3(resident), dim3(kFusedThreads), lds, s, k);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -383,11 +396,11 @@ hipError_t launch_fused_t(FusedArgs& k, int seqs_per_launch, int B, hipStream_t 
 }
 
 template <int DT, bool IL>
-hipError_t launch_fused_tw(FusedArgs& k, int tw, int seqs_per_launch, int B, hipStream_t s) {
+hipError_t launch_fused_tw(FusedArgs& k, int tw, int seqs_per_launch, int resident, int B, hipStream_t s) {
   switch (tw) {
-    case 128: return launch_fused_t<DT, IL, 128, 16>(k, seqs_per_launch, B, s);
-    case 64: return launch_fused_t<DT, IL, 64, 16>(k, seqs_per_launch, B, s);
-    case 32: return launch_fused_t<DT, IL, 32, 8>(k, seqs_per_launch, B, s);
+    case 128: return launch_fused_t<DT, IL, 128, 16>(k, seqs_per_launch, resident, B, s);
+    case 64: return launch_fused_t<DT, IL, 64, 16>(k, seqs_per_launch, resident, B, s);
+    case 32: return launch_fused_t<DT, IL, 32, 8>(k, seqs_per_launch, resident, B, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -437,6 +450,7 @@ FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, i
   p.tile_tokens = tile;
   p.tiles_per_seq = tiles;
   p.seqs_per_launch = resident / tiles;
+  p.resident = resident;
   p.bs_shift = bs_shift;
   return p;
 }
@@ -461,6 +475,8 @@ hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s) {
   k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
   k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
   k.spin_ticks = 200000000LL;   // 2 s of the 100 MHz wall clock
+  k.seq_launch = a.pack;
+  k.seq_wg_base = a.pack + a.B;
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
   hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div64(words, 256)), dim3(256), 0, s, a.xchg, words,
                      a.status);
@@ -469,14 +485,14 @@ hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s) {
   const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
   switch (a.kv_dtype) {
     case TRI_KV_BF16:
-      return il ? launch_fused_tw<TRI_KV_BF16, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
-                : launch_fused_tw<TRI_KV_BF16, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
+      return il ? launch_fused_tw<TRI_KV_BF16, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+                : launch_fused_tw<TRI_KV_BF16, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
     case TRI_KV_FP16:
-      return il ? launch_fused_tw<TRI_KV_FP16, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
-                : launch_fused_tw<TRI_KV_FP16, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
+      return il ? launch_fused_tw<TRI_KV_FP16, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+                : launch_fused_tw<TRI_KV_FP16, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
     case TRI_KV_FP8_E4M3:
-      return il ? launch_fused_tw<TRI_KV_FP8_E4M3, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
-                : launch_fused_tw<TRI_KV_FP8_E4M3, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
+      return il ? launch_fused_tw<TRI_KV_FP8_E4M3, true>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+                : launch_fused_tw<TRI_KV_FP8_E4M3, false>(k, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
     default: return hipErrorInvalidValue;
   }
 }

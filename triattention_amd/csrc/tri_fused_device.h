@@ -26,7 +26,84 @@ struct FusedArgs {
   int tiles_per_seq, tile_tokens, seq_base, num_seqs, Tmax;
   int normalize, window_size, protect_prefill, group_reduce, layer_reduce;
   long long spin_ticks;
+  // Several launches (more workgroups than the device holds at once): which launch a
+  // sequence belongs to and its first workgroup there, written by fused_pack_kernel.
+  const int32_t* seq_launch;
+  const int32_t* seq_wg_base;
+  int packed, launch_idx;
 };
+
+// Which (sequence, workgroup within the sequence) this workgroup serves; false: none.
+// One launch: sequences in order, wgs_per_seq workgroups each.  Several launches: looked up
+// in the packing tables.  `slot` is one int of LDS; contains a __syncthreads().
+__device__ __forceinline__ bool locate_workgroup(const FusedArgs& a, int wgs_per_seq, int wg_mult, int* slot,
+                                                 int& b, int& within) {
+  if (!a.packed) {
+    b = a.seq_base + blockIdx.x / wgs_per_seq;
+    within = blockIdx.x % wgs_per_seq;
+    return b < a.num_seqs;
+  }
+  if (threadIdx.x == 0) *slot = -1;
+  __syncthreads();
+  for (int s = threadIdx.x; s < a.num_seqs; s += blockDim.x) {
+    if (a.seq_launch[s] != a.launch_idx) continue;
+    const int n = ceil_div(a.seq_lens[s], a.tile_tokens) * wg_mult;
+    const int base = a.seq_wg_base[s];
+    if ((int)blockIdx.x >= base && (int)blockIdx.x < base + n) *slot = s;
+  }
+  __syncthreads();
+  b = *slot;
+  if (b < 0) return false;
+  within = blockIdx.x - a.seq_wg_base[b];
+  return true;
+}
+
+// Packs whole sequences into launches of at most `capacity` workgroups: longest first, each
+// into the first of the eight most recently opened launches that still has room.  No
+// launch holds fewer sequences than capacity / (largest sequence) allows, so the number of
+// launches never exceeds what the host provides for.  One workgroup.
+__global__ __launch_bounds__(256) void fused_pack_kernel(const int32_t* seq_lens, int B, int tile_tokens,
+                                                         int wg_mult, int capacity, int32_t* seq_launch,
+                                                         int32_t* seq_wg_base) {
+  constexpr int kMaxSorted = 4096;
+  __shared__ int order[kMaxSorted];
+  const bool sorted = B <= kMaxSorted;
+  if (sorted) {
+    for (int s = threadIdx.x; s < B; s += blockDim.x) {
+      const int n = ceil_div(seq_lens[s], tile_tokens);
+      int rank = 0;
+      for (int c = 0; c < B; ++c) {
+        const int m = ceil_div(seq_lens[c], tile_tokens);
+        rank += (m > n) || (m == n && c < s);
+      }
+      order[rank] = s;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  int used[8];
+  int first = 0, open = 1;          // launches [first, first + open) are candidates
+  for (int i = 0; i < 8; ++i) used[i] = 0;
+  for (int i = 0; i < B; ++i) {
+    const int s = sorted ? order[i] : i;
+    const int n = ceil_div(seq_lens[s], tile_tokens) * wg_mult;
+    int pick = -1;
+    for (int c = 0; c < open; ++c)
+      if (used[c] + n <= capacity) { pick = c; break; }
+    if (pick < 0) {
+      if (open == 8) {               // forget the oldest candidate
+        for (int c = 0; c < 7; ++c) used[c] = used[c + 1];
+        ++first;
+        --open;
+      }
+      pick = open++;
+      used[pick] = 0;
+    }
+    seq_launch[s] = first + pick;
+    seq_wg_base[s] = used[pick];
+    used[pick] += n;
+  }
+}
 
 __device__ __forceinline__ unsigned long long xchg_load(const unsigned long long* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -125,10 +125,10 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int chunk = blockIdx.x % a.HC;
-  const int tile = (blockIdx.x / a.HC) % a.tiles_per_seq;
-  const int b = a.seq_base + blockIdx.x / (a.HC * a.tiles_per_seq);
-  if (b >= a.num_seqs) return;
+  int b, within;
+  if (!locate_workgroup(a, a.HC * a.tiles_per_seq, a.HC, reinterpret_cast<int*>(lds), b, within)) return;
+  const int chunk = within % a.HC;
+  const int tile = within / a.HC;
   const int T = a.seq_lens[b];
   const int n0 = tile * a.tile_tokens;
   if (n0 >= T) return;
@@ -477,17 +477,31 @@ size_t mfma_lds_bytes(int tile_tokens, int bs_shift, bool paged) {
 }
 
 template <int DT, bool IL, int TW, int SL, int QG>
-hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int B, hipStream_t s) {
+hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
   const size_t lds = mfma_lds_bytes<TW, SL, QG>(k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
   if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
   const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  for (int base = 0; base < B; base += seqs_per_launch) {
-    k.seq_base = base;
-    const int n = min(seqs_per_launch, B - base);
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads),
-                       lds, s, k, bmat);
+  if (B <= seqs_per_launch) {
+    k.packed = 0;
+    k.seq_base = 0;
+    const int n = B;
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads), lds, s, k, bmat);
+    return hipGetLastError();
+  }
+  // More workgroups than the device holds at once: whole sequences are packed into
+  // launches on the device (the host does not know the individual lengths); the host
+  // issues as many launches as the worst case needs, surplus ones find no work.
+  k.packed = 1;
+  hipLaunchKernelGGL(fused_pack_kernel, dim3(1), dim3(256), 0, s, k.seq_lens, B, k.tile_tokens, k.HC, resident,
+                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base));
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int launches = ceil_div(B, seqs_per_launch);
+  for (int i = 0; i < launches; ++i) {
+    k.launch_idx = i;
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(resident), dim3(kFusedThreads), lds, s, k, bmat);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -495,18 +509,18 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
 }
 
 template <int DT, bool IL>
-hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int B, hipStream_t s) {
+hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int resident, int B, hipStream_t s) {
   if (k.G > 4) {
     switch (tw) {   // eight query heads per KV head: 32 bytes of ring per token
-      case 512: return launch_mfma_t<DT, IL, 512, 64, 2>(k, bmat, seqs_per_launch, B, s);
-      case 256: return launch_mfma_t<DT, IL, 256, 64, 2>(k, bmat, seqs_per_launch, B, s);
+      case 512: return launch_mfma_t<DT, IL, 512, 64, 2>(k, bmat, seqs_per_launch, resident, B, s);
+      case 256: return launch_mfma_t<DT, IL, 256, 64, 2>(k, bmat, seqs_per_launch, resident, B, s);
       default: return hipErrorInvalidValue;
     }
   }
   switch (tw) {
-    case 1024: return launch_mfma_t<DT, IL, 1024, 64, 1>(k, bmat, seqs_per_launch, B, s);
-    case 512: return launch_mfma_t<DT, IL, 512, 64, 1>(k, bmat, seqs_per_launch, B, s);
-    case 256: return launch_mfma_t<DT, IL, 256, 64, 1>(k, bmat, seqs_per_launch, B, s);
+    case 1024: return launch_mfma_t<DT, IL, 1024, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
+    case 512: return launch_mfma_t<DT, IL, 512, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
+    case 256: return launch_mfma_t<DT, IL, 256, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -539,6 +553,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   p.tile_tokens = tw;
   p.tiles_per_seq = tiles;
   p.seqs_per_launch = resident / (tiles * HC);
+  p.resident = resident;
   p.bs_shift = bs_shift;
   return p;
 }
@@ -563,6 +578,8 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
   k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
   k.spin_ticks = 200000000LL;   // 2 s of the 100 MHz wall clock
+  k.seq_launch = a.pack;
+  k.seq_wg_base = a.pack + a.B;
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
   hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div64(words, 256)), dim3(256), 0, s, a.xchg, words,
                      a.status);
@@ -588,10 +605,10 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
-    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
-  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s)
-            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
 }
 
 }  // namespace tri
