@@ -1,8 +1,8 @@
 // In-place, order-preserving paged K/V compaction for gfx950.
 //
 // keep[] is strictly ascending, so keep[j] >= j: destination slot j always lies at
-// or below its source.  One workgroup owns one (sequence, layer, K or V) and walks the
-// destination slots in ascending tiles, all heads together.  Every tile is read completely
+// or below its source.  One workgroup owns one (sequence, layer, K or V, head) and walks the
+// destination slots in ascending tiles.  Every tile is read completely
 // into registers, the workgroup synchronises, then the tile is written: a tile's writes
 // land below the next tile's first slot while every later source lies at or above
 // it, so nothing that is still to be read is ever overwritten and no staging copy
@@ -48,6 +48,7 @@ struct CompactArgs {
   uint32_t block_units, token_units, head_units;           // the same strides in 16-byte units
   int B, L, Hkv, block_size, bs_shift, block_table_pitch, max_budget;
   int keep_per_layer, shared;
+  int lists_per_wg;        // keep lists (heads) one workgroup of the ordered pass moves together
   int split_bulk;          // 1: the ordered kernel stops at the first source >= budget
   int chunks_per_row;      // 16-byte chunks of one head row (D * elem_bytes / 16)
   int heads_per_slot;      // shared ? Hkv : 1
@@ -71,19 +72,23 @@ constexpr uint32_t kNoSource = 0xffffffffu;
 
 // Ordered pass: the slots whose source token lies inside the kept prefix [0, k).  With keep
 // ascending they form a prefix of every list, and only they can be overwritten before they
-// are read.  One workgroup owns one (sequence, layer, K or V) and moves ALL heads of a tile
-// of destination slots together, so it writes whole token rows and reads, when little is
-// dropped (the steady-state step), from the same few rows it writes.  A tile is read
-// completely, the workgroup synchronises, the tile is written: a tile's writes land below
-// the next tile's first slot while every later source lies at or above it, for every head,
-// so nothing that is still to be read is overwritten.  Slots whose source lies at or beyond
-// k are left to compact_bulk_kernel.
+// are read.  One workgroup owns one (sequence, layer, K or V, group of keep lists) and moves
+// a tile of destination slots of its lists together.  A tile is read completely, the
+// workgroup synchronises, the tile is written: a tile's writes land below the next tile's
+// first slot while every later source lies at or above it, for every list, so nothing that
+// is still to be read is overwritten.  Slots whose source lies at or beyond k are left to
+// compact_bulk_kernel.
 __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a) {
   __shared__ uint32_t src_units[kSegEntries];   // [slot][list], kNoSource: not this pass's
   __shared__ uint32_t dst_units[kSegEntries];   // [slot]
   __shared__ int prefix_len[256];
 
+  // workgroup -> (sequence, layer, K or V, group of lists)
+  const int all_lists = a.shared ? 1 : a.Hkv;
+  const int lists = a.lists_per_wg;
+  const int groups = all_lists / lists;
   int sidx = blockIdx.x;
+  const int list0 = (sidx % groups) * lists; sidx /= groups;
   const int kv = sidx % 2; sidx /= 2;
   const int l = sidx % a.L;
   const int b = sidx / a.L;
@@ -92,8 +97,8 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
   const int T = a.seq_lens[b];
   if (k > T) k = T;
   if (k <= 0) return;
-  const int lists = a.shared ? 1 : a.Hkv;
-  const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * lists * a.max_budget;
+  const int32_t* keep =
+      a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * all_lists + list0) * a.max_budget;
   const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
   char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
 
@@ -154,7 +159,7 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
         const int within = cic % slot_chunks;
         const int h = within / row_chunks, rem = within - h * row_chunks;
         const int hh = rem / a.chunks_per_row, cc = rem - hh * a.chunks_per_row;
-        const uint32_t inner = (uint32_t)((a.shared ? 0 : h) + hh) * a.head_units + (uint32_t)cc;
+        const uint32_t inner = (uint32_t)((a.shared ? 0 : list0 + h) + hh) * a.head_units + (uint32_t)cc;
         const uint32_t su = src_units[sl * lists + h];
         dsto[c] = dst_units[sl] + inner;
         live[c] = in && su != kNoSource;
@@ -410,6 +415,11 @@ CompactArgs make_args(const CompactLaunch& a) {
   c.keep_per_layer = a.keep_per_layer;
   c.shared = a.shared;
   c.split_bulk = 1;
+  // One list per workgroup: the ordered pass is a chain of dependent tiles per workgroup, so
+  // with few sequences its run time is the chain length, and a chain over one head is
+  // Hkv times shorter than one over whole token rows; with many sequences it is bound by
+  // the memory system either way (measured: same time).
+  c.lists_per_wg = 1;
   c.chunks_per_row = a.D * a.elem_bytes / 16;
   c.heads_per_slot = a.shared ? a.Hkv : 1;
   c.streams_per_layer = 2 * (a.shared ? 1 : a.Hkv);
@@ -443,7 +453,8 @@ hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
   // Ordered pass over the slots whose sources lie inside the kept prefix, then the
   // unordered bulk pass over the rest; the first must finish reading before the second
   // writes, which stream order guarantees.
-  hipLaunchKernelGGL(compact_kernel, dim3(a.B * a.L * 2), dim3(kOrderedThreads), 0, s, c);
+  const int ordered_groups = (a.shared ? 1 : a.Hkv) / c.lists_per_wg;
+  hipLaunchKernelGGL(compact_kernel, dim3(a.B * a.L * 2 * ordered_groups), dim3(kOrderedThreads), 0, s, c);
   if (c.split_bulk) {
     hipError_t e0 = hipGetLastError();
     if (e0 != hipSuccess) return e0;
