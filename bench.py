@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument("--cpu-layers", type=int, default=36, help="layers of one sequence the CPU baseline scores")
     ap.add_argument("--seq-len", type=int, default=0,
                     help="override every sequence's cached length (e.g. budget + 128 for the steady-state step)")
+    ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
     ap.add_argument("--two-pass", action="store_true",
                     help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -105,7 +106,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     w = synth.config(args.config)
     if args.seq_len > 0:
-        w = w.scaled(name=f"{w.name}_len{args.seq_len}", seq_lens=(args.seq_len,) * w.num_seqs)
+        nseq = args.sequences if args.sequences > 0 else w.num_seqs
+        w = w.scaled(name=f"{w.name}_b{nseq}_len{args.seq_len}", seq_lens=(args.seq_len,) * nseq)
     t_setup = time.perf_counter()
     tables = synth.make_block_tables(w)
     pool = synth.make_kv_pool(w, tables, dev)
