@@ -471,6 +471,79 @@ def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
         assert ops.select_path(kv, batch, sc, sel) == want, seq_lens
 
 
+def _resident_batch(seed_index):
+    w = small(seq_lens=(3072,) * 16, num_layers=2, budget=256, index=seed_index)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    return w, inp, caches, kv, batch, sc
+
+
+def test_resident_launches_on_two_streams_do_not_starve_each_other():
+    """Each launch wants most of the CUs; issued from two streams at once they are chained on
+    the device, so both finish with a clean status and the same result as alone."""
+    sel = ops.SelectConfig(window_size=12)
+    jobs = [_resident_batch(11), _resident_batch(12)]
+    alone = []
+    for w, inp, caches, kv, batch, sc in jobs:
+        assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+        keep, fin, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+        assert ws.status() == 0
+        alone.append((keep.clone(), fin.clone()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for rep in range(3):
+        for (w, inp, caches, kv, batch, sc), st in zip(jobs, streams):
+            with torch.cuda.stream(st):
+                outs.append(ops.select_paged(kv, batch, sc, sel, want_scores=True))
+    torch.cuda.synchronize()
+    for i, (keep, fin, ws) in enumerate(outs):
+        assert ws.status() == 0
+        assert torch.equal(keep, alone[i % 2][0]) and torch.equal(fin, alone[i % 2][1])
+
+
+def test_compress_step_replays_from_a_hip_graph():
+    """The launch sequence of a step (no allocation, no synchronisation, no memset nodes)
+    captured once and replayed: every replay must equal the eager result."""
+    w = small(seq_lens=(3072,) * 16, num_layers=2, budget=256, index=13)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    pristine = [c.clone() for c in caches]
+    sel = ops.SelectConfig(window_size=12)
+    ws = ops.Workspace(kv, batch, sc)
+    keep = torch.empty(w.num_seqs * w.num_kv_heads, batch.max_budget, dtype=torch.int32, device=DEV)
+    ops.compress_step(kv, batch, sc, sel, ws, keep)
+    torch.cuda.synchronize()
+    want_keep, want_caches = keep.clone(), [c.clone() for c in caches]
+
+    def restore():
+        for c, p in zip(caches, pristine):
+            c.copy_(p)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        restore()
+        ops.compress_step(kv, batch, sc, sel, ws, keep)      # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    restore()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        ops.compress_step(kv, batch, sc, sel, ws, keep)
+    for rep in range(3):
+        restore()
+        keep.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ws.status() == 0
+        assert torch.equal(keep, want_keep), rep
+        for c, wc in zip(caches, want_caches):
+            assert torch.equal(c.view(torch.int16), wc.view(torch.int16)), rep
+
+
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
     for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=64), {}),

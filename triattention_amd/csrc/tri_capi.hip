@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "tri_common.h"
 
@@ -115,6 +116,16 @@ int check_workspace(const tri::Workspace& w, void* ws, uint64_t bytes) {
   return TRI_OK;
 }
 
+struct ResidentGate {
+  static constexpr int kMaxDevices = 64;
+  std::mutex mutex;
+  hipEvent_t event[kMaxDevices] = {};
+};
+ResidentGate& resident_gate() {
+  static ResidentGate gate;
+  return gate;
+}
+
 template <typename T>
 T* at(void* ws, int64_t off) { return reinterpret_cast<T*>(reinterpret_cast<char*>(ws) + off); }
 
@@ -207,8 +218,32 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.fin = fin ? fin : at<float>(ws, w.fin);
   a.plan = w.fused;
   a.bmat = at<char>(ws, w.bmat);
-  e = w.fused.eligible == 2 ? tri::launch_fused_mfma(a, s) : tri::launch_fused_select(a, s);
-  if (e != hipSuccess) return launch_status(e, "fused_select");
+  {
+    // Two resident launches that run at the same time on one device would each hold part of
+    // the CUs and wait for the other's workgroups until their waits expire.  Launches of this
+    // process are therefore chained: each waits (on the device, not on the host) for the
+    // previous one on whatever stream that was.  Streams under graph capture are left alone.
+    ResidentGate& gate = resident_gate();
+    std::lock_guard<std::mutex> lock(gate.mutex);
+    int dev = 0;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool chain = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < ResidentGate::kMaxDevices &&
+                       hipStreamIsCapturing(s, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone;
+    if (chain && gate.event[dev]) {
+      e = hipStreamWaitEvent(s, gate.event[dev], 0);
+      if (e != hipSuccess) return launch_status(e, "resident chain wait");
+    }
+    e = w.fused.eligible == 2 ? tri::launch_fused_mfma(a, s) : tri::launch_fused_select(a, s);
+    if (e != hipSuccess) return launch_status(e, "fused_select");
+    if (chain) {
+      if (!gate.event[dev]) {
+        e = hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming);
+        if (e != hipSuccess) return launch_status(e, "resident chain event");
+      }
+      e = hipEventRecord(gate.event[dev], s);
+      if (e != hipSuccess) return launch_status(e, "resident chain record");
+    }
+  }
   if (!keep) return TRI_OK;   // selection scores only
   return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, keep,
                                              batch->max_budget, s),
