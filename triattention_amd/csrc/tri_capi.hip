@@ -93,7 +93,9 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   const bool f_valu = force && strcmp(force, "valu") == 0;
   const bool f_mfma = force && strcmp(force, "mfma") == 0;
   const bool f_off = force && strcmp(force, "off") == 0;
-  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) && !f_valu;
+  // The matrix-core kernel addresses the 16 rows of a step with 32-bit offsets from a scalar base.
+  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) && !f_valu &&
+                         kv->stride_token > 0 && kv->stride_token < (1 << 25);
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;
   const int resident = f_off ? 0 : tri::fused_resident_workgroups();

@@ -16,8 +16,8 @@
 // The three column groups of a query head are added with row rotations, which leaves every
 // token's four scores spread over the lanes exactly as the ring in LDS wants them.
 //
-// Per 16 tokens of a head: 8 MFMAs, and vector work only for the magnitudes (about 40 %
-// of the vector-unit kernel's instruction count), so the kernel is bound by the key stream.
+// Per 16 tokens of a head: 8 MFMAs, and vector work only for the magnitudes (about a third
+// of the vector-unit kernel's instruction count), so bf16 keys run at the key stream's pace.
 // fp8 e4m3 keys are widened to bf16 (exact) in registers and take the same route; the
 // per-(token, head) scale multiplies the finished score.
 #include "tri_common.h"
@@ -56,6 +56,27 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const uint4& v) { return __builtin_b
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// m[i] = sqrt(x[i].lo^2 + x[i].hi^2) for four packed bf16 pairs, in fp32.  Written out for
+// two reasons: the compiler only selects the accumulating two-operand dot product
+// (v_dot2c_f32_bf16) and spends a v_mov per value on zeroing its destination, and it does
+// not see the opcodes inside an asm statement, so the spacing gfx950 requires between a dot
+// product's write and another vector instruction's read of that register (three
+// instructions) and after a transcendental's write (one) is provided here: four dot
+// products, then the four square roots in the same order, then one idle cycle.
+__device__ __forceinline__ void magnitudes4(const uint32_t (&x)[4], float* m) {
+  asm("v_dot2_f32_bf16 %0, %4, %4, 0\n\t"
+      "v_dot2_f32_bf16 %1, %5, %5, 0\n\t"
+      "v_dot2_f32_bf16 %2, %6, %6, 0\n\t"
+      "v_dot2_f32_bf16 %3, %7, %7, 0\n\t"
+      "v_sqrt_f32 %0, %0\n\t"
+      "v_sqrt_f32 %1, %1\n\t"
+      "v_sqrt_f32 %2, %2\n\t"
+      "v_sqrt_f32 %3, %3\n\t"
+      "s_nop 0"
+      : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(m[3])
+      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+}
 
 // Two fp32 values -> packed bf16 (round to nearest even) and the fp32 remainders.
 __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, float& r1) {
@@ -117,8 +138,9 @@ __global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int Q
 }
 
 // QG: groups of four query heads per KV head (1 or 2).
-template <int DT, bool IL, int TW, int SL, int QG>
+template <int DT, bool IL, int TW, int SL, int QG, int NB>
 __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
+  static_assert(SL % (16 * NB) == 0, "the slack must hold whole rotations of the step buffers");
   constexpr int RING = TW + SL;
   constexpr int RQ = 4 * QG;                                   // ring floats per token
   extern __shared__ __align__(16) float lds[];
@@ -142,17 +164,8 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   float* part = lds + kFusedWaves * (RING * RQ);               // [waves][64][QG][2]
   float* stats = part + kFusedWaves * 128 * QG;                // [2][32*QG score heads][2]
   uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128 * QG);  // arrive count, claimed, ready
-  int* lds_blk = reinterpret_cast<int*>(ctl + 8);
-
   for (int i = threadIdx.x; i < kFusedWaves * 128 * QG; i += kFusedThreads) part[i] = 0.f;
   if (threadIdx.x < 8) ctl[threadIdx.x] = 0;
-  int lb0 = 0;
-  if (a.block_table_pitch >= 0) {
-    lb0 = n0 >> a.bs_shift;
-    const int lb1 = last_tok >> a.bs_shift;
-    for (int i = threadIdx.x; i <= lb1 - lb0; i += kFusedThreads)
-      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
-  }
   __syncthreads();
   // From here on the waves of the workgroup run independently.
   if (wave >= heads_here) return;
@@ -171,108 +184,121 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       for (int o = 0; o < 6; ++o) B[g][o] = p[(g * 6 + o) * 64];
   };
 
-  // Element offset of this lane inside a (token, head) row and of its head inside a token.
-  const int64_t lane_elems = (int64_t)head * a.stride_head + kb * (DT == TRI_KV_FP8_E4M3 ? 16 : 8);
+  // A step is 16 consecutive tokens starting at a multiple of 16, so with blocks of at
+  // least 16 tokens it lies inside one block: lane i keeps the block of step i of the tile
+  // (a tile has at most 64 steps), and a step's block is one v_readlane away.  Dense keys:
+  // the "block" is the sequence.
+  const bool paged = a.block_table_pitch >= 0;
+  int step_blk = b;
+  if (paged) {
+    const int n = min(n0 + 16 * lane, last_tok);
+    step_blk = a.block_table[(int64_t)b * a.block_table_pitch + (n >> a.bs_shift)];
+  }
+  const int bs_mask = paged ? (1 << a.bs_shift) - 1 : -1;
 
-  // Sixteen tokens of layer l starting at local token t (t % 16 == 0): lane's token is
-  // t + lane % 16, clamped to the tile's last token (loaded, never stored).
+  // Sixteen tokens of layer l starting at local token t (t % 16 == 0).  The address splits
+  // into a wave-uniform base (layer, block, first token of the step, head: scalar unit) and
+  // a 32-bit lane offset (row lane % 16 of the step, 16-byte chunk lane / 16); rows past the
+  // tile's last token re-read that token (loaded, never stored).
   constexpr bool FP8 = DT == TRI_KV_FP8_E4M3;
   constexpr int ES = FP8 ? 1 : 2;
-  auto load_step = [&](StepData<DT>& d, int l, int t) __attribute__((always_inline)) {
-    const char* kbase = table_entry(a.k_layers, l);
-    const int n = min(n0 + t + j, last_tok);
-    int64_t row;
-    if (a.block_table_pitch < 0) {
-      row = (int64_t)b * a.stride_block + (int64_t)n * a.stride_token;
-    } else {
-      const int lb = n >> a.bs_shift;
-      row = (int64_t)lds_blk[lb - lb0] * a.stride_block + (int64_t)(n - (lb << a.bs_shift)) * a.stride_token;
-    }
-    GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + (row + lane_elems) * ES;
+  const uint32_t tok_bytes = (uint32_t)(a.stride_token * ES);
+  const uint32_t lane_row = (uint32_t)j * tok_bytes;
+  const uint32_t lane_col = (uint32_t)kb * 16u;
+  const uint32_t lane_scale_row = (uint32_t)(4 * kb + rsel) * (uint32_t)a.Hkv * 4u;   // fp8: token this lane stores
+  struct LayerBase { const char* k; const char* scale; };   // of this wave's head (scalar registers)
+  auto layer_base = [&](int l) __attribute__((always_inline)) {
+    LayerBase lb;
+    lb.k = table_entry(a.k_layers, l) + (int64_t)head * a.stride_head * ES;
+    lb.scale = nullptr;
+    if constexpr (FP8)
+      lb.scale = table_entry(reinterpret_cast<const void* const*>(a.k_scale_layers), l) + head * 4;
+    return lb;
+  };
+  auto load_step = [&](StepData<DT>& d, const LayerBase& lb, int t) __attribute__((always_inline)) {
+    const int blk = __builtin_amdgcn_readlane(step_blk, t >> 4);
+    const int nt = n0 + t;
+    const int in_blk = nt & bs_mask;
+    const uint32_t rows_left = (uint32_t)(last_tok - nt);
+    const int64_t row0 = (int64_t)blk * a.stride_block + (int64_t)in_blk * a.stride_token;
+    const char* base = reinterpret_cast<const char*>(uniform_ptr(lb.k + row0 * ES));
+    const uint32_t off = min(lane_row, rows_left * tok_bytes) + lane_col;
+    GlobalBytes p = (GlobalBytes)(uintptr_t)base + off;
     d.scale = 1.f;
+#pragma unroll
+    for (int s = 0; s < (FP8 ? 2 : 4); ++s) {
+      const u32x4 v = *(GlobalU4)(p + s * 64);
+      d.c[s] = uint4{v.x, v.y, v.z, v.w};
+    }
     if constexpr (FP8) {
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const u32x4 v = *(GlobalU4)(p + s * 64);
-        d.c[s] = uint4{v.x, v.y, v.z, v.w};
-      }
-      // scale of the token this lane stores: local token t + 4*kb + rsel
-      const int ns = min(n0 + t + 4 * kb + rsel, last_tok);
-      int64_t slot;
-      if (a.block_table_pitch < 0) {
-        slot = (int64_t)b * a.block_size + ns;
-      } else {
-        const int lb = ns >> a.bs_shift;
-        slot = (int64_t)lds_blk[lb - lb0] * a.block_size + (ns - (lb << a.bs_shift));
-      }
-      const float* sc = reinterpret_cast<const float*>(
-          table_entry(reinterpret_cast<const void* const*>(a.k_scale_layers), l));
-      d.scale = ((GlobalF32)(uintptr_t)sc)[slot * a.Hkv + head];
-    } else {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4 v = *(GlobalU4)(p + s * 64);
-        d.c[s] = uint4{v.x, v.y, v.z, v.w};
-      }
+      const int64_t slot0 = (int64_t)blk * a.block_size + in_blk;
+      const char* sc = reinterpret_cast<const char*>(uniform_ptr(lb.scale + slot0 * a.Hkv * 4));
+      const uint32_t soff = min(lane_scale_row, rows_left * (uint32_t)a.Hkv * 4u);
+      d.scale = *(GlobalF32)((GlobalBytes)(uintptr_t)sc + soff);
     }
   };
 
+  const uint32_t lane_ring = (uint32_t)(4 * kb + rsel) * RQ + q;
   float s1[QG], s2[QG];
 #pragma unroll
   for (int g = 0; g < QG; ++g) { s1[g] = 0.f; s2[g] = 0.f; }
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
   auto compute_step = [&](const StepData<DT>& raw, int l, int t) __attribute__((always_inline)) {
-    // The four bf16 A operands of the step and the fp32 values of their elements (for the
-    // magnitudes): fp8 keys are widened once and both come out of that, bf16 keys are the
-    // loaded registers and the fp32 values are unpacked from them.
-    struct { uint4 c[4]; } d;
-    float fe[4][8];
+    // The four bf16 A operands of the step as dwords (two elements each): the loaded
+    // registers for bf16 keys, one conversion per dword (exact) for fp8 keys.
+    uint32_t w[4][4];
     if constexpr (FP8) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const uint32_t w[4] = {raw.c[s].x, raw.c[s].y, raw.c[s].z, raw.c[s].w};
+        const uint32_t r[4] = {raw.c[s].x, raw.c[s].y, raw.c[s].z, raw.c[s].w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
-          const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
-          float* f = &fe[2 * s + (i >> 1)][(i & 1) * 4];
-          f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
-          uint32_t* o = &(&d.c[2 * s + (i >> 1)].x)[(i & 1) * 2];
-          o[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
-          o[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+          uint32_t* o = &w[2 * s + (i >> 1)][(i & 1) * 2];
+          o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r[i], 1.0f, false));
+          o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(r[i], 1.0f, true));
         }
       }
     } else {
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        d.c[s] = raw.c[s];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint32_t w = (&raw.c[s].x)[e >> 1];
-          fe[s][e] = (e & 1) ? bf16_hi(w) : bf16_lo(w);
-        }
+        w[s][0] = raw.c[s].x; w[s][1] = raw.c[s].y; w[s][2] = raw.c[s].z; w[s][3] = raw.c[s].w;
       }
     }
+    struct { uint4 c[4]; } d;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) d.c[s] = uint4{w[s][0], w[s][1], w[s][2], w[s][3]};
     f32x4 acc[QG], acc_e[QG];
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-      acc_e[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s)
         acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(d.c[s]), as_bf16x8(B[g][s]), acc[g], 0, 0, 0);
+      acc_e[g] = acc[g];   // the magnitude MFMAs continue the sum (the key MFMAs are long done by then)
     }
 #pragma unroll
     for (int set = 0; set < 2; ++set) {
+      // |k_f|^2 = k_r^2 + k_i^2 straight from the bf16 pairs (v_dot2_f32_bf16).
+      // interleaved: dword e % 4 of operand 2*set + e/4 is the (real, imaginary) pair;
+      // half: real parts in operand `set`, imaginary parts in operand `set + 2`, regrouped
+      // into (real, imaginary) dwords by two byte permutes per dword.
       float mag[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        // interleaved: operands 2*set and 2*set + 1 hold four (real, imaginary) pairs each;
-        // half: real parts in operand `set`, imaginary parts in operand `set + 2`
-        const float kr = IL ? fe[2 * set + (e >> 2)][2 * (e & 3)] : fe[set][e];
-        const float ki = IL ? fe[2 * set + (e >> 2)][2 * (e & 3) + 1] : fe[set + 2][e];
-        mag[e] = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
+      for (int h = 0; h < 2; ++h) {
+        uint32_t x[4];
+        if constexpr (IL) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[i] = w[2 * set + h][i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const uint32_t re = w[set][2 * h + i], im = w[set + 2][2 * h + i];
+            x[2 * i] = __builtin_amdgcn_perm(im, re, 0x05040100u);
+            x[2 * i + 1] = __builtin_amdgcn_perm(im, re, 0x07060302u);
+          }
+        }
+        magnitudes4(x, &mag[4 * h]);
       }
       uint4 hi, lo;
       float r[8];
@@ -292,19 +318,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       }
     }
     const int tl = t + 4 * kb + rsel;
+    // first ring slot of the step (scalar; a step never straddles the wrap: t and RING are
+    // multiples of 16)
+    const uint32_t slot0 = (uint32_t)(l * TW + t) % RING;
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       float v = 0.f;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float x = acc[g][r] + acc_e[g][r];
+        float x = acc_e[g][r];
         x += dpp<kDppRor8m>(x);
         x += dpp<kDppRor4>(x);
         v = (rsel == r) ? x : v;
       }
       if (FP8) v *= raw.scale;
       if (4 * g + q < a.G && tl < ntok) {
-        ring[((uint32_t)(l * TW + tl) % RING) * RQ + 4 * g + q] = v;
+        ring[slot0 * RQ + lane_ring + 4 * g] = v;
         s1[g] += v;
         s2[g] = fmaf(v, v, s2[g]);
       }
@@ -414,45 +443,41 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     }
   };
 
-  // ---- one continuous stream of key rows over (layer, step of 16 tokens).  Four step
-  // buffers rotate; a buffer is refilled as soon as it has been scored.  A layer is padded to
-  // whole rotations (padding steps re-read the last row and are not scored); the rotations
-  // form inner loops that contain nothing but key loads and scoring, and the work at layer
-  // boundaries sits between them.
+  // ---- one continuous stream of key rows over (layer, step of 16 tokens).  NB step
+  // buffers rotate (four of 64 bytes per lane, or eight of 36 for one-byte keys, which keeps
+  // the same number of bytes in flight); a buffer is refilled as soon as it has been scored,
+  // with the step NB ahead.  A layer is padded to whole rotations (padding steps re-read the
+  // last row and are not scored), so the loads of a layer's last rotation are exactly the
+  // first NB steps of the next layer; the rotations form inner loops that contain nothing
+  // but key loads and scoring, and the work at layer boundaries sits between them.
   const int nsteps = (ntok + 15) >> 4;
-  const int rotations = (nsteps + 3) >> 2;
-  const int rot_before_consume = min(SL / 64, rotations);
-  int ld_l = 0, ld_slot = 0;
-  auto fetch = [&](StepData<DT>& d) __attribute__((always_inline)) {
-    const int l = __builtin_amdgcn_readfirstlane(min(ld_l, a.L - 1));
-    const int t = __builtin_amdgcn_readfirstlane(min(ld_slot, nsteps - 1) * 16);
-    load_step(d, l, t);
-    if (++ld_slot >= rotations * 4) { ld_slot = 0; ++ld_l; }
-  };
+  const int rotations = (nsteps + NB - 1) / NB;
+  const int rot_before_consume = min(SL / (16 * NB), rotations);
   auto score = [&](const StepData<DT>& d, int l, int slot) __attribute__((always_inline)) {
     if (slot < nsteps) compute_step(d, l, slot * 16);
   };
-  StepData<DT> buf0, buf1, buf2, buf3;
+  StepData<DT> buf[NB];
+  LayerBase base_cur = layer_base(0), base_next = base_cur;
   auto rotate = [&](int l, int r0, int r1) __attribute__((always_inline)) {
     for (int r = r0; r < r1; ++r) {
-      score(buf0, l, r * 4 + 0);
-      fetch(buf0);
-      score(buf1, l, r * 4 + 1);
-      fetch(buf1);
-      score(buf2, l, r * 4 + 2);
-      fetch(buf2);
-      score(buf3, l, r * 4 + 3);
-      fetch(buf3);
+      const bool wrap = r + 1 >= rotations;
+      const LayerBase lb = {wrap ? base_next.k : base_cur.k, wrap ? base_next.scale : base_cur.scale};
+      const int s0 = wrap ? 0 : (r + 1) * NB;
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        score(buf[i], l, r * NB + i);
+        load_step(buf[i], lb, min(s0 + i, nsteps - 1) * 16);
+      }
     }
   };
   auto settle = [&]() __attribute__((always_inline)) { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
   load_coefs(0);
-  fetch(buf0);
-  fetch(buf1);
-  fetch(buf2);
-  fetch(buf3);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) load_step(buf[i], base_cur, min(i, nsteps - 1) * 16);
   for (int l = 0; l < a.L; ++l) {
+    base_cur = base_next;
+    base_next = layer_base(min(l + 1, a.L - 1));
     settle();
     rotate(l, 0, rot_before_consume);
     if (l > 0) consume(l - 1);
@@ -471,23 +496,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 }
 
 template <int TW, int SL, int QG>
-size_t mfma_lds_bytes(int tile_tokens, int bs_shift, bool paged) {
-  const int blocks = paged ? (tile_tokens >> bs_shift) + 2 : 0;
-  return ((size_t)kFusedWaves * (TW + SL) * 4 * QG + kFusedWaves * 128 * QG + 128 * QG + 8 + blocks) * 4;
+size_t mfma_lds_bytes() {
+  return ((size_t)kFusedWaves * (TW + SL) * 4 * QG + kFusedWaves * 128 * QG + 128 * QG + 8) * 4;
 }
 
-template <int DT, bool IL, int TW, int SL, int QG>
+template <int DT, bool IL, int TW, int SL, int QG, int NB>
 hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
-  const size_t lds = mfma_lds_bytes<TW, SL, QG>(k.tile_tokens, k.bs_shift, k.block_table_pitch >= 0);
+  const size_t lds = mfma_lds_bytes<TW, SL, QG>();
   if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
-  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG>);
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG, NB>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   if (B <= seqs_per_launch) {
     k.packed = 0;
     k.seq_base = 0;
     const int n = B;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads), lds, s, k, bmat);
     return hipGetLastError();
   }
   // More workgroups than the device holds at once: whole sequences are packed into
@@ -501,7 +525,7 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
   const int launches = ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG>), dim3(resident), dim3(kFusedThreads), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB>), dim3(resident), dim3(kFusedThreads), lds, s, k, bmat);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -512,15 +536,18 @@ template <int DT, bool IL>
 hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int resident, int B, hipStream_t s) {
   if (k.G > 4) {
     switch (tw) {   // eight query heads per KV head: 32 bytes of ring per token
-      case 512: return launch_mfma_t<DT, IL, 512, 64, 2>(k, bmat, seqs_per_launch, resident, B, s);
-      case 256: return launch_mfma_t<DT, IL, 256, 64, 2>(k, bmat, seqs_per_launch, resident, B, s);
+      case 512: return launch_mfma_t<DT, IL, 512, 64, 2, 4>(k, bmat, seqs_per_launch, resident, B, s);
+      case 256: return launch_mfma_t<DT, IL, 256, 64, 2, 4>(k, bmat, seqs_per_launch, resident, B, s);
       default: return hipErrorInvalidValue;
     }
   }
+  // One-byte keys: eight step buffers and a slack of 128 tokens (the ring still fits).
+  constexpr int NB = DT == TRI_KV_FP8_E4M3 ? 8 : 4;
+  constexpr int SL = 16 * NB;
   switch (tw) {
-    case 1024: return launch_mfma_t<DT, IL, 1024, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
-    case 512: return launch_mfma_t<DT, IL, 512, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
-    case 256: return launch_mfma_t<DT, IL, 256, 64, 1>(k, bmat, seqs_per_launch, resident, B, s);
+    case 1024: return launch_mfma_t<DT, IL, 1024, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
+    case 512: return launch_mfma_t<DT, IL, 512, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
+    case 256: return launch_mfma_t<DT, IL, 256, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -535,7 +562,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   int bs_shift = -1;
   for (int sft = 0; sft < 31; ++sft)
     if ((1 << sft) == block_size) bs_shift = sft;
-  if (paged && bs_shift < 0) return p;
+  if (paged && bs_shift < 4) return p;    // a 16-token step must lie inside one block
   const int HC = ceil_div(Hkv, 8);
   const int tws[3] = {256, 512, 1024};
   const int ntw = G > 4 ? 2 : 3;          // the ring of a 1024-token tile fits LDS for four query heads only
