@@ -273,16 +273,17 @@ def test_topk_rows_ties_and_order():
             assert torch.equal(got[r, :kk], osel.topk_ascending(x[r:r + 1, :n], kk)[0])
 
 
-def _compact_case(w, kv_axis, shared, per_layer, full):
+def _compact_case(w, kv_axis, shared, per_layer, full, budgets=None):
     inp = build_inputs(w, kv_axis)
     caches = [c.to(DEV) for c in inp["caches"]]
     kv = ops.PagedKV.from_kv_caches(caches, kv_axis=kv_axis)
-    batch = ops.StepBatch(DEV, w.seq_lens, budgets=w.budget, block_tables=inp["tables"])
+    budgets = list(budgets) if budgets is not None else [w.budget] * w.num_seqs
+    batch = ops.StepBatch(DEV, w.seq_lens, budgets=budgets, block_tables=inp["tables"])
     g = torch.Generator().manual_seed(99)
     rows_per = (w.num_layers if per_layer else 1) * (1 if shared else w.num_kv_heads)
     keep = torch.zeros(w.num_seqs * rows_per, batch.max_budget, dtype=torch.int32)
     for b, t in enumerate(w.seq_lens):
-        k = min(w.budget, t)
+        k = min(budgets[b], t)
         for r in range(rows_per):
             keep[b * rows_per + r, :k] = torch.sort(torch.randperm(t, generator=g)[:k]).values.int()
     before = [c.clone() for c in inp["caches"]]
@@ -291,7 +292,7 @@ def _compact_case(w, kv_axis, shared, per_layer, full):
     for l in range(w.num_layers):
         want = before[l].clone()
         for b, t in enumerate(w.seq_lens):
-            k = min(w.budget, t)
+            k = min(budgets[b], t)
             base = b * rows_per + (l * (1 if shared else w.num_kv_heads) if per_layer else 0)
             if shared:
                 ocp.compact_shared(want, inp["tables"][b], w.block_size, keep[base, :k].long(), t,
@@ -318,6 +319,19 @@ def test_compaction_large_budget_and_dims():
     _compact_case(small(seq_lens=(5000,), budget=3000, num_kv_heads=8, num_q_heads=8), 0, False, False, False)
     _compact_case(small(seq_lens=(700,), budget=300, head_dim=64, block_size=32), 0, False, False, False)
     _compact_case(small(seq_lens=(700,), budget=300, head_dim=256, block_size=8), 0, True, False, False)
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_compaction_when_few_tokens_are_dropped_and_budgets_differ(shared):
+    """The rows that come from beyond the budget are a short suffix of every keep list when a
+    step drops few tokens; the copy of that suffix is launched with few workgroups.  Also a
+    batch in which one sequence's own budget is far below the largest one, so its suffix is
+    longer than the launch was sized for."""
+    kw = dict(num_layers=2, num_q_heads=8, num_kv_heads=4)
+    print(f"compact few drops shared={shared}", flush=True)
+    _compact_case(small(seq_lens=(1128, 1000, 1064), budget=1000, **kw), 0, shared, False, False)
+    _compact_case(small(seq_lens=(1100, 1100, 1100), **kw), 0, shared, False, False, budgets=[1000, 500, 37])
+    _compact_case(small(seq_lens=(2176,), budget=2048, num_layers=1, num_q_heads=8, num_kv_heads=8), 1, shared, False, False)
 
 
 @pytest.mark.parametrize("axis", [0, 1])

@@ -9,6 +9,7 @@
 // of the cache is needed.  The reference gathers all T rows of K and V into
 // temporaries and scatters them back (runtime/kv_compaction.py:529-546).
 #include "tri_common.h"
+#include <cstdlib>
 
 namespace tri {
 namespace {
@@ -208,6 +209,12 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
 // Slots whose source token lies at or beyond the budget: sources (>= k) and
 // destinations (< k) cannot overlap, so this is a flat gather copy.  One workgroup
 // moves a tile of destination slots for all heads, i.e. whole contiguous token rows.
+// With keep ascending these slots are a suffix of every list, at most T - k long, so the
+// tiles are counted from the end of the lists and a workgroup stops at the first tile in
+// which no list has such a slot: when a step drops few tokens (T = k + 128) only a few
+// tiles per (sequence, layer) do anything, and the host sizes the grid for that
+// (workgroups stride over the tiles, so a grid smaller than the number of tiles is
+// still complete).
 __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactArgs a) {
   int sidx = blockIdx.y;
   const int kv = sidx % 2; sidx /= 2;
@@ -216,50 +223,58 @@ __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactAr
   int k = a.budgets[b];
   const int T = a.seq_lens[b];
   if (k > T) k = T;
+  if (k <= 0) return;
   const int lists = a.shared ? 1 : a.Hkv;
   const int chunks_per_entry = a.heads_per_slot * a.chunks_per_row;
   const int slots_per_tile = max(kTileChunks / (lists * chunks_per_entry), 1);
-  const int j0 = blockIdx.x * slots_per_tile;
-  if (j0 >= k) return;
   const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * lists * a.max_budget;
   const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
   char* base = reinterpret_cast<char*>(const_cast<void*>(kv ? a.v_layers[l] : a.k_layers[l]));
-  const int nchunks = min(slots_per_tile, k - j0) * lists * chunks_per_entry;
+  const int tiles = ceil_div(k, slots_per_tile);
 
-  // Three dependent lookups per chunk (keep -> block table -> row).  Each level is
-  // issued for all of a thread's chunks before the next one, without branches: idle
-  // chunks are clamped onto valid entries and only their final store is masked.
-  for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
-    bool live[kChunksPerThread];
-    int jj[kChunksPerThread], src[kChunksPerThread];
-    uint32_t inner[kChunksPerThread];
+  for (int t = blockIdx.x; t < tiles; t += gridDim.x) {
+    const int j1 = k - t * slots_per_tile;              // tile t from the end: slots [j0, j1)
+    const int j0 = max(j1 - slots_per_tile, 0);
+    bool any = false;
+    for (int h = 0; h < lists; ++h) any = any || keep[(int64_t)h * a.max_budget + j1 - 1] >= k;
+    if (!any) break;                                    // nor has any tile below this one
+    const int nchunks = (j1 - j0) * lists * chunks_per_entry;
+
+    // Three dependent lookups per chunk (keep -> block table -> row).  Each level is
+    // issued for all of a thread's chunks before the next one, without branches: idle
+    // chunks are clamped onto valid entries and only their final store is masked.
+    for (int c0 = 0; c0 < nchunks; c0 += kTileChunks) {
+      bool live[kChunksPerThread];
+      int jj[kChunksPerThread], src[kChunksPerThread];
+      uint32_t inner[kChunksPerThread];
 #pragma unroll
-    for (int c = 0; c < kChunksPerThread; ++c) {
-      const int ci = c0 + c * kCompactThreads + threadIdx.x;
-      live[c] = ci < nchunks;
-      const int cic = live[c] ? ci : 0;
-      const int e = cic / chunks_per_entry, within = cic % chunks_per_entry;
-      const int h = e % lists;
-      jj[c] = j0 + e / lists;
-      const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
-      inner[c] = (uint32_t)((a.shared ? 0 : h) + hh) * a.head_units + (uint32_t)cc;
-      src[c] = keep[(int64_t)h * a.max_budget + jj[c]];
+      for (int c = 0; c < kChunksPerThread; ++c) {
+        const int ci = c0 + c * kCompactThreads + threadIdx.x;
+        live[c] = ci < nchunks;
+        const int cic = live[c] ? ci : 0;
+        const int e = cic / chunks_per_entry, within = cic % chunks_per_entry;
+        const int h = e % lists;
+        jj[c] = j0 + e / lists;
+        const int hh = within / a.chunks_per_row, cc = within % a.chunks_per_row;
+        inner[c] = (uint32_t)((a.shared ? 0 : h) + hh) * a.head_units + (uint32_t)cc;
+        src[c] = keep[(int64_t)h * a.max_budget + jj[c]];
+      }
+      uint32_t so[kChunksPerThread], dsto[kChunksPerThread];
+#pragma unroll
+      for (int c = 0; c < kChunksPerThread; ++c) {
+        live[c] = live[c] && src[c] >= k;
+        const int sc = live[c] ? src[c] : j0;              // idle chunk: re-read one row of the tile (cache hit)
+        so[c] = slot_units(a, bt, sc) + inner[c];
+        dsto[c] = slot_units(a, bt, jj[c]) + inner[c];
+      }
+      uint4 regs[kChunksPerThread];
+#pragma unroll
+      for (int c = 0; c < kChunksPerThread; ++c)
+        regs[c] = load_chunk(base + ((uint64_t)so[c] << 4));
+#pragma unroll
+      for (int c = 0; c < kChunksPerThread; ++c)
+        if (live[c]) store_chunk(base + ((uint64_t)dsto[c] << 4), regs[c]);
     }
-    uint32_t so[kChunksPerThread], dsto[kChunksPerThread];
-#pragma unroll
-    for (int c = 0; c < kChunksPerThread; ++c) {
-      live[c] = live[c] && src[c] >= k;
-      const int sc = live[c] ? src[c] : j0;              // idle chunk: re-read one row of the tile (cache hit)
-      so[c] = slot_units(a, bt, sc) + inner[c];
-      dsto[c] = slot_units(a, bt, jj[c]) + inner[c];
-    }
-    uint4 regs[kChunksPerThread];
-#pragma unroll
-    for (int c = 0; c < kChunksPerThread; ++c)
-      regs[c] = load_chunk(base + ((uint64_t)so[c] << 4));
-#pragma unroll
-    for (int c = 0; c < kChunksPerThread; ++c)
-      if (live[c]) store_chunk(base + ((uint64_t)dsto[c] << 4), regs[c]);
   }
 }
 
@@ -459,8 +474,14 @@ hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
     hipError_t e0 = hipGetLastError();
     if (e0 != hipSuccess) return e0;
     const int lists = a.shared ? 1 : a.Hkv;
-    const int slots_per_tile = kTileChunks / (lists * c.heads_per_slot * c.chunks_per_row);
-    dim3 grid(ceil_div(a.max_budget, slots_per_tile > 0 ? slots_per_tile : 1), a.B * a.L * 2);
+    const int slots_per_tile = max(kTileChunks / (lists * c.heads_per_slot * c.chunks_per_row), 1);
+    // At most T - k slots of a list take their row from beyond the budget; one more tile
+    // for the misalignment of that suffix against the tile grid.  (A sequence whose own
+    // budget is smaller than max_budget may have a longer suffix: its workgroups take
+    // several tiles each.)
+    const int suffix = max(a.Tmax - a.max_budget, 0);
+    const int tiles = min(ceil_div(suffix, slots_per_tile) + 1, ceil_div(a.max_budget, slots_per_tile));
+    dim3 grid(max(tiles, 1), a.B * a.L * 2);
     hipLaunchKernelGGL(compact_bulk_kernel, grid, dim3(kCompactThreads), 0, s, c);
   }
   hipError_t e = hipGetLastError();
