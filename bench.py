@@ -49,6 +49,9 @@ def parse_args():
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
     ap.add_argument("--two-pass", action="store_true",
                     help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
+    ap.add_argument("--hook-latency", action="store_true",
+                    help="also time the runner hook (triattention_apply_compression) for one request of "
+                         "budget + 128 tokens, host side included")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (reference point for HBM byte counters)")
     return ap.parse_args()
@@ -88,6 +91,62 @@ def cpu_baseline(w, layers: int):
     return {"value": keys_per_s, "unit": "keys/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"1 sequence x {t} tokens x {layers} of {w.num_layers} layers, {dt:.2f} s on the host; "
                       f"rate scaled to all {w.num_layers} layers"}
+
+
+def hook_latency(w, dev, calls: int = 30):
+    """Wall time of one call of the runner hook for a single request of budget + 128 tokens
+    (the steady state of a long generation): host logic, launches and the two host reads of
+    the keep-index check, synchronised before and after."""
+    import tempfile
+    import types
+    from triattention_amd import synth
+    from triattention_amd.runtime import CompressionSignal, TriAttentionRuntimeConfig, install_runner_compression_hook
+
+    t = w.budget + 128
+    qc, qa = synth.make_stats(w)
+    entries = {f"layer{l:02d}_head{h:02d}": {"q_mean_real": qc[l, h, :, 0].clone(), "q_mean_imag": qc[l, h, :, 1].clone(),
+                                            "q_abs_mean": qa[l, h].clone()}
+               for l in range(w.num_layers) for h in range(w.num_q_heads)}
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "stats.pt")
+        torch.save({"metadata": {"head_dim": w.head_dim, "rope_style": w.rope_style,
+                                 "inv_freq": synth.rope_inv_freq(w).clone(),
+                                 "sampled_heads": [[l, h] for l in range(w.num_layers) for h in range(w.num_q_heads)]},
+                    "stats": entries}, path)
+        cfg = TriAttentionRuntimeConfig(kv_budget=w.budget, divide_length=128, window_size=w.window_size,
+                                        sparse_stats_path=path, log_decisions=False)
+        nblk = (t + w.block_size - 1) // w.block_size + 8
+        ids = torch.randperm(nblk + 64, generator=torch.Generator().manual_seed(1))[:nblk].tolist()
+        caches = [torch.randn(2, nblk + 64, w.block_size, w.num_kv_heads, w.head_dim, device=dev).to(torch.bfloat16)
+                  for _ in range(w.num_layers)]
+        req = types.SimpleNamespace(num_computed_tokens=t, block_ids=(list(ids),))
+        runner = types.SimpleNamespace(requests={"r": req}, kv_caches=caches,
+                                       cache_config=types.SimpleNamespace(block_size=w.block_size))
+        install_runner_compression_hook(runner, cfg)
+        sched = types.SimpleNamespace(num_scheduled_tokens={"r": 1})
+
+        def call():
+            req.num_computed_tokens = t
+            req.block_ids = (list(ids),)
+            sig = CompressionSignal(req_id="r", should_compress=True, reason="length_threshold",
+                                    estimated_cache_len=t + 1, step=1, kv_usage=None, protect_prefill=False,
+                                    prefill_len=0, scheduled_tokens=1)
+            return runner.triattention_apply_compression(req_id="r", signal=sig, scheduler_output=sched)
+
+        for _ in range(3):
+            res = call()
+        if not res["applied"]:
+            raise RuntimeError(f"hook did not compress: {res}")
+        times = []
+        for _ in range(calls):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            call()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+    times.sort()
+    return {"tokens": t, "budget": w.budget, "layers": w.num_layers, "calls": calls,
+            "ms_median": times[len(times) // 2], "ms_min": times[0], "ms_max": times[-1]}
 
 
 def main() -> int:
@@ -261,6 +320,8 @@ def main() -> int:
         torch.cuda.synchronize()
         out["copy_calibration_bytes"] = 1 << 30
         del src, dst
+    if args.hook_latency and w.kv_dtype != "fp8":
+        out["hook_call"] = hook_latency(w, dev)
     if not args.no_cpu_baseline:
         del saved, caches, pool
         torch.cuda.empty_cache()

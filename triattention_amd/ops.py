@@ -111,6 +111,31 @@ class PagedKV:
         ks, vs = zip(*(split_kv_axes(t, kv_axis) for t in kv_caches))
         return cls(ks, vs, rope_style)
 
+    _recent: "dict[tuple, PagedKV]" = {}
+
+    @classmethod
+    def for_kv_caches(cls, kv_caches: Sequence[torch.Tensor], rope_style: str = "half",
+                      kv_axis: int | None = None) -> "PagedKV":
+        """``from_kv_caches`` for callers that come back with the same cache tensors on every
+        call (a serving loop): the description of a set of layer tensors, pointer tables on
+        the device included, is built once per (addresses, geometry) and reused.  The cached
+        object holds no reference to the cache tensors; it is only ever handed to a caller
+        who holds tensors of that geometry at those addresses."""
+        c0 = kv_caches[0]
+        key = (tuple(int(t.data_ptr()) for t in kv_caches), tuple(c0.shape), tuple(c0.stride()), c0.dtype,
+               str(c0.device), rope_style, kv_axis)
+        hit = cls._recent.get(key)
+        if hit is None:
+            for t in kv_caches:
+                if t.shape != c0.shape or t.stride() != c0.stride() or t.dtype != c0.dtype:
+                    raise ValueError("all layers must share shape, strides, dtype and device")
+            hit = cls.from_kv_caches(kv_caches, rope_style, kv_axis)
+            hit._keep = None
+            if len(cls._recent) >= 16:
+                cls._recent.pop(next(iter(cls._recent)))
+            cls._recent[key] = hit
+        return hit
+
     @classmethod
     def from_dense_keys(cls, key_states: torch.Tensor, rope_style: str = "half") -> "PagedKV":
         """[B, H, T, D] keys as one 'block' per sequence (score-only)."""
@@ -130,31 +155,51 @@ class StepBatch:
         self.num_seqs = len(self.seq_lens_host)
         if self.num_seqs == 0:
             raise ValueError("empty batch")
-        self.seq_lens = _i32(self.seq_lens_host, device)
-        self.round_start = _i32(round_start if round_start is not None else self.seq_lens_host, device)
-        self.prefill_lens = _i32(prefill_lens, device) if prefill_lens is not None else None
+        n = self.num_seqs
+
+        def host_list(values, what):
+            if values is None:
+                return None
+            v = values.tolist() if isinstance(values, torch.Tensor) else values
+            if isinstance(v, int):
+                v = [v] * n
+            v = [int(x) for x in v]
+            if len(v) != n:
+                raise ValueError(f"{what} has {len(v)} entries for {n} sequences")
+            return v
+
+        rs = host_list(round_start, "round_start") or self.seq_lens_host
+        pf = host_list(prefill_lens, "prefill_lens")
         self.budgets_host = None
-        self.budgets = None
-        if budgets is not None:
-            b = budgets.tolist() if isinstance(budgets, torch.Tensor) else budgets
-            if isinstance(b, int):
-                b = [b] * self.num_seqs
-            self.budgets_host = [min(int(x), t) for x, t in zip(b, self.seq_lens_host)]
-            self.budgets = _i32(self.budgets_host, device)
+        bud = host_list(budgets, "budgets")
+        if bud is not None:
+            self.budgets_host = [min(x, t) for x, t in zip(bud, self.seq_lens_host)]
+        rows, pitch = None, 0
+        if block_tables is not None and not isinstance(block_tables, torch.Tensor):
+            if len(block_tables) != n:
+                raise ValueError("block table rows != number of sequences")
+            pitch = max(len(r) for r in block_tables)
+            rows = [int(x) for r in block_tables for x in (list(r) + [0] * (pitch - len(r)))]
+        # One host-to-device copy for all the small integer arrays of the step.
+        parts = [self.seq_lens_host, rs, pf or [], self.budgets_host or [], rows or []]
+        flat = torch.tensor([x for part in parts for x in part], dtype=torch.int32, device=device)
+        cuts, pos = [], 0
+        for part in parts:
+            cuts.append(flat[pos:pos + len(part)])
+            pos += len(part)
+        self.seq_lens, self.round_start = cuts[0], cuts[1]
+        self.prefill_lens = cuts[2] if pf is not None else None
+        self.budgets = cuts[3] if self.budgets_host is not None else None
         self.block_table = None
-        pitch = 0
-        if block_tables is not None:
-            if isinstance(block_tables, torch.Tensor):
-                bt = block_tables.to(device=device, dtype=torch.int32)
-                if bt.ndim == 1:
-                    bt = bt.unsqueeze(0)
-                self.block_table = bt.contiguous()
-            else:
-                pitch = max(len(r) for r in block_tables)
-                rows = [list(map(int, r)) + [0] * (pitch - len(r)) for r in block_tables]
-                self.block_table = torch.tensor(rows, dtype=torch.int32, device=device)
+        if rows is not None:
+            self.block_table = cuts[4].view(n, pitch)
+        elif block_tables is not None:
+            bt = block_tables.to(device=device, dtype=torch.int32)
+            if bt.ndim == 1:
+                bt = bt.unsqueeze(0)
+            self.block_table = bt.contiguous()
             pitch = int(self.block_table.shape[1])
-            if int(self.block_table.shape[0]) != self.num_seqs:
+            if int(self.block_table.shape[0]) != n:
                 raise ValueError("block table rows != number of sequences")
         self.max_seq_len = max(self.seq_lens_host)
         self.max_budget = max(self.budgets_host) if self.budgets_host else 0

@@ -44,6 +44,8 @@ def clear_kv_layout_axis_hints_for_tests() -> None:
 
 
 def kv_axis_hint(kv_cache: torch.Tensor):
+    if not _KV_AXIS_HINTS:          # the usual case: nothing registered, no key to build
+        return None
     return _KV_AXIS_HINTS.get(_hint_key(kv_cache))
 
 
@@ -132,7 +134,7 @@ def _run_compaction(kv_caches, block_ids, block_size: int, keep_rows: torch.Tens
     hints = {kv_axis_hint(c) for c in kv_caches}
     if len(hints) != 1:
         raise ValueError("layers of one group disagree on the K/V axis hint")
-    kv = ops.PagedKV.from_kv_caches(kv_caches, kv_axis=hints.pop())
+    kv = ops.PagedKV.for_kv_caches(kv_caches, kv_axis=hints.pop())
     if kv.block_size != block_size:
         raise ValueError(f"block_size={block_size} does not match the cache's {kv.block_size}")
     k = int(keep_rows.shape[1])

@@ -137,7 +137,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
 
     def _paged_kv(caches):
         hints = {kv_axis_hint(c) for c in caches}
-        return ops.PagedKV.from_kv_caches(caches, rope_style=_stats().rope_style,
+        return ops.PagedKV.for_kv_caches(caches, rope_style=_stats().rope_style,
                                           kv_axis=hints.pop() if len(hints) == 1 else None)
 
     def _score_and_select(kv: ops.PagedKV, layer_ids: tuple, block_ids, total_tokens: int, prefill_len: int,
