@@ -473,6 +473,43 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
                             ft, k, tie_tol=2e-3 * scale)
 
 
+@pytest.mark.parametrize("kernel", ["mfma", "valu"])
+def test_resident_selection_on_dense_keys(kernel, monkeypatch):
+    """[B, H, T, D] keys without a block table (the selector's keys_dense call shape) through
+    the resident kernels: the 'block' of a sequence is the sequence itself."""
+    g = torch.Generator().manual_seed(11)
+    b, hkv, hq, t, d = 3, 4, 8, 700, 128
+    keys = (torch.randn(b, hkv, t, d, generator=g) + torch.randn(1, hkv, 1, d, generator=g)).to(torch.bfloat16).to(DEV)
+    qc = torch.randn(2, hq, d // 2, 2, generator=g)
+    qa = qc.pow(2).sum(-1).sqrt() + torch.rand(2, hq, d // 2, generator=g)
+    sc = ops.ScoreConfig(ops.fold_stats(qc.to(DEV), qa.to(DEV), torch.ones_like(qa).to(DEV)),
+                         synth.rope_inv_freq(small()).to(DEV), synth.geometric_offsets().to(DEV))
+    # two "layers" that share the key tensor (a PagedKV of dense keys holds one view per layer)
+    view = keys.permute(0, 2, 1, 3)
+    kv = ops.PagedKV([view, view], None)
+    lens = [t, 333, 512]
+    batch = ops.StepBatch(DEV, lens, round_start=[900, 400, 512], budgets=128)
+    sel = ops.SelectConfig(window_size=16)
+    print(f"dense keys kernel={kernel}", flush=True)
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_" + kernel
+    keep_r, fin_r, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    torch.cuda.synchronize()
+    assert ws.status() == 0
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    assert ops.select_path(kv, batch, sc, sel) == "two_pass"
+    keep_t, fin_t, _ = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    torch.cuda.synchronize()
+    for i, n in enumerate(lens):
+        fr, ft = fin_r[i * hkv:(i + 1) * hkv, :n].cpu(), fin_t[i * hkv:(i + 1) * hkv, :n].cpu()
+        assert torch.equal(torch.isinf(fr), torch.isinf(ft))
+        finite = torch.isfinite(ft)
+        scale = float(ft[finite].abs().max())
+        assert float((fr[finite] - ft[finite]).abs().max()) <= 5e-4 * scale
+        assert_keep_matches(keep_r[i * hkv:(i + 1) * hkv, :128].cpu().long(), keep_t[i * hkv:(i + 1) * hkv, :128].cpu().long(),
+                            ft, 128, tie_tol=2e-3 * scale)
+
+
 def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
     sel = ops.SelectConfig(window_size=12)
     for seq_lens, want in (((300,), "two_pass"), ((3072,) * 16, "resident_mfma"), ((2176,) * 16, "two_pass")):
