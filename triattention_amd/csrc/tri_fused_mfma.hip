@@ -541,9 +541,11 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_
       default: return hipErrorInvalidValue;
     }
   }
-  // One-byte keys: eight step buffers.  Slack of 128 tokens (the ring of a 1024-token tile still fits).
+  // One-byte keys: eight step buffers.
   constexpr int NB = DT == TRI_KV_FP8_E4M3 ? 8 : 4;
-  constexpr int SL = 128;   // 1.4 % faster than 64 on 16 x 16384 tokens x 36 layers: more room before a layer's statistics are needed
+  // Slack: as much as LDS allows beside the ring of a 1024-token tile, in whole rotations
+  // (16 x 16384 tokens x 36 layers, bf16, warm GPU: 3.54 ms with 64, 3.49 with 128, 3.45 with 192).
+  constexpr int SL = DT == TRI_KV_FP8_E4M3 ? 128 : 192;
   switch (tw) {
     case 1024: return launch_mfma_t<DT, IL, 1024, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
     case 512: return launch_mfma_t<DT, IL, 512, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
