@@ -253,6 +253,31 @@ def test_layer_selection_matches_reference_golden(tag, kw, fixture):
     assert torch.equal(got, gold[f"layer1_{tag}_keep"])
 
 
+@pytest.mark.parametrize("width", [3000, 8192, 16384, 20001, 32768, 40000])
+def test_topk_rows_by_width(width):
+    """Rows up to 8192 / 16384 / 32768 elements are selected from registers (three kernel
+    instances), longer ones by the streaming kernel; ties keep the lowest index."""
+    g = torch.Generator().manual_seed(width)
+    x = torch.randn(6, width, generator=g)
+    x[1, 100:width // 2] = 0.5
+    x[2, :] = -3.0
+    x[3, -50:] = float("inf")
+    x[4, ::7] = float("-inf")
+    x[5] = torch.round(x[5] * 4) / 4              # many small tie classes
+    print(f"topk width={width}", flush=True)
+    xd = x.to(DEV)
+    for k in (1, 130, 2048, width - 1, width):
+        got = ops.topk_rows(xd, k).cpu().long()
+        assert torch.equal(got[:, :k], osel.topk_ascending(x, k)), k
+    lens = [width, 10, 1, width - 3, 777, width // 2 + 1]
+    ks = [5, 20, 1, 2048, 0, width // 3]
+    got = ops.topk_rows(xd, ks, lens).cpu().long()
+    for r, (n, k) in enumerate(zip(lens, ks)):
+        kk = min(k, n)
+        if kk:
+            assert torch.equal(got[r, :kk], osel.topk_ascending(x[r:r + 1, :n], kk)[0])
+
+
 def test_topk_rows_ties_and_order():
     g = torch.Generator().manual_seed(1)
     x = torch.randn(5, 3000, generator=g)

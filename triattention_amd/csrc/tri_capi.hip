@@ -247,7 +247,7 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
     }
   }
   if (!keep) return TRI_OK;   // selection scores only
-  return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, keep,
+  return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, a.Tmax, keep,
                                              batch->max_budget, s),
                        "topk_rows");
 }
@@ -381,7 +381,7 @@ int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, cons
   if (!scores || !row_lens || !row_ks || !keep) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_topk_rows: NULL pointer");
   if (num_rows < 0 || rows_per_entry <= 0 || row_pitch < max_len || keep_pitch <= 0 || max_len <= 0)
     return fail(TRI_ERR_INVALID_ARGUMENT, "tri_topk_rows: bad sizes");
-  return launch_status(tri::launch_topk_rows(scores, row_pitch, num_rows, row_lens, row_ks, rows_per_entry, keep,
+  return launch_status(tri::launch_topk_rows(scores, row_pitch, num_rows, row_lens, row_ks, rows_per_entry, max_len, keep,
                                              keep_pitch, (hipStream_t)stream),
                        "topk_rows");
 }

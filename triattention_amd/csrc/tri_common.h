@@ -121,7 +121,7 @@ struct SelectLaunch {
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
 hipError_t launch_clear_status(uint32_t* status, hipStream_t s);
 hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
-                            const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry,
+                            const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry, int max_len,
                             int32_t* keep, int keep_pitch, hipStream_t s);
 
 struct FusedLaunch {
