@@ -479,3 +479,21 @@ def test_request_state_views_and_group_tensors():
     assert hook_mod.infer_layer_idx("model.layers.17.self_attn", object(), 3) == 17
     assert hook_mod.infer_layer_idx("attn", types.SimpleNamespace(layer_idx=4), 3) == 4
     assert hook_mod.scheduled_tokens_for_req(types.SimpleNamespace(num_scheduled_tokens={"r": 0}), "r") == 1
+
+
+def test_keep_tensors_from_the_selector_are_remembered_by_identity():
+    """The compaction functions skip their host-side index check only for the very tensor the
+    selector returned, and only for the token count it was selected from."""
+    import gc
+    from triattention_amd.runtime import kv_compaction as kc
+    keep = torch.arange(12).reshape(2, 6)
+    same_values = keep.clone()
+    kc.mark_keep_validated(keep, 40)
+    assert kc._is_validated(keep, 40)
+    assert not kc._is_validated(keep, 41)
+    assert not kc._is_validated(same_values, 40)
+    assert not kc._is_validated([[0, 1]], 40)
+    key = id(keep)
+    del keep
+    gc.collect()
+    assert key not in kc._VALIDATED_KEEP

@@ -14,6 +14,7 @@ Differences, all on purpose:
 """
 from __future__ import annotations
 
+import weakref
 from typing import Iterable
 
 import torch
@@ -21,6 +22,23 @@ import torch
 from .. import ops
 
 _KV_AXIS_HINTS: dict = {}
+
+# Keep-index tensors that came out of this package's own top-k kernel: ascending, unique and
+# inside [0, T) by construction (whatever the scores were), so the host-side check of the
+# compaction functions (two device-to-host reads, each a stream synchronisation in the middle
+# of a compression) is skipped for them.  Anything else is checked as the reference does.
+_VALIDATED_KEEP: dict = {}     # id(tensor) -> (weak reference, number of tokens it was selected from)
+
+
+def mark_keep_validated(keep: torch.Tensor, total_tokens: int) -> torch.Tensor:
+    key = id(keep)
+    _VALIDATED_KEEP[key] = (weakref.ref(keep, lambda _ref, key=key: _VALIDATED_KEEP.pop(key, None)), int(total_tokens))
+    return keep
+
+
+def _is_validated(keep, total_tokens: int) -> bool:
+    entry = _VALIDATED_KEEP.get(id(keep))
+    return entry is not None and entry[0]() is keep and entry[1] == int(total_tokens)
 
 
 def _hint_key(kv_cache: torch.Tensor):
@@ -171,6 +189,7 @@ def compact_request_kv_in_place_per_head(kv_cache, block_ids, block_size: int, k
     caches = list(kv_cache) if isinstance(kv_cache, (list, tuple)) else [kv_cache]
     key_cache, _ = _split_kv_axes(caches[0])
     device, heads = key_cache.device, int(key_cache.shape[2])
+    trusted = _is_validated(keep_token_indices_per_head, total_tokens)
     if isinstance(keep_token_indices_per_head, torch.Tensor):
         keep = keep_token_indices_per_head.to(device=device, dtype=torch.long)
     else:
@@ -185,7 +204,8 @@ def compact_request_kv_in_place_per_head(kv_cache, block_ids, block_size: int, k
     k = int(keep.shape[1])
     if k <= 0:
         return 0
-    _check_rows(keep, total_tokens, "per-head keep indices")
+    if not trusted:
+        _check_rows(keep, total_tokens, "per-head keep indices")
     if k >= total_tokens:
         return k
     _run_compaction(caches, block_ids, block_size, keep, total_tokens, shared=False,

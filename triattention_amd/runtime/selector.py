@@ -19,7 +19,7 @@ import torch
 from .. import ops
 from ..core import stats as stats_mod
 from .config import TriAttentionRuntimeConfig
-from .kv_compaction import kv_axis_hint
+from .kv_compaction import kv_axis_hint, mark_keep_validated
 from .models import TRITON_SCORING_REQUIRED_MARKER as MARK
 
 
@@ -158,7 +158,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
             keep, _, _ = ops.select_paged(kv, batch, sc, sel)
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
-        return keep.to(torch.long)
+        return mark_keep_validated(keep.to(torch.long), total_tokens)
 
     def _select_keep_indices(*, keys_dense: torch.Tensor | None = None, kv_cache: torch.Tensor | None = None,
                              block_ids=None, block_size: int | None = None, total_tokens: int, prefill_len: int,
