@@ -573,9 +573,10 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
     if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   const int tiles = ceil_div(Tmax, tw);
   if ((int64_t)tiles * HC > resident) return p;
-  // A launch that fills fewer than ~70 % of the CUs loses to the two-pass kernels, which
-  // spread a small problem over the whole chip (crossover measured at B = 16: T ~ 2500).
-  if (!any_fill && (int64_t)B * tiles * HC * 10 < (int64_t)resident * 7) return p;
+  // A launch that fills fewer than ~60 % of the CUs loses to the two-pass kernels, which
+  // spread a small problem over the whole chip (16 sequences: even at 2176 tokens = 56 % of
+  // the CUs, 10 % ahead at 2560 = 62 %, 21 % ahead at 3072 = 75 %).
+  if (!any_fill && (int64_t)B * tiles * HC * 10 < (int64_t)resident * 6) return p;
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;
