@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--hook-latency", action="store_true",
                     help="also time the runner hook (triattention_apply_compression) for one request of "
                          "budget + 128 tokens, host side included")
+    ap.add_argument("--query-stats", action="store_true",
+                    help="also time the calibration statistics kernel on one layer's captured queries "
+                         "(32 heads x 32768 tokens x 128, bf16)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (reference point for HBM byte counters)")
     return ap.parse_args()
@@ -147,6 +150,35 @@ def hook_latency(w, dev, calls: int = 30):
     times.sort()
     return {"tokens": t, "budget": w.budget, "layers": w.num_layers, "calls": calls,
             "ms_median": times[len(times) // 2], "ms_min": times[0], "ms_max": times[-1]}
+
+
+def query_stats_leg(dev, heads: int = 32, tokens: int = 32768, dim: int = 128, calls: int = 20):
+    """ops.query_stats on one layer of captured query states in the layout a Hugging Face
+    attention module produces them ([1, T, H, D] viewed as [H, T, D]).  The operand that has
+    to come from HBM is q_rot: heads * tokens * dim * 2 bytes."""
+    from triattention_amd import ops
+
+    q = torch.randn(1, tokens, heads, dim, device=dev).to(torch.bfloat16).transpose(1, 2)[0]
+    inv = 1e6 ** (-torch.arange(0, dim, 2, device=dev, dtype=torch.float32) / dim)
+    ang = torch.arange(tokens, device=dev, dtype=torch.float32)[:, None] * inv[None]
+    emb = torch.cat((ang, ang), -1)
+    cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    for _ in range(3):
+        ops.query_stats(q, cos, sin)
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(calls):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        ops.query_stats(q, cos, sin)
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+    times.sort()
+    nbytes = heads * tokens * dim * 2
+    med = times[len(times) // 2]
+    return {"heads": heads, "tokens": tokens, "head_dim": dim, "dtype": "bf16", "ms_median": med,
+            "query_bytes": nbytes, "gbs": nbytes / (med * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 def main() -> int:
@@ -320,6 +352,8 @@ def main() -> int:
         torch.cuda.synchronize()
         out["copy_calibration_bytes"] = 1 << 30
         del src, dst
+    if args.query_stats:
+        out["query_stats"] = query_stats_leg(dev)
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
     if not args.no_cpu_baseline:

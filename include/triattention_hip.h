@@ -195,6 +195,22 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
                       const tri_select_params* sel, int32_t* keep, void* workspace,
                       uint64_t workspace_bytes, void* stream);
 
+/* Calibration: per-query-head frequency statistics of one layer's captured query states;
+ * replaces the RoPE inversion and the per-head means of scripts/calibrate.py:196-224
+ * (helpers :38-98; same arithmetic as triattention/methods/pruning_utils.py:40-98).
+ * q_rot[h*stride_head + t*stride_token + d] are the queries after RoPE times the attention
+ * scale, cos / sin are [num_tokens][head_dim] rotary tables, all in `dtype` (TRI_KV_BF16 or
+ * TRI_KV_FP16); every elementwise step of the inversion rounds to that dtype, as the
+ * reference's tensors do.  out_real / out_imag / out_abs: fp32 [num_heads][head_dim/2], the
+ * mean over tokens of the un-rotated query per frequency pair (real, imaginary) and of its
+ * modulus: the "q_mean_real" / "q_mean_imag" / "q_abs_mean" entries of the stats file.
+ * workspace: tri_qstats_workspace_bytes() bytes of device memory, 16-byte aligned. */
+uint64_t tri_qstats_workspace_bytes(int32_t num_heads, int32_t num_tokens, int32_t head_dim);
+int tri_qstats(const void* q_rot, int64_t stride_head, int64_t stride_token, const void* cos,
+               const void* sin, int32_t num_heads, int32_t num_tokens, int32_t head_dim,
+               int32_t dtype, int32_t rope_style, float scale, float* out_real, float* out_imag,
+               float* out_abs, void* workspace, uint64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,7 @@ CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB_NAME = "libtriattention_hip.so"
 LIB_PATH = PKG / LIB_NAME
-SOURCES = ["tri_capi.hip", "tri_score.hip", "tri_fused.hip", "tri_fused_mfma.hip", "tri_select.hip", "tri_compact.hip"]
+SOURCES = ["tri_capi.hip", "tri_score.hip", "tri_fused.hip", "tri_fused_mfma.hip", "tri_select.hip", "tri_compact.hip", "tri_calib.hip"]
 
 # Packed fp32 instructions are switched off on purpose: hipcc forms them from
 # ordinary float code and some forms have given wrong results on this hardware.

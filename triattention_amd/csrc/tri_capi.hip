@@ -442,4 +442,39 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
   return launch_status(tri::launch_compact(c, s), "compact");
 }
 
+uint64_t tri_qstats_workspace_bytes(int32_t num_heads, int32_t num_tokens, int32_t head_dim) {
+  if (num_heads <= 0 || num_tokens <= 0 || (head_dim != 64 && head_dim != 128 && head_dim != 256)) return 0;
+  return (uint64_t)tri::qstats_workspace_bytes(num_heads, num_tokens, head_dim);
+}
+
+int tri_qstats(const void* q_rot, int64_t stride_head, int64_t stride_token, const void* cos, const void* sin,
+               int32_t num_heads, int32_t num_tokens, int32_t head_dim, int32_t dtype, int32_t rope_style,
+               float scale, float* out_real, float* out_imag, float* out_abs, void* workspace,
+               uint64_t workspace_bytes, void* stream) {
+  if (!q_rot || !cos || !sin || !out_real || !out_imag || !out_abs)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_qstats: NULL pointer");
+  if (num_heads <= 0 || num_tokens <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_qstats: bad sizes");
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(TRI_ERR_UNSUPPORTED, "head_dim %d not in {64,128,256}", head_dim);
+  if (dtype != TRI_KV_BF16 && dtype != TRI_KV_FP16)
+    return fail(TRI_ERR_UNSUPPORTED, "tri_qstats: dtype %d (bf16 or fp16 query states)", dtype);
+  if (rope_style != TRI_ROPE_HALF && rope_style != TRI_ROPE_INTERLEAVED)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "rope_style %d", rope_style);
+  if (scale == 0.f) return fail(TRI_ERR_INVALID_ARGUMENT, "attention scaling factor must be non-zero");
+  if (stride_token < head_dim || stride_token % 2 || stride_head % 2 || !is_aligned(q_rot, 4) || !is_aligned(cos, 4) ||
+      !is_aligned(sin, 4))
+    return fail(TRI_ERR_INVALID_ARGUMENT, "tri_qstats: rows must be 4-byte aligned and head_dim contiguous");
+  const uint64_t need = tri_qstats_workspace_bytes(num_heads, num_tokens, head_dim);
+  if (!workspace || workspace_bytes < need || !is_aligned(workspace, 16))
+    return fail(TRI_ERR_WORKSPACE, "tri_qstats: workspace of %llu bytes needed", (unsigned long long)need);
+  tri::QStatsLaunch q{};
+  q.q_rot = q_rot; q.cos = cos; q.sin = sin;
+  q.stride_head = stride_head; q.stride_token = stride_token;
+  q.H = num_heads; q.T = num_tokens; q.D = head_dim; q.dtype = dtype; q.rope_style = rope_style;
+  q.scale = scale;
+  q.out_real = out_real; q.out_imag = out_imag; q.out_abs = out_abs;
+  q.workspace = workspace;
+  return launch_status(tri::launch_qstats(q, (hipStream_t)stream), "qstats");
+}
+
 }  // extern "C"

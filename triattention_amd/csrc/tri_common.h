@@ -162,6 +162,22 @@ struct CompactLaunch {
   void* staging;       // full-permutation mode only
 };
 hipError_t launch_compact(const CompactLaunch& a, hipStream_t s);
+
+// Calibration statistics of one layer's captured queries (tri_calib.hip).
+struct QStatsLaunch {
+  const void* q_rot;      // [H][T][D] through (stride_head, stride_token), 16-bit elements
+  const void* cos;        // [T][D]
+  const void* sin;        // [T][D]
+  int64_t stride_head, stride_token;
+  int H, T, D, dtype, rope_style;
+  float scale;
+  float* out_real;        // [H][D/2]
+  float* out_imag;
+  float* out_abs;
+  void* workspace;
+};
+int64_t qstats_workspace_bytes(int H, int T, int D);
+hipError_t launch_qstats(const QStatsLaunch& q, hipStream_t s);
 hipError_t launch_compact_full(const CompactLaunch& a, hipStream_t s);
 
 }  // namespace tri

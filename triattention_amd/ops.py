@@ -419,6 +419,41 @@ def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] 
     return keep
 
 
+def query_stats(q_rot: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, scale: float = 1.0,
+                rope_style: str = "half"):
+    """Frequency statistics of one layer's captured query states (scripts/calibrate.py:196-224).
+
+    q_rot [H, T, D] (any strides with contiguous D), cos / sin [T, D], all bf16 or all fp16 on
+    the device.  Returns fp32 [H, D/2] tensors (q_mean_real, q_mean_imag, q_abs_mean).
+    """
+    lib = _lib.load()
+    if not q_rot.is_cuda:
+        raise RuntimeError("query_stats needs device tensors (there is no CPU fallback)")
+    if q_rot.ndim != 3 or q_rot.dtype not in (torch.bfloat16, torch.float16) or q_rot.stride(2) != 1:
+        raise ValueError("q_rot must be a [H, T, D] bf16/fp16 tensor with contiguous head_dim")
+    H, T, D = (int(x) for x in q_rot.shape)
+    if T == 0:
+        raise ValueError("no tokens")
+    tables = []
+    for name, t in (("cos", cos), ("sin", sin)):
+        if t.ndim == 3 and t.shape[0] == 1:
+            t = t[0]
+        if tuple(t.shape) != (T, D) or t.dtype != q_rot.dtype or t.device != q_rot.device:
+            raise ValueError(f"{name} must be a [{T}, {D}] tensor of q_rot's dtype on its device")
+        tables.append(t.contiguous())
+    if rope_style not in ("half", "interleaved"):
+        raise ValueError(f"rope_style must be 'half' or 'interleaved', got {rope_style!r}")
+    nbytes = int(lib.tri_qstats_workspace_bytes(H, T, D))
+    if nbytes == 0:
+        raise ValueError(f"unsupported head_dim {D} (64, 128 or 256)")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q_rot.device)
+    out = torch.empty(3, H, D // 2, dtype=torch.float32, device=q_rot.device)
+    _lib.check(lib.tri_qstats(_ptr(q_rot), int(q_rot.stride(0)), int(q_rot.stride(1)), _ptr(tables[0]), _ptr(tables[1]),
+                              H, T, D, _DTYPES[q_rot.dtype], ROPE_INTERLEAVED if rope_style == "interleaved" else ROPE_HALF,
+                              float(scale), _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _ptr(ws), nbytes, _stream()))
+    return out[0], out[1], out[2]
+
+
 def topk_batch(scores: torch.Tensor, batch: StepBatch, rows_per_seq: int, keep: torch.Tensor | None = None):
     """keep rows (ascending int32 [rows, max_budget]) from selection scores [rows, Tmax] with
     the batch's own device-side lengths and budgets; rows_per_seq rows belong to a sequence."""
