@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 1
+#define TRI_ABI_VERSION 2
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -94,6 +94,10 @@ typedef struct tri_select_params {
   int32_t group_reduce;         /* tri_reduce over the query heads of a KV head (runtime/selector_hf.py:277-297) */
   int32_t layer_reduce;         /* tri_reduce over layers; -1 = none (one keep set per layer) */
   int32_t shared;               /* 1: max over KV heads, one index list per (seq[, layer]) (runtime/selector_hf.py:636-637) */
+  int32_t group_first;          /* 0: normalise every score head, then reduce over the query heads of a KV head (vLLM
+                                   runtime, runtime/selector_hf.py:916-989).  1: reduce first, then normalise per
+                                   (layer, KV head) with torch mean / unbiased std (SGLang backend,
+                                   sglang/scheduler_hooks.py:655-690, core/utils.py:466-480) */
 } tri_select_params;
 
 int tri_abi_version(void);

@@ -61,6 +61,7 @@ class SelectParams(C.Structure):
     _fields_ = [
         ("normalize", C.c_int32), ("window_size", C.c_int32), ("protect_prefill", C.c_int32),
         ("group_reduce", C.c_int32), ("layer_reduce", C.c_int32), ("shared", C.c_int32),
+        ("group_first", C.c_int32),
     ]
 
 
@@ -113,8 +114,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         if fn.restype is C.c_int and name not in ("tri_abi_version",):
             fn.restype = C.c_int
-    if lib.tri_abi_version() != 1:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 1; rebuild the library")
+    if lib.tri_abi_version() != 2:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 2; rebuild the library")
     _lib = lib
     return lib
 

@@ -173,6 +173,7 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
   a.max_budget = batch->max_budget;
   a.normalize = sel->normalize; a.window_size = sel->window_size; a.protect_prefill = sel->protect_prefill;
   a.group_reduce = sel->group_reduce; a.layer_reduce = sel->layer_reduce; a.shared = sel->shared;
+  a.group_first = sel->group_first ? 1 : 0;
   a.seq_lens = batch->seq_lens; a.prefill_lens = batch->prefill_lens; a.budgets = batch->budgets;
   a.partial = at<float>(ws, w.partial); a.mustd = at<float>(ws, w.mustd);
   a.raw = raw; a.raw_stride_layer = rs_layer; a.raw_stride_token = rs_token; a.raw_stride_head = rs_head;
@@ -186,7 +187,7 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
 int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
                     hipStream_t s) {
-  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared;
+  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first;
   if (!fused) {
     // The status word belongs to the resident kernel; on this path it just reads "fine".
     const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
@@ -372,7 +373,7 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared) ? w.fused.eligible : 0;
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first) ? w.fused.eligible : 0;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,

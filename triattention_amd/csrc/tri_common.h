@@ -107,7 +107,7 @@ hipError_t launch_score(const ScoreLaunch& a, hipStream_t s);
 
 struct SelectLaunch {
   int B, L, Hkv, A, G, Tmax, num_tiles, max_budget;
-  int normalize, window_size, protect_prefill, group_reduce, layer_reduce, shared;
+  int normalize, window_size, protect_prefill, group_reduce, layer_reduce, shared, group_first;
   const int32_t* seq_lens;
   const int32_t* prefill_lens;
   const int32_t* budgets;

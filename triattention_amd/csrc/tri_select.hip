@@ -4,6 +4,10 @@
 //                          scorer's per-tile sums (runtime/selector_hf.py:896-913).
 //  combine_kernel        : z-score, +inf guards, reduce over the query heads of a KV
 //                          head, reduce over layers (runtime/selector_hf.py:916-989).
+//  group_stats_kernel    : the other order of operations (the reference's SGLang backend,
+//                          sglang/scheduler_hooks.py:655-690): reduce over the query heads of
+//                          a KV head first, then normalise per (layer, KV head) with
+//                          core/utils.py:466-480 (torch mean / unbiased std).
 //  topk_rows_kernel      : order-preserving radix select on the monotone integer
 //                          image of the float, then an ordered compaction that emits
 //                          the kept token indices ascending; ties at the threshold
@@ -42,6 +46,56 @@ __global__ void finalize_stats_kernel(const float* partial, const int32_t* seq_l
   mustd[(int64_t)idx * 2 + 1] = sd;
 }
 
+// Reduce-first order: mean and std over the tokens of m[n] = reduce over the query heads of
+// raw[n][h*G .. h*G+G), per (sequence, layer, KV head), with torch's definitions
+// (core/utils.py:476-479: mean, unbiased std, std < 1e-8 -> 1).  Sums in double; one
+// workgroup per (sequence, layer, KV head).  mustd[(b*L + l)*A*2 + h*2] = (mean, std).
+__global__ __launch_bounds__(256) void group_stats_kernel(const float* raw, int64_t stride_layer, int64_t stride_token,
+                                                          int64_t stride_head, const int32_t* seq_lens, int L, int Hkv,
+                                                          int A, int G, int group_reduce, int normalize, float* mustd) {
+  __shared__ double red[256][2];
+  const int h = blockIdx.x % Hkv;
+  const int bl = blockIdx.x / Hkv, b = bl / L;
+  float* out = mustd + ((int64_t)bl * A + h) * 2;
+  if (!normalize) {
+    if (threadIdx.x == 0) { out[0] = 0.f; out[1] = 1.f; }
+    return;
+  }
+  const int T = seq_lens[b];
+  const float* base = raw + (int64_t)bl * stride_layer + (int64_t)h * G * stride_head;
+  double s = 0.0, q = 0.0;
+  for (int n = threadIdx.x; n < T; n += 256) {
+    const float* p = base + (int64_t)n * stride_token;
+    float m = (group_reduce == TRI_REDUCE_MAX) ? -INFINITY : 0.f;
+    for (int g = 0; g < G; ++g) {
+      const float x = p[(int64_t)g * stride_head];
+      m = (group_reduce == TRI_REDUCE_MAX) ? fmaxf(m, x) : __fadd_rn(m, x);
+    }
+    if (group_reduce != TRI_REDUCE_MAX) m = __fdiv_rn(m, (float)G);
+    s += (double)m;
+    q += (double)m * (double)m;
+  }
+  red[threadIdx.x][0] = s;
+  red[threadIdx.x][1] = q;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if (threadIdx.x < off) {
+      red[threadIdx.x][0] += red[threadIdx.x + off][0];
+      red[threadIdx.x][1] += red[threadIdx.x + off][1];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const double mean = red[0][0] / (double)T;
+    double var = T > 1 ? (red[0][1] - (double)T * mean * mean) / (double)(T - 1) : 0.0;
+    if (var < 0.0) var = 0.0;
+    float sd = (float)sqrt(var);
+    if (sd < 1e-8f) sd = 1.f;     // also a single token, where torch's unbiased std is undefined
+    out[0] = (float)mean;
+    out[1] = sd;
+  }
+}
+
 struct CombineArgs {
   const float* raw;
   const float* mustd;
@@ -51,6 +105,7 @@ struct CombineArgs {
   int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
   int B, L, Hkv, A, G, Tmax;
   int window_size, protect_prefill, group_reduce, layer_reduce, shared;
+  int group_first;    // 1: reduce over the query heads of a KV head before normalising (mustd is per KV head)
   int rows_per_seq;   // rows per (sequence[, layer]): shared ? 1 : Hkv
   int tokens_per_wg;  // 256 / rows_per_seq
 };
@@ -134,10 +189,12 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
           float gv = (a.group_reduce == TRI_REDUCE_MAX) ? -INFINITY : 0.f;
           for (int q = 0; q < a.G; ++q) {
             const int ah = h * a.G + q;
-            const float z = zscore(raw_l[(int64_t)ah * a.raw_stride_head], ms[ah * 2], ms[ah * 2 + 1]);
+            const float x = raw_l[(int64_t)ah * a.raw_stride_head];
+            const float z = a.group_first ? x : zscore(x, ms[ah * 2], ms[ah * 2 + 1]);
             gv = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(gv, z) : __fadd_rn(gv, z);
           }
           if (a.group_reduce != TRI_REDUCE_MAX) gv = __fdiv_rn(gv, (float)a.G);
+          if (a.group_first) gv = zscore(gv, ms[h * 2], ms[h * 2 + 1]);
           v = fmaxf(v, gv);
         }
         if (guard) v = INFINITY;
@@ -414,8 +471,13 @@ hipError_t launch_clear_status(uint32_t* status, hipStream_t s) {
 
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const int n = a.B * a.L * a.A;
-  hipLaunchKernelGGL(finalize_stats_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s, a.partial, a.seq_lens,
-                     a.B, a.L, a.A, a.num_tiles, a.normalize, a.mustd);
+  if (a.group_first)
+    hipLaunchKernelGGL(group_stats_kernel, dim3(a.B * a.L * a.Hkv), dim3(256), 0, s, a.raw, a.raw_stride_layer,
+                       a.raw_stride_token, a.raw_stride_head, a.seq_lens, a.L, a.Hkv, a.A, a.G, a.group_reduce,
+                       a.normalize, a.mustd);
+  else
+    hipLaunchKernelGGL(finalize_stats_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s, a.partial, a.seq_lens,
+                       a.B, a.L, a.A, a.num_tiles, a.normalize, a.mustd);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
 
@@ -434,12 +496,13 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   c.group_reduce = a.group_reduce;
   c.layer_reduce = a.layer_reduce;
   c.shared = a.shared;
+  c.group_first = a.group_first;
   c.rows_per_seq = a.shared ? 1 : a.Hkv;
   c.tokens_per_wg = 256 / c.rows_per_seq;
   const bool per_layer = a.layer_reduce < 0;
   dim3 grid(ceil_div(a.Tmax, c.tokens_per_wg), per_layer ? a.L : 1, a.B);
   const size_t smem = (size_t)c.rows_per_seq * c.tokens_per_wg * sizeof(float);
-  const bool vec4 = a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
+  const bool vec4 = !a.group_first && a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
                     a.raw_stride_layer % 4 == 0 && (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(a.mustd) % 16) == 0;
   if (vec4)

@@ -244,13 +244,14 @@ class SelectConfig:
     group_reduce: str = "max"
     layer_reduce: str | None = "mean"    # None: one keep set per layer
     shared: bool = False
+    group_first: bool = False            # reduce over the query heads of a KV head before normalising
 
     def struct(self) -> SelectParams:
         lr = REDUCE_NONE if self.layer_reduce is None else (REDUCE_MAX if self.layer_reduce == "max" else REDUCE_MEAN)
         return SelectParams(normalize=int(self.normalize), window_size=int(self.window_size),
                             protect_prefill=int(self.protect_prefill),
                             group_reduce=REDUCE_MAX if self.group_reduce == "max" else REDUCE_MEAN,
-                            layer_reduce=lr, shared=int(self.shared))
+                            layer_reduce=lr, shared=int(self.shared), group_first=int(self.group_first))
 
 
 def fold_stats(q_mean_complex: torch.Tensor, q_abs_mean: torch.Tensor, freq_scale_sq: torch.Tensor,
