@@ -41,7 +41,9 @@ typedef enum tri_reduce { TRI_REDUCE_MEAN = 0, TRI_REDUCE_MAX = 1 } tri_reduce;
  * which covers both vLLM layouts, [2, nb, bs, H, D] and [nb, 2, bs, H, D]
  * (runtime/kv_compaction.py:38-53,94-117), by passing separate K and V bases.
  * A dense [B, H, T, D] tensor (core/scoring.py:93) is the same thing with
- * block_size = T, one block per sequence and an identity block table. */
+ * block_size = T, one block per sequence and an identity block table; a token-level
+ * pool [total_slots, H, D] with a (request, position) -> slot table
+ * (sglang/kv_compaction.py:56-137) is the same thing with block_size = 1. */
 typedef struct tri_kv_layout {
   int32_t num_layers;
   int32_t num_kv_heads;
