@@ -346,6 +346,16 @@ def test_compaction_large_budget_and_dims():
     _compact_case(small(seq_lens=(700,), budget=300, head_dim=256, block_size=8), 0, True, False, False)
 
 
+@pytest.mark.parametrize("heads", [3, 5, 6, 7])
+def test_shared_compaction_with_token_rows_that_do_not_divide_a_tile(heads):
+    """One index list for all heads moves whole token rows; with 3, 5, 6 or 7 heads a row's
+    chunk count does not divide the 1024-chunk tile of the ordered pass, so a tile has spare
+    chunk slots (they must not write anything of their own)."""
+    print(f"shared compaction heads={heads}", flush=True)
+    _compact_case(small(seq_lens=(3000, 500), budget=1500, num_kv_heads=heads, num_q_heads=heads), 0, True, False, False)
+    _compact_case(small(seq_lens=(1600,), budget=1500, num_kv_heads=heads, num_q_heads=heads), 1, True, True, False)
+
+
 @pytest.mark.parametrize("shared", [False, True])
 def test_compaction_when_few_tokens_are_dropped_and_budgets_differ(shared):
     """The rows that come from beyond the budget are a short suffix of every keep list when a
@@ -706,6 +716,45 @@ def test_fp8_step_scores_selects_and_compacts():
             rows = got[b * h:(b + 1) * h, :k]
             ocp.compact_per_head(ref, inp["tables"][b], w.block_size, rows, t, full_permutation=False)
             ocp.compact_per_head(ref_s, inp["tables"][b], w.block_size, rows, t, full_permutation=False)
+            blk, off = ocp.token_slots(inp["tables"][b], w.block_size, torch.arange(k))
+            assert torch.equal(dev_c[:, blk, off], ref[:, blk, off]), (l, b)
+            assert torch.equal(dev_s[:, blk, off], ref_s[:, blk, off]), (l, b)
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_fp8_compaction_moves_scales_with_the_rows(shared):
+    """Random keep lists on an fp8 cache with three KV heads and a budget of several scale
+    tiles: codes and per-(token, head) scales of K and V bit-exact against the oracle."""
+    w = small(kv_dtype="fp8", seq_lens=(3000, 900, 1501), num_layers=2, num_q_heads=3, num_kv_heads=3, budget=1500)
+    inp = build_inputs(w)
+    caches, kv, batch, _ = device_objects(w, inp, DEV)
+    h = w.num_kv_heads
+    rows_per = 1 if shared else h
+    g = torch.Generator().manual_seed(17)
+    keep = torch.zeros(w.num_seqs * rows_per, batch.max_budget, dtype=torch.int32)
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        for r in range(rows_per):
+            keep[b * rows_per + r, :k] = torch.sort(torch.randperm(t, generator=g)[:k]).values.int()
+    print(f"fp8 compaction shared={shared}", flush=True)
+    ops.compact(kv, batch, keep.to(DEV), shared=shared)
+    torch.cuda.synchronize()
+    ks_dev, vs_dev = kv._keep[2], kv._keep[3]
+    for l in range(w.num_layers):
+        ref = inp["caches"][l].clone().view(torch.uint8)
+        nb = ref.shape[1]
+        ref_s = torch.stack([inp["k_scales"][l].view(nb, w.block_size, h, 1),
+                             inp["v_scales"][l].view(nb, w.block_size, h, 1)]).clone()
+        dev_c = caches[l].cpu().view(torch.uint8)
+        dev_s = torch.stack([ks_dev[l].cpu().view(nb, w.block_size, h, 1), vs_dev[l].cpu().view(nb, w.block_size, h, 1)])
+        for b, t in enumerate(w.seq_lens):
+            k = min(w.budget, t)
+            rows = keep[b * rows_per:(b + 1) * rows_per, :k].long()
+            for tgt in (ref, ref_s):
+                if shared:
+                    ocp.compact_shared(tgt, inp["tables"][b], w.block_size, rows[0], t, full_permutation=False)
+                else:
+                    ocp.compact_per_head(tgt, inp["tables"][b], w.block_size, rows, t, full_permutation=False)
             blk, off = ocp.token_slots(inp["tables"][b], w.block_size, torch.arange(k))
             assert torch.equal(dev_c[:, blk, off], ref[:, blk, off]), (l, b)
             assert torch.equal(dev_s[:, blk, off], ref_s[:, blk, off]), (l, b)

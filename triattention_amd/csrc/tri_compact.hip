@@ -152,7 +152,9 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
       uint32_t so[kChunksPerThread];
 #pragma unroll
       for (int c = 0; c < kChunksPerThread; ++c) {
-        // Branch-free: an idle chunk re-reads its own destination and only its store is masked.
+        // Branch-free: a chunk index beyond the tile (a token row whose chunk count does not
+        // divide the tile) repeats the pass's first chunk, load and store alike, so what it
+        // writes is what that chunk writes.
         const int ci = c0 + c * kOrderedThreads + threadIdx.x;
         const bool in = ci < nchunks;
         const int cic = in ? ci : c0;
@@ -163,7 +165,7 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
         const uint32_t inner = (uint32_t)((a.shared ? 0 : list0 + h) + hh) * a.head_units + (uint32_t)cc;
         const uint32_t su = src_units[sl * lists + h];
         dsto[c] = dst_units[sl] + inner;
-        live[c] = in && su != kNoSource;
+        live[c] = su != kNoSource;
         so[c] = live[c] ? su + inner : dsto[c];
       }
       r0 = load_chunk(base + ((uint64_t)so[0] << 4));
@@ -291,8 +293,16 @@ struct ScaleArgs {
 };
 
 __global__ __launch_bounds__(256) void compact_scales_kernel(ScaleArgs a) {
+  // One workgroup per (sequence, layer, K or V) moves the scales of all heads: a thread owns
+  // (slot, head) pairs with the head fastest, so the eight heads of a destination slot are
+  // written by neighbouring threads as one 32-byte piece (one workgroup per head wrote it
+  // as eight separate 4-byte pieces at different times).  Tiles of 256 * kScalesPerThread
+  // pairs; every level of the dependent lookups (keep -> block table -> scale) is issued
+  // for all of a thread's pairs before the next one.  Within a tile all reads precede all
+  // writes (barrier); a later tile reads sources at or beyond its own first slot, which
+  // earlier tiles (writing below that slot) never touch.
+  constexpr int kScalesPerThread = 8;
   int sidx = blockIdx.x;
-  const int h = sidx % a.Hkv; sidx /= a.Hkv;
   const int kv = sidx % 2; sidx /= 2;
   const int l = sidx % a.L;
   const int b = sidx / a.L;
@@ -301,23 +311,40 @@ __global__ __launch_bounds__(256) void compact_scales_kernel(ScaleArgs a) {
   if (k > T) k = T;
   if (k <= 0) return;
   const int rows = a.shared ? 1 : a.Hkv;
-  const int row = a.shared ? 0 : h;
-  const int32_t* keep = a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows + row) * a.max_budget;
+  const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows * a.max_budget;
   const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;
   float* sc = const_cast<float*>(kv ? a.v_scale_layers[l] : a.k_scale_layers[l]);
-  for (int t0 = 0; t0 < k; t0 += 256) {
-    const int j = t0 + threadIdx.x;
-    float v = 0.f;
-    int64_t d = 0;
-    const bool live = j < k;
-    if (live) {
-      const int src = keep[j];
-      const int64_t s = ((int64_t)bt[src / a.block_size] * a.block_size + src % a.block_size) * a.Hkv + h;
-      d = ((int64_t)bt[j / a.block_size] * a.block_size + j % a.block_size) * a.Hkv + h;
-      v = sc[s];
+  const int slots_per_tile = max(256 * kScalesPerThread / a.Hkv, 1);
+  for (int t0 = 0; t0 < k; t0 += slots_per_tile) {
+    int src[kScalesPerThread], jj[kScalesPerThread], hh[kScalesPerThread];
+    bool live[kScalesPerThread];
+#pragma unroll
+    for (int i = 0; i < kScalesPerThread; ++i) {
+      const int p = i * 256 + threadIdx.x;
+      const int sl = p / a.Hkv;
+      hh[i] = p - sl * a.Hkv;
+      live[i] = sl < slots_per_tile && t0 + sl < k;
+      jj[i] = live[i] ? t0 + sl : 0;
+      src[i] = keep[(int64_t)(a.shared ? 0 : hh[i]) * a.max_budget + jj[i]];
+    }
+    int sblk[kScalesPerThread], dblk[kScalesPerThread];
+#pragma unroll
+    for (int i = 0; i < kScalesPerThread; ++i) {
+      sblk[i] = bt[src[i] / a.block_size];
+      dblk[i] = bt[jj[i] / a.block_size];
+    }
+    float v[kScalesPerThread];
+    int64_t d[kScalesPerThread];
+#pragma unroll
+    for (int i = 0; i < kScalesPerThread; ++i) {
+      const int64_t from = ((int64_t)sblk[i] * a.block_size + src[i] % a.block_size) * a.Hkv + hh[i];
+      d[i] = ((int64_t)dblk[i] * a.block_size + jj[i] % a.block_size) * a.Hkv + hh[i];
+      v[i] = sc[from];
     }
     __syncthreads();
-    if (live) sc[d] = v;
+#pragma unroll
+    for (int i = 0; i < kScalesPerThread; ++i)
+      if (live[i]) sc[d[i]] = v[i];
   }
 }
 
@@ -455,7 +482,7 @@ hipError_t launch_scales(const CompactLaunch& a, hipStream_t s) {
   sa.max_budget = a.max_budget;
   sa.keep_per_layer = a.keep_per_layer;
   sa.shared = a.shared;
-  hipLaunchKernelGGL(compact_scales_kernel, dim3(a.B * a.L * 2 * a.Hkv), dim3(256), 0, s, sa);
+  hipLaunchKernelGGL(compact_scales_kernel, dim3(a.B * a.L * 2), dim3(256), 0, s, sa);
   return hipGetLastError();
 }
 
