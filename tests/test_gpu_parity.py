@@ -460,6 +460,8 @@ RESIDENT_CASES = {
     "layer_max_group_mean": dict(w=small(num_layers=3), sel=dict(layer_reduce="max", group_reduce="mean")),
     "no_normalize": dict(w=small(), sel=dict(normalize=False)),
     "prefill_guard": dict(w=small(seq_lens=(400, 90)), sel=dict(protect_prefill=True), prefill_lens=[37, 5]),
+    "tile320": dict(w=small(seq_lens=(2176,) * 30 + (1700, 33), budget=256, num_layers=2)),
+    "tile256_fp8": dict(w=small(kv_dtype="fp8", seq_lens=(3000,) * 15 + (2990,), budget=256, num_layers=2)),
     "tw64": dict(w=small(seq_lens=(9000,) * 20, budget=512, num_layers=2)),
     "tw128": dict(w=small(seq_lens=(40000, 3000, 25001), budget=2048, num_layers=2)),
     "two_launches": dict(w=small(seq_lens=(70000, 100, 66000, 69000), budget=1024, num_layers=2)),
@@ -547,7 +549,11 @@ def test_resident_selection_on_dense_keys(kernel, monkeypatch):
 
 def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
     sel = ops.SelectConfig(window_size=12)
-    for seq_lens, want in (((300,), "two_pass"), ((3072,) * 16, "resident_mfma"), ((2176,) * 16, "two_pass")):
+    cases = (((300,), "two_pass"), ((3072,) * 16, "resident_mfma"), ((2176,) * 16, "resident_mfma"),
+             ((16384,), "two_pass"),           # one sequence: at most 64 tiles, a quarter of the chip
+             ((2176,) * 4, "two_pass"),        # 4 x 17 tiles of 128
+             ((8192,) * 4, "resident_mfma"))   # 4 x 64 tiles of 128
+    for seq_lens, want in cases:
         w = small(seq_lens=seq_lens, num_layers=1)
         tables = synth.make_block_tables(w)
         cache = torch.zeros(2, w.pool_blocks, w.block_size, w.num_kv_heads, w.head_dim, dtype=torch.bfloat16, device=DEV)

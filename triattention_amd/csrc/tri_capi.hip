@@ -102,7 +102,7 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   tri::FusedPlan fused{};
   if (want_mfma)
     fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
-                                 sp->aggregation, b->max_seq_len, resident, f_mfma);
+                                 sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype);
   if (!fused.eligible && !f_mfma)
     fused = tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged, sp->aggregation,
                             b->max_seq_len, resident, f_valu);

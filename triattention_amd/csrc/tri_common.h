@@ -39,7 +39,7 @@ int fused_resident_workgroups();
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                      int resident, bool any_fill);
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill);
+                          int resident, bool any_fill, int kv_dtype);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {

@@ -557,7 +557,7 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_
 }  // namespace
 
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill) {
+                          int resident, bool any_fill, int kv_dtype) {
   FusedPlan p{};
   if (resident <= 0 || D != 128 || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
@@ -571,8 +571,22 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   int tw = tws[ntw - 1];
   for (int i = 0; i < ntw; ++i)
     if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
-  const int tiles = ceil_div(Tmax, tw);
+  int tile = tw, tiles = ceil_div(Tmax, tw);
   if ((int64_t)tiles * HC > resident) return p;
+  if ((int64_t)B * tiles * HC <= resident) {
+    // The whole batch is one launch: cut the sequences into as many tiles as the chip has
+    // room for, in whole rotations of the step buffers (64 tokens, 128 for one-byte keys), so
+    // that e.g. 16 sequences of 3072 tokens run as 16 x 16 tiles of 192 instead of 16 x 12 of
+    // 256.  Not below 128 tokens and not more than 64 tiles per sequence: smaller tiles pay the
+    // per-layer work of a workgroup too often, and every workgroup gathers the statistics of
+    // all tiles of its sequence (one sequence of 16384 tokens as 256 tiles of 64 fills the
+    // chip and takes 1.14 ms; the two-pass kernels take 0.38).
+    const int granule = kv_dtype == TRI_KV_FP8_E4M3 ? 128 : 64;
+    const int tiles_max = min(resident / (B * HC), 64);
+    tile = ceil_div(ceil_div(Tmax, tiles_max), granule) * granule;
+    tile = min(tw, max(128, tile));
+    tiles = ceil_div(Tmax, tile);
+  }
   // A launch that fills fewer than ~60 % of the CUs loses to the two-pass kernels, which
   // spread a small problem over the whole chip (16 sequences: even at 2176 tokens = 56 % of
   // the CUs, 10 % ahead at 2560 = 62 %, 21 % ahead at 3072 = 75 %).
@@ -580,7 +594,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;
-  p.tile_tokens = tw;
+  p.tile_tokens = tile;
   p.tiles_per_seq = tiles;
   p.seqs_per_launch = resident / (tiles * HC);
   p.resident = resident;
