@@ -200,10 +200,13 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
     return do_select(kv, batch, sp, sel, raw, rs_layer, A, 1, fin, keep, ws, w, s);
   }
   const int F = kv->head_dim / 2;
-  hipError_t e = tri::launch_prepare(sp->folded, sp->omega, sp->offsets, sp->num_offsets, batch->round_start,
-                                     batch->num_seqs, kv->num_layers, sp->num_score_heads, F, sp->aggregation,
-                                     at<float>(ws, w.coef), at<float>(ws, w.trig), s);
-  if (e != hipSuccess) return launch_status(e, "prepare");
+  hipError_t e = hipSuccess;
+  if (w.fused.eligible != 2) {   // the matrix-core kernel has a preparation launch of its own
+    e = tri::launch_prepare(sp->folded, sp->omega, sp->offsets, sp->num_offsets, batch->round_start,
+                            batch->num_seqs, kv->num_layers, sp->num_score_heads, F, sp->aggregation,
+                            at<float>(ws, w.coef), at<float>(ws, w.trig), s);
+    if (e != hipSuccess) return launch_status(e, "prepare");
+  }
   tri::FusedLaunch a{};
   a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
   a.block_size = kv->block_size; a.kv_dtype = kv->kv_dtype; a.rope_style = kv->rope_style;
@@ -215,6 +218,8 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.block_table = batch->block_table; a.block_table_pitch = batch->block_table_pitch;
   a.seq_lens = batch->seq_lens; a.prefill_lens = batch->prefill_lens;
   a.coef = at<float>(ws, w.coef);
+  a.folded = sp->folded; a.omega = sp->omega; a.offsets = sp->offsets; a.NO = sp->num_offsets;
+  a.round_start = batch->round_start;
   a.xchg = at<unsigned long long>(ws, w.xchg);
   a.status = at<uint32_t>(ws, w.status);
   a.pack = at<int32_t>(ws, w.pack);

@@ -134,7 +134,9 @@ struct FusedLaunch {
   int block_table_pitch;
   const int32_t* seq_lens;
   const int32_t* prefill_lens;
-  const float* coef;             // workspace
+  const float* coef;             // workspace (vector-unit kernel: written by launch_prepare)
+  // matrix-core kernel: it prepares its own coefficients from these
+  const float* folded; const float* omega; const float* offsets; int NO; const int32_t* round_start;
   unsigned long long* xchg;      // workspace
   uint32_t* status;              // workspace
   int32_t* pack;                 // workspace

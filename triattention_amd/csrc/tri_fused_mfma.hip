@@ -87,54 +87,109 @@ __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, fl
   return packed;
 }
 
-// Coefficient slabs of one (sequence, layer, head) in MFMA B-operand order:
+// Everything the resident kernel needs before it starts, in one launch: workgroup (l, b)
+//  - clears its share of the exchange words (and workgroup (0, 0) the status word);
+//  - evaluates cos / sin of (round_start[b] + offset_j) * omega_f for all offsets and their
+//    means over the offsets, the way trig_kernel does (phase_cos_sin, means summed in offset
+//    order in double);
+//  - combines the means with the folded statistics of layer l into P = a1*C - a2*S,
+//    R = a2*C + a1*S, E (as coef_kernel) and writes them as MFMA B operands:
 // bmat[(((b*L + l)*Hkv + head)*QG + g)*6 + o][lane][8] bf16.  Group g holds query heads
 // 4g..4g+3 of the KV head.  Operand o: 0..3 the key slabs of MFMA o, 4 and 5 the magnitudes
 // of pair sets 0 and 1.  Lane (j = lane % 16, kb): column j = (query head 4g + j % 4, split
-// j / 4); element e = k index kb*8 + e of the slab.
+// j / 4); element e = k index kb*8 + e of the slab.  Piece `split` of a coefficient x is
+// what is left of x after `split` roundings to bf16 (x = x1 + x2 + x3).
+constexpr int kPrepThreads = 1024;
+constexpr int kPrepHeads = 64;      // query heads whose coefficients are staged at a time
+constexpr int kPrepPitch = 193;
+
 template <int DT, bool IL>
-__global__ void coef_mfma_kernel(const float* coef, int Hkv, int G, int A, int QG, int64_t n_heads_total,
-                                 uint4* bmat) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (head instance, group, operand, lane)
-  if (idx >= n_heads_total * QG * 6 * 64) return;
-  const int lane = (int)(idx % 64);
-  const int o = (int)((idx / 64) % 6);
-  const int g = (int)((idx / (64 * 6)) % QG);
-  const int64_t hi = idx / (64 * 6 * QG);            // (b*L + l)*Hkv + head
-  const int head = (int)(hi % Hkv);
-  const int64_t bl = hi / Hkv;
-  const int j = lane & 15, kb = lane >> 4;
-  const int q = 4 * g + (j & 3), sp = j >> 2;
-  uint32_t out[4] = {0, 0, 0, 0};
-  if (q < G && sp < 3) {
-    const float* c = coef + ((bl * A + (int64_t)head * G + q) * 3) * 64;   // [P | R | E][64]
-    float v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      int which, pair;   // which: 0 = P, 1 = R, 2 = E
-      if (o < 4) {
-        const int el = slab_elem<DT>(o, kb, e);
-        if (IL) { which = el & 1; pair = el >> 1; }
-        else { which = el >= 64 ? 1 : 0; pair = el & 63; }
-      } else {
-        which = 2;
-        const int set = o - 4;
-        // interleaved: pairs of MFMAs 2*set and 2*set + 1; half: real parts of MFMA `set`
-        if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
-        else pair = slab_elem<DT>(set, kb, e) & 63;
-      }
-      float x = c[which * 64 + pair];
-      // piece sp of x = x1 + x2 + x3 (each bf16, round to nearest even)
-      for (int s = 0; s < sp; ++s) x = x - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x) << 16);
-      v[e] = x;
+__global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* folded, const float* omega,
+                                                                 const float* offsets, int NO,
+                                                                 const int32_t* round_start, int L, int Hkv, int G,
+                                                                 int A, int QG, uint4* bmat,
+                                                                 unsigned long long* xchg, int64_t words,
+                                                                 uint32_t* status) {
+  // One buffer, used twice: the per-offset cos / sin values, then the coefficients of up to
+  // kPrepHeads query heads as [head][P | R | E][64] with a row pitch of 193 floats (the four
+  // query heads and four k blocks a wave reads at once then fall into 16 different banks).
+  __shared__ float buf[kPrepHeads * kPrepPitch];
+  __shared__ float mean_cs[2][64];
+  static_assert(kPrepHeads * kPrepPitch >= 2 * kMaxOffsets * 64, "the trig values must fit the buffer");
+  float (*part)[kMaxOffsets][64] = reinterpret_cast<float (*)[kMaxOffsets][64]>(buf);
+  const int l = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int64_t wg = (int64_t)b * gridDim.x + l, nwg = (int64_t)gridDim.x * gridDim.y;
+  for (int64_t i = wg * kPrepThreads + tid; i < words; i += nwg * kPrepThreads) xchg[i] = 0ull;
+  if (wg == 0 && tid == 0) *status = 0u;
+
+  const float rs = (float)round_start[b];
+  for (int i = tid; i < NO * 64; i += kPrepThreads) {
+    const int j = i >> 6, f = i & 63;
+    phase_cos_sin(__fmul_rn(__fadd_rn(rs, offsets[j]), omega[f]), part[0][j][f], part[1][j][f]);
+  }
+  __syncthreads();
+  if (tid < 128) {
+    const int which = tid >> 6, f = tid & 63;
+    double sum = 0.0;
+    for (int j = 0; j < NO; ++j) sum += part[which][j][f];
+    mean_cs[which][f] = (float)(sum / NO);
+  }
+
+  const int heads_per_pass = max(1, kPrepHeads / G);        // whole KV heads
+  for (int head0 = 0; head0 < Hkv; head0 += heads_per_pass) {
+    const int nh = min(heads_per_pass, Hkv - head0);
+    __syncthreads();                                        // means written; buffer free
+    // P = a1*C - a2*S, R = a2*C + a1*S, E, of query heads head0*G .. (head0 + nh)*G - 1
+    const float* in = folded + ((int64_t)l * A + (int64_t)head0 * G) * 3 * 64;   // [head][a1 | a2 | e][64]
+    for (int i = tid; i < nh * G * 64; i += kPrepThreads) {
+      const int q = i >> 6, f = i & 63;
+      const float a1 = in[q * 192 + f], a2 = in[q * 192 + 64 + f], e = in[q * 192 + 128 + f];
+      const float c = mean_cs[0][f], sn = mean_cs[1][f];
+      buf[q * kPrepPitch + f] = fmaf(a1, c, -a2 * sn);
+      buf[q * kPrepPitch + 64 + f] = fmaf(a2, c, a1 * sn);
+      buf[q * kPrepPitch + 128 + f] = e;
     }
+    __syncthreads();
+    const int items = nh * QG * 6 * 64;                     // (head, group, operand, lane)
+    uint4* out_base = bmat + (((int64_t)b * L + l) * Hkv + head0) * QG * 6 * 64;
+    for (int idx = tid; idx < items; idx += kPrepThreads) {
+      const int lane = idx & 63;
+      const int o = (idx >> 6) % 6;
+      const int g = (idx / (64 * 6)) % QG;
+      const int head = idx / (64 * 6 * QG);
+      const int j = lane & 15, kb = lane >> 4;
+      const int q = 4 * g + (j & 3), sp = j >> 2;
+      uint32_t out[4] = {0, 0, 0, 0};
+      if (q < G && sp < 3) {
+        const float* c = buf + (head * G + q) * kPrepPitch;
+        float v[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const f32x2 x = {v[2 * e], v[2 * e + 1]};
-      out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+        for (int e = 0; e < 8; ++e) {
+          int which, pair;   // which: 0 = P, 1 = R, 2 = E
+          if (o < 4) {
+            const int el = slab_elem<DT>(o, kb, e);
+            if (IL) { which = el & 1; pair = el >> 1; }
+            else { which = el >= 64 ? 1 : 0; pair = el & 63; }
+          } else {
+            which = 2;
+            const int set = o - 4;
+            // interleaved: pairs of MFMAs 2*set and 2*set + 1; half: real parts of MFMA `set`
+            if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
+            else pair = slab_elem<DT>(set, kb, e) & 63;
+          }
+          float x = c[which * 64 + pair];
+          for (int s = 0; s < sp; ++s) x = x - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x) << 16);
+          v[e] = x;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const f32x2 x = {v[2 * e], v[2 * e + 1]};
+          out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+        }
+      }
+      out_base[idx] = uint4{out[0], out[1], out[2], out[3]};
     }
   }
-  bmat[idx] = uint4{out[0], out[1], out[2], out[3]};
 }
 
 // QG: groups of four query heads per KV head (1 or 2).
@@ -609,7 +664,7 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.block_table = a.block_table;
   k.seq_lens = a.seq_lens;
   k.prefill_lens = a.prefill_lens;
-  k.coef = a.coef;
+  k.coef = nullptr;   // this kernel takes its coefficients from bmat
   k.xchg = a.xchg;
   k.fin = a.fin;
   k.status = a.status;
@@ -625,28 +680,24 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.seq_launch = a.pack;
   k.seq_wg_base = a.pack + a.B;
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
-  hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div64(words, 256)), dim3(256), 0, s, a.xchg, words,
-                     a.status);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
-  const int64_t heads_total = (int64_t)a.B * a.L * a.Hkv;
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
   const int QG = a.G > 4 ? 2 : 1;
-  const unsigned cgrid = (unsigned)ceil_div64(heads_total * QG * 6 * 64, 256);
   const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
   if (a.kv_dtype != TRI_KV_BF16 && !fp8) return hipErrorInvalidValue;
-  auto coef_launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(cgrid), dim3(256), 0, s, a.coef, a.Hkv, a.G, a.A, QG, heads_total, bmat);
+  if (a.NO <= 0 || a.NO > kMaxOffsets || a.D != 128) return hipErrorInvalidValue;
+  auto prep_launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)a.L, (unsigned)a.B), dim3(kPrepThreads), 0, s, a.folded, a.omega,
+                       a.offsets, a.NO, a.round_start, a.L, a.Hkv, a.G, a.A, QG, bmat, a.xchg, words, a.status);
   };
   if (fp8) {
-    if (il) coef_launch(coef_mfma_kernel<TRI_KV_FP8_E4M3, true>);
-    else coef_launch(coef_mfma_kernel<TRI_KV_FP8_E4M3, false>);
+    if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, true>);
+    else prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, false>);
   } else {
-    if (il) coef_launch(coef_mfma_kernel<TRI_KV_BF16, true>);
-    else coef_launch(coef_mfma_kernel<TRI_KV_BF16, false>);
+    if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true>);
+    else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false>);
   }
-  e = hipGetLastError();
+  hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
     return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)

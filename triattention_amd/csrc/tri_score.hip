@@ -511,9 +511,7 @@ __global__ void fold_stats_kernel(const float* qr, const float* qi, const float*
   o[2 * F + f] = s * coef;
 }
 
-// cos/sin of the fp32-rounded phase t*w, evaluated in double and rounded once:
-// the correctly rounded value of what torch.cos(t * omega) approximates in fp32
-// (core/scoring.py:322-324).
+// cos/sin of the fp32-rounded phase t*w per offset (phase_cos_sin) and their means over the offsets.
 __global__ void trig_kernel(const float* omega, const float* offsets, int NO, const int32_t* round_start,
                             int F, float* trig, float* mean_cs) {
   const int b = blockIdx.x, f = threadIdx.x;
@@ -523,8 +521,8 @@ __global__ void trig_kernel(const float* omega, const float* offsets, int NO, co
   double sc = 0.0, ss = 0.0;
   for (int j = 0; j < NO; ++j) {
     const float t = __fadd_rn(rs, offsets[j]);
-    const double ph = (double)__fmul_rn(t, w);
-    const float c = (float)cos(ph), s = (float)sin(ph);
+    float c, s;
+    phase_cos_sin(__fmul_rn(t, w), c, s);
     if (trig) {
       trig[((int64_t)(b * NO + j) * 2 + 0) * F + f] = c;
       trig[((int64_t)(b * NO + j) * 2 + 1) * F + f] = s;

