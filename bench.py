@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=1, help="BASELINE.json config index (default 1)")
+    ap.add_argument("--config", type=int, default=1, help="workload index 0..4 (default 1: 36 layers, 16 x 16384 tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=36, help="layers of one sequence the CPU baseline scores")
     ap.add_argument("--seq-len", type=int, default=0,

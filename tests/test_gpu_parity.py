@@ -414,7 +414,7 @@ def test_compress_step_equals_chained_calls():
 
 
 def test_end_to_end_c0_against_oracle():
-    """BASELINE config 0: score, select at budget 2048, compact; kept K/V bit-exact."""
+    """One layer, one sequence of 4096 tokens: score, select at budget 2048, compact; kept K/V bit-exact."""
     w = synth.config(0)
     inp = build_inputs(w)
     caches, kv, batch, sc = device_objects(w, inp, DEV)
