@@ -120,9 +120,10 @@ uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
 
 /* Byte offset inside the workspace of a 32-bit status word: tri_select_paged and
  * tri_compress_step clear it and the resident kernel sets it to non-zero if one of its
- * bounded waits on another workgroup expired (results are then invalid).  The caller
- * may read it after synchronising the stream.  Host-only; no counterpart in the
- * reference. */
+ * bounded waits on another workgroup expired (results are then invalid; the compaction
+ * inside tri_compress_step sees the word and moves nothing, so the cache is intact and
+ * the caller can repeat the step with TRIATTN_RESIDENT_KERNEL=off).  The caller may read
+ * it after synchronising the stream.  Host-only; no counterpart in the reference. */
 uint64_t tri_workspace_status_offset(const tri_kv_layout* kv, const tri_batch* batch,
                                      const tri_score_params* sp);
 

@@ -638,6 +638,35 @@ def test_compress_step_replays_from_a_hip_graph():
             assert torch.equal(c.view(torch.int16), wc.view(torch.int16)), rep
 
 
+@pytest.mark.parametrize("kernel", ["mfma", "valu"])
+def test_expired_wait_raises_the_status_word_and_the_step_leaves_the_cache_alone(kernel, monkeypatch):
+    """The resident kernels' failure path, forced from the host: with a negative wait limit every
+    wait on another workgroup gives up at once, all workgroups still run to their end, the status
+    word reads non-zero and the compaction of compress_step moves nothing.  The same call
+    without the limit then gives the result of the chained calls."""
+    w, inp, caches, kv, batch, sc = _resident_batch(21)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_" + kernel
+    before = [c.clone() for c in caches]
+    monkeypatch.setenv("TRIATTN_RESIDENT_SPIN_TICKS", "-1")
+    print(f"forced expiry, kernel={kernel}", flush=True)
+    _, ws = ops.compress_step(kv, batch, sc, sel)
+    assert ws.status() != 0
+    for c, c0 in zip(caches, before):
+        assert torch.equal(c.view(torch.int16), c0.view(torch.int16))
+    monkeypatch.delenv("TRIATTN_RESIDENT_SPIN_TICKS")
+    keep, ws = ops.compress_step(kv, batch, sc, sel, ws=ws)
+    assert ws.status() == 0
+    caches2, kv2, batch2, sc2 = device_objects(w, inp, DEV)
+    keep2, _, ws2 = ops.select_paged(kv2, batch2, sc2, sel)
+    ops.compact(kv2, batch2, keep2)
+    torch.cuda.synchronize()
+    assert torch.equal(keep, keep2)
+    for c, c2 in zip(caches, caches2):
+        assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
+
+
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
     for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=64), {}),

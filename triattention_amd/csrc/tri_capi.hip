@@ -445,6 +445,9 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
   tri::CompactLaunch c{};
   rc = fill_compact(kv, batch, keep, sel->layer_reduce < 0, sel->shared, c);
   if (rc) return rc;
+  // A resident kernel whose bounded wait expired leaves meaningless keep lists and a raised
+  // status word: the compaction kernels look at that word and then leave the cache alone.
+  c.guard = at<uint32_t>(workspace, w.status);
   return launch_status(tri::launch_compact(c, s), "compact");
 }
 

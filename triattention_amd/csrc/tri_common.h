@@ -144,6 +144,10 @@ struct FusedLaunch {
   float* fin;                    // [B*Hkv][Tmax]
   FusedPlan plan;
 };
+// Limit of the resident kernels' waits on other workgroups, in ticks of the 100 MHz wall
+// clock: 2 s, or TRIATTN_RESIDENT_SPIN_TICKS (tests: a negative value makes every wait give
+// up at once, which raises the status word while every workgroup still runs to its end).
+long long resident_spin_ticks();
 hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s);
 hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s);
 
@@ -162,6 +166,7 @@ struct CompactLaunch {
   const int32_t* keep;
   int Tmax;
   void* staging;       // full-permutation mode only
+  const uint32_t* guard;   // optional: a device word; the kernels move nothing when it is non-zero
 };
 hipError_t launch_compact(const CompactLaunch& a, hipStream_t s);
 

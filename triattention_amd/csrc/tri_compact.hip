@@ -45,6 +45,7 @@ struct CompactArgs {
   const int32_t* seq_lens;
   const int32_t* budgets;
   const int32_t* keep;
+  const uint32_t* guard;   // optional; non-zero word: move nothing
   int64_t stride_block_b, stride_token_b, stride_head_b;   // bytes
   uint32_t block_units, token_units, head_units;           // the same strides in 16-byte units
   int B, L, Hkv, block_size, bs_shift, block_table_pitch, max_budget;
@@ -71,6 +72,12 @@ __device__ __forceinline__ uint32_t slot_units(const CompactArgs& a, const int32
 
 constexpr uint32_t kNoSource = 0xffffffffu;
 
+// The keep lists of a step come from a resident kernel whose waits are bounded; when one
+// expired the lists are meaningless, and the step's compaction must not touch the cache.
+__device__ __forceinline__ bool guard_raised(const uint32_t* guard) {
+  return guard && __hip_atomic_load(guard, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+}
+
 // Ordered pass: the slots whose source token lies inside the kept prefix [0, k).  With keep
 // ascending they form a prefix of every list, and only they can be overwritten before they
 // are read.  One workgroup owns one (sequence, layer, K or V, group of keep lists) and moves
@@ -83,6 +90,7 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
   __shared__ uint32_t src_units[kSegEntries];   // [slot][list], kNoSource: not this pass's
   __shared__ uint32_t dst_units[kSegEntries];   // [slot]
   __shared__ int prefix_len[256];
+  if (guard_raised(a.guard)) return;
 
   // workgroup -> (sequence, layer, K or V, group of lists)
   const int all_lists = a.shared ? 1 : a.Hkv;
@@ -218,6 +226,7 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
 // (workgroups stride over the tiles, so a grid smaller than the number of tiles is
 // still complete).
 __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactArgs a) {
+  if (guard_raised(a.guard)) return;
   int sidx = blockIdx.y;
   const int kv = sidx % 2; sidx /= 2;
   const int l = sidx % a.L;
@@ -289,6 +298,7 @@ struct ScaleArgs {
   const int32_t* seq_lens;
   const int32_t* budgets;
   const int32_t* keep;
+  const uint32_t* guard;
   int B, L, Hkv, block_size, block_table_pitch, max_budget, keep_per_layer, shared;
 };
 
@@ -302,6 +312,7 @@ __global__ __launch_bounds__(256) void compact_scales_kernel(ScaleArgs a) {
   // writes (barrier); a later tile reads sources at or beyond its own first slot, which
   // earlier tiles (writing below that slot) never touch.
   constexpr int kScalesPerThread = 8;
+  if (guard_raised(a.guard)) return;
   int sidx = blockIdx.x;
   const int kv = sidx % 2; sidx /= 2;
   const int l = sidx % a.L;
@@ -441,6 +452,7 @@ CompactArgs make_args(const CompactLaunch& a) {
   c.seq_lens = a.seq_lens;
   c.budgets = a.budgets;
   c.keep = a.keep;
+  c.guard = a.guard;
   c.stride_block_b = a.stride_block * a.elem_bytes;
   c.stride_token_b = a.stride_token * a.elem_bytes;
   c.stride_head_b = a.stride_head * a.elem_bytes;
@@ -476,6 +488,7 @@ hipError_t launch_scales(const CompactLaunch& a, hipStream_t s) {
   sa.seq_lens = a.seq_lens;
   sa.budgets = a.budgets;
   sa.keep = a.keep;
+  sa.guard = a.guard;
   sa.B = a.B; sa.L = a.L; sa.Hkv = a.Hkv;
   sa.block_size = a.block_size;
   sa.block_table_pitch = a.block_table_pitch;

@@ -25,6 +25,8 @@
 // launch never has more workgroups than the device has CUs (workgroups that must queue
 // behind another stream's kernels start late, they are never starved).  Every wait is
 // also bounded in time and raises a status word instead of spinning forever.
+#include <cstdlib>
+
 #include "tri_common.h"
 #include "tri_score_device.h"
 #include "tri_fused_device.h"
@@ -455,6 +457,12 @@ FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, i
   return p;
 }
 
+long long resident_spin_ticks() {
+  const char* v = std::getenv("TRIATTN_RESIDENT_SPIN_TICKS");
+  if (v && *v) return std::atoll(v);
+  return 200000000LL;
+}
+
 hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s) {
   FusedArgs k{};
   k.k_layers = a.k_layers;
@@ -474,7 +482,7 @@ hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s) {
   k.seq_base = 0; k.num_seqs = a.B; k.Tmax = a.Tmax;
   k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
   k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
-  k.spin_ticks = 200000000LL;   // 2 s of the 100 MHz wall clock
+  k.spin_ticks = resident_spin_ticks();
   k.seq_launch = a.pack;
   k.seq_wg_base = a.pack + a.B;
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;

@@ -162,6 +162,10 @@ __device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, in
   const unsigned long long* in = a.xchg + ((int64_t)(b * a.L + l) * a.tiles_per_seq * a.A + ah0) * 2;
   const uint32_t want = (uint32_t)(l + 1);
   const long long t_begin = wall_clock64();
+  if (a.spin_ticks < 0 && !aborted) {   // set by the host to exercise the failure path: give up without waiting
+    aborted = true;
+    if (lane == 0) atomicExch(a.status, 1u);
+  }
   for (int base = 0; base < items; base += 64) {
     const int item = base + lane;
     const bool live = item < items;

@@ -676,7 +676,7 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.seq_base = 0; k.num_seqs = a.B; k.Tmax = a.Tmax;
   k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
   k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
-  k.spin_ticks = 200000000LL;   // 2 s of the 100 MHz wall clock
+  k.spin_ticks = resident_spin_ticks();
   k.seq_launch = a.pack;
   k.seq_wg_base = a.pack + a.B;
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
