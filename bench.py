@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--two-pass", action="store_true",
                     help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
     ap.add_argument("--hook-latency", action="store_true",
-                    help="also time the runner hook (triattention_apply_compression) for one request of "
+                    help="also time the runner hook for one request and the batch hook for a batch of requests of "
                          "budget + 128 tokens, host side included")
     ap.add_argument("--query-stats", action="store_true",
                     help="also time the calibration statistics kernel on one layer's captured queries "
@@ -96,10 +96,12 @@ def cpu_baseline(w, layers: int):
                       f"rate scaled to all {w.num_layers} layers"}
 
 
-def hook_latency(w, dev, calls: int = 30):
-    """Wall time of one call of the runner hook for a single request of budget + 128 tokens
-    (the steady state of a long generation): host logic, launches and the two host reads of
-    the keep-index check, synchronised before and after."""
+def hook_latency(w, dev, calls: int = 30, requests: int = 1):
+    """Wall time of the runner hook for requests of budget + 128 tokens (the steady state of a
+    long generation): host logic, launches and host reads, synchronised before and after.
+    One request: one call of ``triattention_apply_compression``.  Several: the same requests
+    through one call of ``triattention_apply_compression_batch`` and, for comparison, through
+    the one-by-one hook in a loop."""
     import tempfile
     import types
     from triattention_amd import synth
@@ -118,38 +120,55 @@ def hook_latency(w, dev, calls: int = 30):
                     "stats": entries}, path)
         cfg = TriAttentionRuntimeConfig(kv_budget=w.budget, divide_length=128, window_size=w.window_size,
                                         sparse_stats_path=path, log_decisions=False)
-        nblk = (t + w.block_size - 1) // w.block_size + 8
-        ids = torch.randperm(nblk + 64, generator=torch.Generator().manual_seed(1))[:nblk].tolist()
+        per_req = (t + w.block_size - 1) // w.block_size + 8
+        nblk = per_req * requests
+        perm = torch.randperm(nblk + 64, generator=torch.Generator().manual_seed(1))[:nblk].tolist()
+        ids = {f"r{i}": perm[i * per_req:(i + 1) * per_req] for i in range(requests)}
         caches = [torch.randn(2, nblk + 64, w.block_size, w.num_kv_heads, w.head_dim, device=dev).to(torch.bfloat16)
                   for _ in range(w.num_layers)]
-        req = types.SimpleNamespace(num_computed_tokens=t, block_ids=(list(ids),))
-        runner = types.SimpleNamespace(requests={"r": req}, kv_caches=caches,
+        reqs = {rid: types.SimpleNamespace(num_computed_tokens=t, block_ids=(list(b),)) for rid, b in ids.items()}
+        runner = types.SimpleNamespace(requests=reqs, kv_caches=caches,
                                        cache_config=types.SimpleNamespace(block_size=w.block_size))
         install_runner_compression_hook(runner, cfg)
-        sched = types.SimpleNamespace(num_scheduled_tokens={"r": 1})
+        sched = types.SimpleNamespace(num_scheduled_tokens={rid: 1 for rid in reqs})
 
-        def call():
-            req.num_computed_tokens = t
-            req.block_ids = (list(ids),)
-            sig = CompressionSignal(req_id="r", should_compress=True, reason="length_threshold",
-                                    estimated_cache_len=t + 1, step=1, kv_usage=None, protect_prefill=False,
-                                    prefill_len=0, scheduled_tokens=1)
-            return runner.triattention_apply_compression(req_id="r", signal=sig, scheduler_output=sched)
+        def signals():
+            for rid, req in reqs.items():
+                req.num_computed_tokens = t
+                req.block_ids = (list(ids[rid]),)
+            return {rid: CompressionSignal(req_id=rid, should_compress=True, reason="length_threshold",
+                                           estimated_cache_len=t + 1, step=1, kv_usage=None, protect_prefill=False,
+                                           prefill_len=0, scheduled_tokens=1) for rid in reqs}
 
-        for _ in range(3):
-            res = call()
-        if not res["applied"]:
-            raise RuntimeError(f"hook did not compress: {res}")
-        times = []
-        for _ in range(calls):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            call()
-            torch.cuda.synchronize()
-            times.append((time.perf_counter() - t0) * 1e3)
-    times.sort()
-    return {"tokens": t, "budget": w.budget, "layers": w.num_layers, "calls": calls,
-            "ms_median": times[len(times) // 2], "ms_min": times[0], "ms_max": times[-1]}
+        def one_by_one():
+            return [runner.triattention_apply_compression(req_id=rid, signal=sig, scheduler_output=sched)
+                    for rid, sig in signals().items()]
+
+        def together():
+            return list(runner.triattention_apply_compression_batch(signals=signals(), scheduler_output=sched).values())
+
+        def timed(fn):
+            for _ in range(3):
+                res = fn()
+            if not all(r["applied"] for r in res):
+                raise RuntimeError(f"hook did not compress: {res}")
+            times = []
+            for _ in range(calls):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                fn()
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t0) * 1e3)
+            times.sort()
+            return {"ms_median": times[len(times) // 2], "ms_min": times[0], "ms_max": times[-1]}
+
+        out = {"requests": requests, "tokens": t, "budget": w.budget, "layers": w.num_layers, "calls": calls}
+        if requests == 1:
+            out.update(timed(one_by_one))
+        else:
+            out["batch_hook"] = timed(together)
+            out["one_by_one"] = timed(one_by_one)
+    return out
 
 
 def query_stats_leg(dev, heads: int = 32, tokens: int = 32768, dim: int = 128, calls: int = 20):
@@ -356,6 +375,7 @@ def main() -> int:
         out["query_stats"] = query_stats_leg(dev)
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
+        out["hook_batch_call"] = hook_latency(w, dev, calls=20, requests=len(w.seq_lens))
     if not args.no_cpu_baseline:
         del saved, caches, pool
         torch.cuda.empty_cache()

@@ -208,6 +208,100 @@ def test_runner_hook_end_to_end(tmp_path):
     assert again["applied"] is False and again["reason"] == "under_budget"
 
 
+def _fake_runner(w, inp, tmp_path, **cfg_kw):
+    """A runner with one request per sequence of the workload, all in one paged pool."""
+    from triattention_amd import synth
+    _write_stats(tmp_path / "s.pt", inp["qc"], inp["qa"], inp["omega"], w.head_dim)
+    cfg = TriAttentionRuntimeConfig(kv_budget=w.budget, divide_length=16, window_size=w.window_size,
+                                    sparse_stats_path=tmp_path / "s.pt", **cfg_kw)
+    caches = [c.to(DEV) for c in inp["caches"]]
+    reqs = {f"r{b}": types.SimpleNamespace(num_computed_tokens=t, block_ids=([int(x) for x in inp["tables"][b]],))
+            for b, t in enumerate(w.seq_lens)}
+    runner = types.SimpleNamespace(requests=reqs, kv_caches=caches,
+                                   cache_config=types.SimpleNamespace(block_size=w.block_size))
+    install_runner_compression_hook(runner, cfg)
+    sched = types.SimpleNamespace(num_scheduled_tokens={rid: 1 for rid in reqs})
+    signals = {f"r{b}": _signal(req_id=f"r{b}", estimated_cache_len=t + 1, prefill_len=7 + b)
+               for b, t in enumerate(w.seq_lens)}
+    return runner, reqs, caches, sched, signals
+
+
+def test_batch_hook_equals_the_hook_called_request_by_request(tmp_path, monkeypatch):
+    """All triggered requests of a step through ``triattention_apply_compression_batch``: same
+    result dictionaries, same truncated block lists and bit-identical caches as the
+    one-by-one hook (same kernels: the resident kernel is switched off for this comparison).
+    One request is under budget and one asks for the prefill guard."""
+    from helpers import build_inputs
+    from triattention_amd import synth
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    w = synth.Workload(name="t", num_layers=3, num_q_heads=8, num_kv_heads=2, head_dim=128,
+                       seq_lens=(300, 1000, 97, 513, 60), budget=96, block_size=16, window_size=12, rope_theta=1e6,
+                       index=31)
+    inp = build_inputs(w)
+    one = _fake_runner(w, inp, tmp_path)
+    two = _fake_runner(w, inp, tmp_path)
+    for _, _, _, _, signals in (one, two):
+        signals["r3"] = _signal(req_id="r3", estimated_cache_len=514, prefill_len=40, protect_prefill=True)
+    runner, reqs, caches, sched, signals = one
+    want = {rid: RunnerHookCompressionExecutor(runner).execute(rid, sig, sched) for rid, sig in signals.items()}
+    runner2, reqs2, caches2, sched2, signals2 = two
+    got = RunnerHookCompressionExecutor(runner2).execute_batch(signals2, sched2)
+    torch.cuda.synchronize()
+    assert list(got) == list(want)
+    for rid in want:
+        assert got[rid] == want[rid], rid
+        assert reqs2[rid].block_ids == reqs[rid].block_ids
+    assert want["r4"].reason == "under_budget" and want["r0"].applied and want["r0"].cache_len_after == 96
+    for a, b in zip(caches, caches2):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # a second step right away: everything deferred, nothing launched
+    again = RunnerHookCompressionExecutor(runner2).execute_batch(
+        {rid: _signal(req_id=rid, estimated_cache_len=98) for rid in signals2}, sched2)
+    assert all(not r.applied and r.reason == "under_budget" for r in again.values())
+
+
+def test_batch_hook_on_the_resident_kernel(tmp_path, monkeypatch):
+    """Sixteen requests of 3072 tokens fill the chip: the batch hook runs the resident kernel;
+    result equal to the library calls on the same batch, and, when the resident launch is made to
+    fail, to the one-by-one path (the caches were not touched by the failed step)."""
+    from helpers import build_inputs
+    from triattention_amd import ops, synth
+    w = synth.Workload(name="t", num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128, seq_lens=(3072,) * 16,
+                       budget=256, block_size=16, window_size=12, rope_theta=1e6, index=32)
+    inp = build_inputs(w)
+    runner, reqs, caches, sched, signals = _fake_runner(w, inp, tmp_path)
+    got = RunnerHookCompressionExecutor(runner).execute_batch(signals, sched)
+    torch.cuda.synchronize()
+    assert all(r.applied and r.cache_len_after == 256 for r in got.values())
+    ref = [c.to(DEV) for c in inp["caches"]]
+    kv = ops.PagedKV.from_kv_caches(ref)
+    batch = ops.StepBatch(DEV, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=inp["tables"],
+                          prefill_lens=[0] * 16)
+    sc = ops.ScoreConfig(ops.fold_stats(inp["qc"].to(DEV), inp["qa"].to(DEV), inp["fs"].to(DEV)),
+                         inp["omega"].to(DEV), inp["offsets"].to(DEV))
+    sel = ops.SelectConfig(window_size=w.window_size)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    _, ws = ops.compress_step(kv, batch, sc, sel)
+    assert ws.status() == 0
+    for a, b in zip(caches, ref):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for b in range(16):
+        assert reqs[f"r{b}"].block_ids == ([int(x) for x in inp["tables"][b]][:16],)
+
+    # forced failure of the resident launch: the hook repeats the step request by request
+    runner_f, reqs_f, caches_f, sched_f, signals_f = _fake_runner(w, inp, tmp_path)
+    monkeypatch.setenv("TRIATTN_RESIDENT_SPIN_TICKS", "-1")
+    failed = RunnerHookCompressionExecutor(runner_f).execute_batch(signals_f, sched_f)
+    monkeypatch.delenv("TRIATTN_RESIDENT_SPIN_TICKS")
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    runner_s, reqs_s, caches_s, sched_s, signals_s = _fake_runner(w, inp, tmp_path)
+    single = {rid: RunnerHookCompressionExecutor(runner_s).execute(rid, sig, sched_s) for rid, sig in signals_s.items()}
+    torch.cuda.synchronize()
+    assert failed == single
+    for a, b in zip(caches_f, caches_s):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
 def test_dense_scoring_api_against_reference_scores():
     gold = load_golden("scoring_pytorch.pt")
     for name, style in (("d128_half", "half"), ("d64_inter", "interleaved")):

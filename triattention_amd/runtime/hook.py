@@ -11,6 +11,7 @@ access is used on the runner, so any object with ``requests``, ``kv_caches`` and
 """
 from __future__ import annotations
 
+import os
 import re
 from dataclasses import dataclass
 from typing import Any, Callable
@@ -22,9 +23,9 @@ from .kv_compaction import (build_keep_token_indices, compact_request_kv_in_plac
                             compact_request_kv_in_place_per_head, gather_request_k_dense,
                             register_kv_layout_axis_hint)
 from .models import TRITON_SCORING_REQUIRED_MARKER as MARK, CompressionSignal
-from .pipeline import (finalize_hook_placement_result, normalize_mutable_block_ids_by_group,
-                       run_group_compaction_pipeline)
-from .selector import build_triattention_selector as _build_triattention_selector
+from .pipeline import (GroupPipelineOutcome, finalize_hook_placement_result, normalize_mutable_block_ids_by_group,
+                       num_required_blocks, run_group_compaction_pipeline, truncate_tail_reclaim_group)
+from .selector import ResidentLaunchFailed, build_triattention_selector as _build_triattention_selector
 
 
 # --------------------------------------------------------------- executor side
@@ -61,6 +62,26 @@ class RunnerHookCompressionExecutor(CompressionExecutor):
             return CompressionExecutionResult(bool(d.get("applied", False)), str(d.get("reason", "runner_hook_result")),
                                               d.get("cache_len_after"), d)
         return CompressionExecutionResult(False, f"unsupported_hook_result:{type(out).__name__}")
+
+    batch_hook_name = "triattention_apply_compression_batch"
+
+    def execute_batch(self, signals: dict, scheduler_output) -> dict:
+        """All triggered requests of a step in one call (no counterpart in the reference, whose
+        runner walks them one by one, runtime/runner_compression_actions.py:24-70):
+        ``{req_id: CompressionExecutionResult}``.  Falls back to ``execute`` per request when
+        the runner carries no batch hook."""
+        hook = getattr(self._base_runner, self.batch_hook_name, None)
+        todo = {rid: sig for rid, sig in signals.items() if getattr(sig, "should_compress", True)}
+        if not callable(hook):
+            return {rid: self.execute(rid, sig, scheduler_output) for rid, sig in todo.items()}
+        out = hook(signals=todo, scheduler_output=scheduler_output)
+        results = {}
+        for rid in todo:
+            d = dict(out.get(rid) or {"applied": False, "reason": "runner_hook_result_missing"})
+            results[rid] = CompressionExecutionResult(bool(d.get("applied", False)),
+                                                      str(d.get("reason", "runner_hook_result")),
+                                                      d.get("cache_len_after"), d)
+        return results
 
 
 # ------------------------------------------------------------- request lookup
@@ -387,6 +408,26 @@ def build_hook_runtime_context(*, base_runner: Any, config: TriAttentionRuntimeC
                               int(recent) if isinstance(recent, int) else None, bool(defer))
 
 
+@dataclass
+class _Ready:
+    """A triggered request that passed every check in front of the kernels."""
+    req_id: str
+    signal: CompressionSignal
+    req_state: Any
+    ctx: HookRuntimeContext
+    original_ids: Any
+    mutable_ids: list
+    block_size: int
+    strict: bool
+
+
+def _debug_env_active() -> bool:
+    """Debug switches that only the one-by-one path implements."""
+    on = {"1", "true", "yes", "on"}
+    return bool(os.environ.get("TRIATTN_DEBUG_OVERRIDE_FIRST_KEEP_JSON", "").strip()) or \
+        os.environ.get("TRIATTN_DEBUG_FORCE_PRESERVE_DROPPED", "0").strip().lower() in on
+
+
 # ------------------------------------------------------------------- the hook
 def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeConfig) -> Callable[..., dict]:
     """runtime/hook_impl.py:30-165."""
@@ -396,8 +437,11 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
         select_layer, select_group, selector_status = _build_triattention_selector(config)
     group_tensors: dict | None = None
     compressed_once: set = set()
+    compress_batch = getattr(select_group, "_compress_batch", None) if select_group is not None else None
 
-    def _hook(req_id: str, signal: CompressionSignal, scheduler_output: Any) -> dict:
+    def _prepare(req_id: str, signal: CompressionSignal, scheduler_output: Any):
+        """Everything before the kernels: a result dictionary when the request is skipped,
+        else the facts the compaction needs."""
         nonlocal group_tensors
         setattr(base_runner, "_triattention_active_req_id", req_id)
         strict = bool(config.enable_experimental_kv_compaction and config.require_triton_scoring)
@@ -440,24 +484,151 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
         mutable_ids = normalize_mutable_block_ids_by_group(original_ids)
         if mutable_ids is None:
             return {"applied": False, "reason": "invalid_block_ids_container"}
-
         if group_tensors is None:
             group_tensors = resolve_group_tensors(base_runner)
+        return _Ready(req_id, signal, req_state, ctx, original_ids, mutable_ids, block_size, strict)
+
+    def _finish(r: "_Ready", out) -> dict:
+        if isinstance(out, dict):
+            return out
+        compressed_once.add(r.req_id)
+        return finalize_hook_placement_result(
+            req_state=r.req_state, original_block_ids_by_group=r.original_ids, config=config,
+            selector_status=str(selector_status), outcome=out, effective_tokens=r.ctx.effective_tokens,
+            budget_total=r.ctx.budget_total, recent_unabsorbed_tokens=r.ctx.recent_unabsorbed_tokens)
+
+    def _run_single(r: "_Ready") -> dict:
+        setattr(base_runner, "_triattention_active_req_id", r.req_id)
         out = run_group_compaction_pipeline(
-            req_id=req_id, signal=signal, config=config, strict_triton_required=strict,
-            num_computed_tokens=ctx.num_computed_tokens, effective_tokens=ctx.effective_tokens,
-            budget_total=ctx.budget_total, block_size=block_size, mutable_block_ids_by_group=mutable_ids,
+            req_id=r.req_id, signal=r.signal, config=config, strict_triton_required=r.strict,
+            num_computed_tokens=r.ctx.num_computed_tokens, effective_tokens=r.ctx.effective_tokens,
+            budget_total=r.ctx.budget_total, block_size=r.block_size, mutable_block_ids_by_group=r.mutable_ids,
             group_tensors=group_tensors, select_keep_indices=select_layer,
             select_keep_indices_for_group=select_group, shared_compact_fn=compact_request_kv_in_place,
             per_head_compact_fn=compact_request_kv_in_place_per_head, gather_dense_fn=gather_request_k_dense)
-        if isinstance(out, dict):
-            return out
-        compressed_once.add(req_id)
-        return finalize_hook_placement_result(
-            req_state=req_state, original_block_ids_by_group=original_ids, config=config,
-            selector_status=str(selector_status), outcome=out, effective_tokens=ctx.effective_tokens,
-            budget_total=ctx.budget_total, recent_unabsorbed_tokens=ctx.recent_unabsorbed_tokens)
+        return _finish(r, out)
 
+    def _hook(req_id: str, signal: CompressionSignal, scheduler_output: Any) -> dict:
+        ready = _prepare(req_id, signal, scheduler_output)
+        return ready if isinstance(ready, dict) else _run_single(ready)
+
+    def _batchable(r: "_Ready") -> bool:
+        """True when the one-by-one path would take the group selector and the ordered
+        per-head compaction for every KV-cache group of this request, with nothing that only
+        that path knows how to do (debug overrides, the keep-everything and prefill early outs)."""
+        if compress_batch is None or _debug_env_active():
+            return False
+        sig = r.signal
+        groups = 0
+        for gid, ids in enumerate(r.mutable_ids):
+            if not ids or not group_tensors.get(gid):
+                continue
+            total = min(r.ctx.effective_tokens, len(ids) * r.block_size)
+            if total <= 0:
+                continue
+            budget = min(r.ctx.budget_total, total)
+            if budget <= 0 or total <= budget:
+                return False
+            if sig.protect_prefill and config.include_prefill_in_budget and min(int(sig.prefill_len), total) > budget:
+                return False
+            groups += 1
+        return groups > 0
+
+    def _run_batch(batch: list) -> dict:
+        """One launch sequence per KV-cache group for all requests of ``batch``."""
+        cache_len = {r.req_id: None for r in batch}
+        reclaim = {r.req_id: [] for r in batch}
+        gids = sorted({gid for r in batch for gid, ids in enumerate(r.mutable_ids) if ids and group_tensors.get(gid)})
+        for gid in gids:
+            members, requests = [], []
+            for r in batch:
+                ids = r.mutable_ids[gid] if gid < len(r.mutable_ids) else None
+                if not ids:
+                    continue
+                total = min(r.ctx.effective_tokens, len(ids) * r.block_size)
+                if total <= 0:
+                    continue
+                members.append((r, ids, total))
+                requests.append(dict(block_ids=ids, total_tokens=total,
+                                     prefill_len=min(int(r.signal.prefill_len), total),
+                                     protect_prefill=bool(r.signal.protect_prefill),
+                                     round_start=int(max(0, r.ctx.num_computed_tokens)),
+                                     budget_total=min(r.ctx.budget_total, total)))
+            if not members:
+                continue
+            try:
+                selected = compress_batch(layer_kv=group_tensors[gid], block_size=batch[0].block_size,
+                                          requests=requests)
+            except ResidentLaunchFailed:
+                raise
+            except Exception as exc:
+                raise RuntimeError(f"{MARK}:batch:gid={gid}:global_per_head:{type(exc).__name__}") from exc
+            for (r, ids, total), res in zip(members, selected):
+                after = int(res["indices"].shape[1])
+                if cache_len[r.req_id] is not None and cache_len[r.req_id] != after:
+                    raise RuntimeError(f"{MARK}:inconsistent_cache_len_after:req={r.req_id}:gid={gid}:"
+                                       f"expected={cache_len[r.req_id]}:actual={after}")
+                cache_len[r.req_id] = after
+                if config.enable_experimental_block_reclaim:
+                    kept, removed, group = truncate_tail_reclaim_group(gid=gid, normalized_block_ids=ids,
+                                                                       cache_len_after=after,
+                                                                       block_size=r.block_size)
+                    if config.require_physical_reclaim:
+                        expected = max(0, num_required_blocks(total, r.block_size)
+                                       - num_required_blocks(after, r.block_size))
+                        if expected > 0 and len(removed) < expected:
+                            raise RuntimeError(f"{MARK}:physical_reclaim_missing:req={r.req_id}:gid={gid}:"
+                                               f"expected_removed>={expected}:actual_removed={len(removed)}:"
+                                               f"effective_tokens={total}:cache_len_after={after}")
+                    r.mutable_ids[gid] = list(kept)
+                    if group is not None:
+                        reclaim[r.req_id].append(group)
+        out = {}
+        for r in batch:
+            if cache_len[r.req_id] is None:
+                out[r.req_id] = {"applied": False, "reason": "no_compactable_groups"}
+                continue
+            out[r.req_id] = _finish(r, GroupPipelineOutcome(
+                cache_len_after=int(cache_len[r.req_id]), selection_mode="per_head:hf_aligned_global_per_head",
+                block_reclaim_groups=reclaim[r.req_id], mutable_block_ids_by_group=r.mutable_ids))
+        return out
+
+    def _batch_hook(signals: dict, scheduler_output: Any) -> dict:
+        """All triggered requests of a scheduler step at once: ``{req_id: result}`` with the
+        result dictionaries the one-by-one hook returns.  Requests that qualify (the default
+        per-head mode, something to drop) are scored, selected and compacted together, one
+        launch sequence per KV-cache group; the others go through the one-by-one path."""
+        results, together = {}, []
+        for req_id, signal in signals.items():
+            if not getattr(signal, "should_compress", True):
+                continue
+            ready = _prepare(req_id, signal, scheduler_output)
+            if isinstance(ready, dict):
+                results[req_id] = ready
+            elif _batchable(ready):
+                together.append(ready)
+            else:
+                results[req_id] = _run_single(ready)
+        if len(together) == 1:
+            results[together[0].req_id] = _run_single(together[0])
+        elif together:
+            try:
+                results.update(_run_batch(together))
+            except ResidentLaunchFailed:
+                # Nothing was moved.  Repeat on the kernels that do not wait for each other.
+                previous = os.environ.get("TRIATTN_RESIDENT_KERNEL")
+                os.environ["TRIATTN_RESIDENT_KERNEL"] = "off"
+                try:
+                    for r in together:
+                        results[r.req_id] = _run_single(r)
+                finally:
+                    if previous is None:
+                        os.environ.pop("TRIATTN_RESIDENT_KERNEL", None)
+                    else:
+                        os.environ["TRIATTN_RESIDENT_KERNEL"] = previous
+        return {req_id: results[req_id] for req_id in signals if req_id in results}
+
+    _hook.batch = _batch_hook
     return _hook
 
 
@@ -465,5 +636,6 @@ def install_runner_compression_hook(base_runner: Any, config: TriAttentionRuntim
     """Install the hook unless the runner already has one (runtime/hook_impl.py:174-185)."""
     if hasattr(base_runner, "triattention_apply_compression"):
         return
-    setattr(base_runner, "triattention_apply_compression",
-            make_runner_compression_hook(base_runner=base_runner, config=config))
+    hook = make_runner_compression_hook(base_runner=base_runner, config=config)
+    setattr(base_runner, "triattention_apply_compression", hook)
+    setattr(base_runner, RunnerHookCompressionExecutor.batch_hook_name, hook.batch)

@@ -75,6 +75,11 @@ class _DeviceStats:
         return out
 
 
+class ResidentLaunchFailed(RuntimeError):
+    """The resident kernel gave up waiting for its other workgroups (the GPU was shared with
+    another workload for seconds); nothing was compacted, the step can be repeated."""
+
+
 def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: Any | None = None):
     """(select_keep_indices, select_keep_indices_for_group, status)."""
     mode = config.pruning_mode
@@ -238,6 +243,57 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                 "group_agg_mode": agg, "debug_group_layer_indices": list(layer_ids),
                 "debug_recent_count": _recent_count(total_tokens)}
 
+    def _compress_group_batch(*, layer_kv: list, block_size: int, requests: list) -> list:
+        """Selection **and** compaction of several requests of one KV-cache group in one launch
+        sequence (no counterpart in the reference, which walks the requests one by one,
+        runner_compression_actions.py:24; per request the result equals what
+        ``_select_keep_indices_for_group_per_head`` followed by the per-head compaction gives).
+
+        ``layer_kv``: [(layer_idx, kv_cache)] of the group; ``requests``: one dict per request
+        with ``block_ids, total_tokens, prefill_len, protect_prefill, round_start, budget_total``
+        and ``total_tokens > budget_total > 0``.  Returns the selector result dictionaries in
+        request order; the caches then hold the kept rows in slots ``0..k-1``.  Raises
+        ``ResidentLaunchFailed`` with the caches untouched when a wait inside the resident
+        kernel expired."""
+        if mode != "per_head" or semantics != "hf_aligned_global_per_head":
+            raise RuntimeError("batched compression serves the per_head / hf_aligned_global_per_head mode only")
+        agg = os.environ.get("TRIATTN_RUNTIME_DEBUG_GROUP_PERHEAD_AGG_MODE", "mean").strip().lower()
+        if agg not in {"mean", "max"}:
+            agg = "mean"
+        layer_ids = tuple(int(li) for li, _ in layer_kv)
+        kv = _paged_kv([c for _, c in layer_kv])
+        if int(kv.block_size) != int(block_size):
+            raise RuntimeError("layers of one KV-cache group must share one block size")
+        score_heads, _ = _head_layout(kv.num_kv_heads)
+        st = _stats()
+        omega, offsets = st.vectors(kv.device)
+        sc = ops.ScoreConfig(st.folded(layer_ids, score_heads, kv.device), omega, offsets,
+                             config.sparse_score_aggregation)
+        totals = [int(r["total_tokens"]) for r in requests]
+        ks = [min(int(r["budget_total"]), t) for r, t in zip(requests, totals)]
+        if any(k <= 0 or k >= t for k, t in zip(ks, totals)):
+            raise RuntimeError("batched compression expects total_tokens > budget_total > 0")
+        guards = [int(r["prefill_len"]) if r["protect_prefill"] and int(r["prefill_len"]) > 0 else 0 for r in requests]
+        batch = ops.StepBatch(kv.device, totals, round_start=[int(r["round_start"]) for r in requests], budgets=ks,
+                              block_tables=[[int(x) for x in r["block_ids"]] for r in requests],
+                              prefill_lens=guards)
+        sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
+                               protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg)
+        resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
+        try:
+            keep, ws = ops.compress_step(kv, batch, sc, sel)
+        except Exception as exc:
+            raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
+        if resident and ws.status() != 0:
+            raise ResidentLaunchFailed("a wait inside the resident kernel expired; the caches were left untouched")
+        h = kv.num_kv_heads
+        return [{"mode": "per_head", "indices": keep[b * h:(b + 1) * h, :k].to(torch.long),
+                 "semantic": "hf_aligned_global_per_head", "group_agg_mode": agg,
+                 "debug_group_layer_indices": list(layer_ids), "debug_recent_count": _recent_count(t)}
+                for b, (k, t) in enumerate(zip(ks, totals))]
+
     setattr(_select_keep_indices, "_supports_paged", True)
     setattr(_select_keep_indices_for_group_per_head, "_supports_paged_group", True)
+    if mode == "per_head" and semantics == "hf_aligned_global_per_head":
+        setattr(_select_keep_indices_for_group_per_head, "_compress_batch", _compress_group_batch)
     return _select_keep_indices, _select_keep_indices_for_group_per_head, "enabled"
