@@ -57,7 +57,11 @@ typedef struct tri_kv_layout {
   const void* const* k_layers; /* device array [num_layers] of device pointers */
   const void* const* v_layers; /* device array [num_layers]; may be NULL for score-only calls */
   /* fp8 only: per-(token, head) fp32 dequantisation scales, element
-   * (l, p, o, h) at k_scale_layers[l] + (p*block_size + o)*num_kv_heads + h. */
+   * (l, p, o, h) at k_scale_layers[l] + (p*block_size + o)*num_kv_heads + h.
+   * v_scale_layers == NULL: the rows carry no scales of their own (a cache with one scale
+   * per tensor, as vLLM's fp8 KV cache); compaction then moves rows only, and
+   * k_scale_layers must still point to readable scales for the scorer (all ones; the
+   * entries of every layer may point to the same array). */
   const float* const* k_scale_layers;
   const float* const* v_scale_layers;
 } tri_kv_layout;

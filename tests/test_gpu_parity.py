@@ -795,6 +795,45 @@ def test_fp8_compaction_moves_scales_with_the_rows(shared):
             assert torch.equal(dev_s[:, blk, off], ref_s[:, blk, off]), (l, b)
 
 
+def test_fp8_cache_without_row_scales(monkeypatch):
+    """A cache with one scale per tensor (vLLM's fp8 KV cache; the codes sit in uint8 tensors):
+    the codes are scored as they are and compaction moves rows only.  Selection identical to the
+    one with explicit arrays of ones (that path is pinned against the oracle by the fp8 cases
+    above), on the two-pass kernels and on the resident one; kept rows bit-exact against the
+    oracle's compaction."""
+    w = small(kv_dtype="fp8", seq_lens=(300, 45, 1000), num_layers=2)
+    inp = build_inputs(w)
+    ones = [torch.ones_like(t) for t in inp["k_scales"]]
+    caches_a, kv_a, batch, sc = device_objects(w, dict(inp, k_scales=ones, v_scales=ones), DEV)
+    caches_b = [c.to(DEV).view(torch.uint8) for c in inp["caches"]]
+    kv_b = ops.PagedKV.from_kv_caches(caches_b, w.rope_style)
+    assert kv_b.struct.v_scale_layers is None or not kv_b.struct.v_scale_layers
+    sel = ops.SelectConfig(window_size=w.window_size)
+    for kernel in ("off", "mfma"):
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+        print(f"unscaled fp8, resident kernel setting {kernel}", flush=True)
+        keep_a, fin_a, _ = ops.select_paged(kv_a, batch, sc, sel, want_scores=True)
+        keep_b, fin_b, _ = ops.select_paged(kv_b, batch, sc, sel, want_scores=True)
+        torch.cuda.synchronize()
+        for b, t in enumerate(w.seq_lens):          # entries beyond a sequence's own budget / length are not written
+            rows, k = slice(b * w.num_kv_heads, (b + 1) * w.num_kv_heads), min(w.budget, t)
+            assert torch.equal(keep_a[rows, :k], keep_b[rows, :k]), (kernel, b)
+            assert torch.equal(fin_a[rows, :t], fin_b[rows, :t]), (kernel, b)
+    ops.compact(kv_b, batch, keep_b)
+    torch.cuda.synchronize()
+    h = w.num_kv_heads
+    keep = keep_b.cpu()
+    for l in range(w.num_layers):
+        ref = inp["caches"][l].clone().view(torch.uint8)
+        dev = caches_b[l].cpu()
+        for b, t in enumerate(w.seq_lens):
+            k = min(w.budget, t)
+            ocp.compact_per_head(ref, inp["tables"][b], w.block_size, keep[b * h:(b + 1) * h, :k].long(), t,
+                                 full_permutation=False)
+            blk, off = ocp.token_slots(inp["tables"][b], w.block_size, torch.arange(k))
+            assert torch.equal(dev[:, blk, off], ref[:, blk, off]), (l, b)
+
+
 def test_invalid_arguments_raise():
     w = small()
     inp = build_inputs(w)

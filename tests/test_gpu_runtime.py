@@ -302,6 +302,31 @@ def test_batch_hook_on_the_resident_kernel(tmp_path, monkeypatch):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+def test_runner_hook_on_an_fp8_cache_kept_in_uint8_tensors(tmp_path):
+    """vLLM keeps an fp8 KV cache as uint8 tensors with one scale per tensor: the hook scores
+    the codes as they are and moves rows only.  Same result dictionary and the same bytes as
+    the same cache handed over as float8_e4m3fn tensors."""
+    from helpers import build_inputs
+    from triattention_amd import synth
+    w = synth.Workload(name="t", num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128, seq_lens=(300,),
+                       budget=96, block_size=16, window_size=12, rope_theta=1e6, index=33, kv_dtype="fp8")
+    inp = build_inputs(w)
+    results, after = [], []
+    for as_uint8 in (True, False):
+        runner, reqs, caches, sched, signals = _fake_runner(w, inp, tmp_path)
+        if as_uint8:
+            runner.kv_caches = caches = [c.view(torch.uint8) for c in caches]
+        res = RunnerHookCompressionExecutor(runner).execute("r0", signals["r0"], sched)
+        torch.cuda.synchronize()
+        assert res.applied and res.cache_len_after == 96
+        results.append(res)
+        after.append([c.cpu().view(torch.uint8) for c in caches])
+    assert results[0] == results[1]
+    for a, b in zip(*after):
+        assert torch.equal(a, b)
+    assert not torch.equal(after[0][0], inp["caches"][0].view(torch.uint8))      # something moved
+
+
 def test_dense_scoring_api_against_reference_scores():
     gold = load_golden("scoring_pytorch.pt")
     for name, style in (("d128_half", "half"), ("d64_inter", "interleaved")):

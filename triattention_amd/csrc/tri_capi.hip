@@ -50,8 +50,8 @@ int check_layout(const tri_kv_layout* kv, bool need_v) {
   if (need_v && !kv->v_layers) return fail(TRI_ERR_INVALID_ARGUMENT, "v_layers is NULL");
   if (kv->kv_dtype == TRI_KV_FP8_E4M3 && !kv->k_scale_layers)
     return fail(TRI_ERR_INVALID_ARGUMENT, "fp8 cache without k_scale_layers");
-  if (kv->kv_dtype == TRI_KV_FP8_E4M3 && need_v && !kv->v_scale_layers)
-    return fail(TRI_ERR_INVALID_ARGUMENT, "fp8 cache without v_scale_layers");
+  // v_scale_layers may be NULL: the rows then carry no scales of their own (a cache with one
+  // scale per tensor) and compaction moves rows only.
   return TRI_OK;
 }
 
@@ -270,7 +270,7 @@ int fill_compact(const tri_kv_layout* kv, const tri_batch* batch, const int32_t*
   a.B = batch->num_seqs; a.L = kv->num_layers; a.Hkv = kv->num_kv_heads; a.D = kv->head_dim;
   a.block_size = kv->block_size; a.elem_bytes = eb; a.max_budget = batch->max_budget;
   a.keep_per_layer = keep_per_layer ? 1 : 0; a.shared = shared ? 1 : 0;
-  a.has_scales = kv->kv_dtype == TRI_KV_FP8_E4M3;
+  a.has_scales = kv->kv_dtype == TRI_KV_FP8_E4M3 && kv->v_scale_layers != nullptr;
   a.stride_block = kv->stride_block; a.stride_token = kv->stride_token; a.stride_head = kv->stride_head;
   a.k_layers = kv->k_layers; a.v_layers = kv->v_layers;
   a.k_scale_layers = kv->k_scale_layers; a.v_scale_layers = kv->v_scale_layers;

@@ -15,8 +15,23 @@ from ._lib import (KV_BF16, KV_FP16, KV_FP8_E4M3, REDUCE_MAX, REDUCE_MEAN, REDUC
                    ROPE_INTERLEAVED, Batch, KvLayout, ScoreParams, SelectParams)
 
 _DTYPES = {torch.bfloat16: KV_BF16, torch.float16: KV_FP16}
+_UNIT_SCALES: dict = {}
+
+
+def _unit_scales(device, count: int) -> torch.Tensor:
+    """An array of ones standing in for the per-(token, head) scales of an fp8 cache that has none."""
+    key = (str(device), int(count))
+    hit = _UNIT_SCALES.get(key)
+    if hit is None:
+        if len(_UNIT_SCALES) >= 4:
+            _UNIT_SCALES.pop(next(iter(_UNIT_SCALES)))
+        hit = _UNIT_SCALES[key] = torch.ones(count, dtype=torch.float32, device=device)
+    return hit
+
+
 if hasattr(torch, "float8_e4m3fn"):
     _DTYPES[torch.float8_e4m3fn] = KV_FP8_E4M3
+    _DTYPES[torch.uint8] = KV_FP8_E4M3      # vLLM keeps the codes of an fp8 cache in uint8 tensors
 
 
 def _stream() -> int:
@@ -91,9 +106,16 @@ class PagedKV:
         self.v_ptrs = (torch.tensor([t.data_ptr() for t in v_views], dtype=torch.int64, device=self.device)
                        if v_views is not None else None)
         self.ks_ptrs = self.vs_ptrs = None
-        if self.dtype == getattr(torch, "float8_e4m3fn", None):
+        if _DTYPES[self.dtype] == KV_FP8_E4M3:
             if k_scales is None:
-                raise ValueError("fp8 cache needs per-(token, head) scales")
+                # A cache with one scale per tensor (vLLM's fp8 KV cache): the codes are scored as
+                # they are (a factor common to a layer cancels in the normalised scores; callers
+                # that do not normalise fold it into freq_scale_sq), and rows move without scales.
+                if v_scales is not None:
+                    raise ValueError("v_scales without k_scales")
+                unit = _unit_scales(self.device, self.num_blocks * self.block_size * self.num_kv_heads)
+                k_scales = [unit] * self.num_layers
+                self._unit = unit           # ours, so kept alive here whatever becomes of _keep
             self.ks_ptrs = torch.tensor([t.data_ptr() for t in k_scales], dtype=torch.int64, device=self.device)
             if v_scales is not None:
                 self.vs_ptrs = torch.tensor([t.data_ptr() for t in v_scales], dtype=torch.int64, device=self.device)
