@@ -428,6 +428,93 @@ def test_hook_skip_reasons_and_executor(monkeypatch):
         {"applied": False, "reason": "plan_only", "cache_len_after": 8}
 
 
+def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
+    """Host logic of ``triattention_apply_compression_batch`` with a stand-in for the kernels:
+    requests with something to drop go to one batched call per KV-cache group, the others get
+    the one-by-one hook's answers; block lists are truncated per request; a failed resident launch
+    sends every request of the batch through the one-by-one path."""
+    calls = {"batch": [], "single": []}
+
+    def select_group(*, layer_kv_iter=None, total_tokens, budget_total, **kw):
+        calls["single"].append(total_tokens)
+        k = min(total_tokens, budget_total)
+        return {"mode": "per_head", "indices": torch.arange(k).repeat(2, 1), "semantic": "hf_aligned_global_per_head"}
+
+    def compress_batch(*, layer_kv, block_size, requests):
+        calls["batch"].append([dict(r) for r in requests])
+        if fail["now"]:
+            raise hook_mod.ResidentLaunchFailed("forced")
+        return [{"mode": "per_head", "indices": torch.arange(r["budget_total"]).repeat(2, 1),
+                 "semantic": "hf_aligned_global_per_head"} for r in requests]
+
+    fail = {"now": False}
+    select_group._supports_paged_group = True
+    select_group._compress_batch = compress_batch
+    select_layer = lambda **kw: None
+    select_layer._supports_paged = True
+    monkeypatch.setattr(hook_mod, "_build_triattention_selector", lambda config, base_runner=None: (select_layer, select_group, "enabled"))
+    moved = []
+    monkeypatch.setattr(hook_mod, "compact_request_kv_in_place_per_head",
+                        lambda **kw: moved.append(kw["total_tokens"]) or int(kw["keep_token_indices_per_head"].shape[1]))
+    cfg = TriAttentionRuntimeConfig(kv_budget=8, divide_length=2, window_size=2,
+                                    sparse_stats_path=GOLDEN / "qwen3_8b_stats_slice.pt")
+
+    def runner_with(lengths):
+        reqs = {f"r{i}": types.SimpleNamespace(num_computed_tokens=t, block_ids=(list(range(100 * i, 100 * i + 10)),))
+                for i, t in enumerate(lengths)}
+        r = _Runner(requests=reqs, kv_caches=[torch.zeros(2, 400, 4, 2, 64)],
+                    cache_config=types.SimpleNamespace(block_size=4))
+        install_runner_compression_hook(r, cfg)
+        sig = {rid: _signal(req_id=rid, estimated_cache_len=q.num_computed_tokens + 1, prefill_len=3)
+               for rid, q in reqs.items()}
+        sched = types.SimpleNamespace(num_scheduled_tokens={rid: 1 for rid in reqs})
+        return r, reqs, sig, sched
+
+    runner, reqs, sig, sched = runner_with([40, 6, 30, 17])
+    sig["r2"] = _signal(req_id="r2", estimated_cache_len=31, prefill_len=5, protect_prefill=True)
+    sig["idle"] = _signal(req_id="idle", should_compress=False)
+    out = RunnerHookCompressionExecutor(runner).execute_batch(sig, sched)
+    assert list(out) == ["r0", "r1", "r2", "r3"]
+    assert out["r1"].reason == "under_budget" and not out["r1"].applied
+    assert len(calls["batch"]) == 1 and not calls["single"]
+    sent = calls["batch"][0]
+    assert [r["total_tokens"] for r in sent] == [40, 30, 17] and [r["budget_total"] for r in sent] == [8, 8, 8]
+    assert [r["round_start"] for r in sent] == [40, 30, 17]
+    assert [(r["protect_prefill"], r["prefill_len"]) for r in sent] == [(False, 3), (True, 5), (False, 3)]
+    assert sent[0]["block_ids"] == list(range(0, 10))
+    for rid in ("r0", "r2", "r3"):
+        assert out[rid].applied and out[rid].cache_len_after == 8
+        assert out[rid].reason == "kv_compacted:per_head:hf_aligned_global_per_head"
+        first = reqs[rid].block_ids[0][0]
+        assert reqs[rid].block_ids == ([first, first + 1],)
+        assert out[rid].details["reclaimed_block_count"] == 8
+    # the same requests one by one give the same dictionaries
+    runner1, reqs1, sig1, sched1 = runner_with([40, 6, 30, 17])
+    sig1["r2"] = sig["r2"]
+    one = {rid: RunnerHookCompressionExecutor(runner1).execute(rid, s_, sched1) for rid, s_ in sig1.items()}
+    assert one == out and calls["single"] == [40, 30, 17] and moved == [40, 30, 17]
+    # a single candidate does not need the batched call
+    calls["batch"].clear(); calls["single"].clear(); moved.clear()
+    runner2, reqs2, sig2, sched2 = runner_with([40, 5])
+    out2 = RunnerHookCompressionExecutor(runner2).execute_batch(sig2, sched2)
+    assert out2["r0"].applied and not calls["batch"] and calls["single"] == [40]
+    # failed resident launch: everything is repeated one by one, with the resident kernel switched off meanwhile
+    calls["batch"].clear(); calls["single"].clear(); moved.clear()
+    fail["now"] = True
+    seen_env = []
+    monkeypatch.setattr(hook_mod, "compact_request_kv_in_place_per_head",
+                        lambda **kw: seen_env.append(__import__("os").environ.get("TRIATTN_RESIDENT_KERNEL")) or 8)
+    runner3, reqs3, sig3, sched3 = runner_with([40, 30])
+    out3 = RunnerHookCompressionExecutor(runner3).execute_batch(sig3, sched3)
+    assert len(calls["batch"]) == 1 and calls["single"] == [40, 30] and seen_env == ["off", "off"]
+    assert all(r.applied and r.cache_len_after == 8 for r in out3.values())
+    assert "TRIATTN_RESIDENT_KERNEL" not in __import__("os").environ
+    # a runner without the batch hook: execute_batch loops over execute
+    bare = _Runner(triattention_apply_compression=lambda **kw: {"applied": True, "reason": "x", "cache_len_after": 1})
+    res = RunnerHookCompressionExecutor(bare).execute_batch({"a": _signal(req_id="a"), "b": _signal(req_id="b")}, sched)
+    assert set(res) == {"a", "b"} and all(r.applied for r in res.values())
+
+
 def test_runtime_context_lengths_defer_and_regression_guard():
     cfg = TriAttentionRuntimeConfig(kv_budget=8, divide_length=2)
     runner, req = _fake_runner(num_computed=40)
