@@ -164,6 +164,31 @@ def test_compaction_api_matches_reference_and_raises_like_it(axis):
     assert compact_request_kv_in_place(amb, [0, 1], 4, [1, 2], 8) == 2
 
 
+@pytest.mark.parametrize("preserve", [True, False])
+def test_compaction_self_check_switch(preserve, monkeypatch):
+    """TRIATTN_DEBUG_VALIDATE_COMPACTION_CONTENT=1 (the reference's switch): the rows are
+    gathered before the move and the compacted prefix is compared with them afterwards; a
+    correct move passes, and the check itself notices a prefix that does not hold them."""
+    from triattention_amd.runtime import kv_compaction as kvc
+    g = load_golden("compaction.pt")["axis0"]
+    bs, t = int(g["block_size"]), int(g["total_tokens"])
+    pad = torch.zeros(*g["kv_before"].shape[:-1], 64, dtype=torch.bfloat16)
+    pad[..., :16] = g["kv_before"]
+    monkeypatch.setenv("TRIATTN_DEBUG_VALIDATE_COMPACTION_CONTENT", "1")
+    a = pad.to(DEV)
+    assert compact_request_kv_in_place_per_head(a, g["block_ids"], bs, g["keep_per_head"].to(DEV), t,
+                                                preserve_dropped_tokens=preserve) == g["keep_per_head"].shape[1]
+    b = pad.to(DEV)
+    assert compact_request_kv_in_place(b, g["block_ids"], bs, g["keep_shared"].to(DEV), t,
+                                       preserve_dropped_tokens=preserve) == g["keep_shared"].numel()
+    # the checker against rows that are not there
+    c = pad.to(DEV)
+    keep = g["keep_shared"].to(DEV).long().unsqueeze(0)
+    expected = [kvc._rows_of(c, g["block_ids"], bs, keep, True)]
+    with pytest.raises(RuntimeError, match="TRIATTN_DEBUG_COMPACTION_KEY_MISMATCH:shared_prefix_content_mismatch"):
+        kvc._validate_prefix([c], g["block_ids"], bs, int(keep.shape[1]), expected, True)      # nothing was moved
+
+
 def _signal(**kw):
     base = dict(req_id="r", should_compress=True, reason="length_threshold", estimated_cache_len=301, step=1,
                 kv_usage=None, protect_prefill=False, prefill_len=20, scheduled_tokens=1)

@@ -515,6 +515,18 @@ def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
     assert set(res) == {"a", "b"} and all(r.applied for r in res.values())
 
 
+def test_verify_rope_alignment():
+    a = rope.default_inv_freq(128, 1e6)
+    rope.verify_rope_alignment(a, types.SimpleNamespace(inv_freq=a.clone()))
+    with pytest.raises(ValueError, match="mismatch"):
+        rope.verify_rope_alignment(a, rope.default_inv_freq(128, 1e4))
+    with pytest.raises(ValueError, match="shape"):
+        rope.verify_rope_alignment(a, rope.default_inv_freq(64, 1e6))
+    with pytest.raises(ValueError, match="inv_freq attribute"):
+        rope.verify_rope_alignment(types.SimpleNamespace(), a)
+    rope.verify_rope_alignment(rope.llama3_inv_freq(128), rope.llama3_inv_freq(128) + 5e-6)
+
+
 def test_runtime_context_lengths_defer_and_regression_guard():
     cfg = TriAttentionRuntimeConfig(kv_budget=8, divide_length=2)
     runner, req = _fake_runner(num_computed=40)

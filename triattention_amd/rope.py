@@ -56,3 +56,21 @@ def inv_freq_from_rope_config(head_dim: int, rope_theta: float | None,
         return llama3_inv_freq(head_dim, theta, float(rs["factor"]), float(rs["low_freq_factor"]),
                                float(rs["high_freq_factor"]), int(rs["original_max_position_embeddings"]))
     raise ValueError(f"unsupported rope_type {kind!r}: put inv_freq into the stats file's metadata")
+
+
+def verify_rope_alignment(pruner_rotary: Any, model_rotary: Any, tolerance: float = 1e-5) -> None:
+    """Raise ``ValueError`` unless both objects carry the same ``inv_freq`` (shape, and values
+    within ``tolerance``): statistics scored with other frequencies than the model's rotate to
+    meaningless scores without any error (core/utils.py:364-405).  Tensors are taken as they are."""
+    def freqs(obj, name):
+        f = obj if isinstance(obj, torch.Tensor) else getattr(obj, "inv_freq", None)
+        if f is None:
+            raise ValueError(f"{name} does not have inv_freq attribute")
+        return f
+    a, b = freqs(pruner_rotary, "pruner_rotary"), freqs(model_rotary, "model_rotary")
+    if a.shape != b.shape:
+        raise ValueError(f"RoPE inv_freq shape mismatch: pruner={tuple(a.shape)}, model={tuple(b.shape)}")
+    worst = float((a.detach().double().cpu() - b.detach().double().cpu()).abs().max())
+    if worst > tolerance:
+        raise ValueError(f"RoPE inv_freq mismatch (max diff={worst:.2e} > tolerance={tolerance:.2e}): the "
+                         "statistics and the model disagree on the rotary frequencies (rope_theta or scaling)")

@@ -14,6 +14,7 @@ Differences, all on purpose:
 """
 from __future__ import annotations
 
+import os
 import weakref
 from typing import Iterable
 
@@ -147,8 +148,47 @@ def _check_rows(keep: torch.Tensor, total_tokens: int, what: str) -> None:
             raise ValueError(f"{what} must be ascending for in-place compaction")
 
 
+def _debug_validate_compaction_content() -> bool:
+    """The reference's self-check switch (kv_compaction.py:24-25)."""
+    return os.environ.get("TRIATTN_DEBUG_VALIDATE_COMPACTION_CONTENT", "0") == "1"
+
+
+def _rows_of(cache, block_ids, block_size: int, keep_rows: torch.Tensor, shared: bool):
+    """K and V rows ``[k, H, D]`` (as bytes) that the slots 0..k-1 must hold after compaction."""
+    out = []
+    for side in _split_kv_axes(cache):
+        if shared:
+            blk, off = _token_slots(block_ids, block_size, keep_rows[0], side.device)
+            rows = side[blk, off]
+        else:
+            per_head = []
+            for h in range(int(side.shape[2])):
+                blk, off = _token_slots(block_ids, block_size, keep_rows[h], side.device)
+                per_head.append(side[blk, off, h])
+            rows = torch.stack(per_head, dim=1)
+        out.append(rows.contiguous().view(torch.uint8).clone())
+    return out
+
+
+def _validate_prefix(kv_caches, block_ids, block_size: int, k: int, expected: list, shared: bool) -> None:
+    """Re-read the compacted prefix and compare it bit for bit with the rows gathered before
+    the move (kv_compaction.py:441-456,548-563; same exception texts)."""
+    label = "shared" if shared else "per_head"
+    for cache, (want_k, want_v) in zip(kv_caches, expected):
+        key_cache, value_cache = _split_kv_axes(cache)
+        tok = torch.arange(k, device=key_cache.device, dtype=torch.long)
+        blk, off = _token_slots(block_ids, block_size, tok, key_cache.device)
+        if not torch.equal(key_cache[blk, off].contiguous().view(torch.uint8), want_k):
+            raise RuntimeError(f"TRIATTN_DEBUG_COMPACTION_KEY_MISMATCH:{label}_prefix_content_mismatch")
+        if not torch.equal(value_cache[blk, off].contiguous().view(torch.uint8), want_v):
+            raise RuntimeError(f"TRIATTN_DEBUG_COMPACTION_VALUE_MISMATCH:{label}_prefix_content_mismatch")
+
+
 def _run_compaction(kv_caches, block_ids, block_size: int, keep_rows: torch.Tensor, total_tokens: int,
                     shared: bool, full_permutation: bool) -> None:
+    expected = None
+    if _debug_validate_compaction_content():
+        expected = [_rows_of(c, block_ids, block_size, keep_rows, shared) for c in kv_caches]
     hints = {kv_axis_hint(c) for c in kv_caches}
     if len(hints) != 1:
         raise ValueError("layers of one group disagree on the K/V axis hint")
@@ -159,6 +199,8 @@ def _run_compaction(kv_caches, block_ids, block_size: int, keep_rows: torch.Tens
     batch = ops.StepBatch(kv.device, [total_tokens], budgets=[k], block_tables=[_block_ids_list(block_ids)])
     ops.compact(kv, batch, keep_rows.to(device=kv.device, dtype=torch.int32).contiguous(),
                 shared=shared, full_permutation=full_permutation)
+    if expected is not None:
+        _validate_prefix(kv_caches, block_ids, block_size, k, expected, shared)
 
 
 def compact_request_kv_in_place(kv_cache, block_ids, block_size: int, keep_token_indices,
