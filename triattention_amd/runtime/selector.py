@@ -287,7 +287,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         if resident and ws.status() != 0:
             raise ResidentLaunchFailed("a wait inside the resident kernel expired; the caches were left untouched")
         h = kv.num_kv_heads
-        return [{"mode": "per_head", "indices": keep[b * h:(b + 1) * h, :k].to(torch.long),
+        keep = keep.to(torch.long)           # one conversion; the per-request results are views
+        return [{"mode": "per_head", "indices": keep[b * h:(b + 1) * h, :k],
                  "semantic": "hf_aligned_global_per_head", "group_agg_mode": agg,
                  "debug_group_layer_indices": list(layer_ids), "debug_recent_count": _recent_count(t)}
                 for b, (k, t) in enumerate(zip(ks, totals))]
