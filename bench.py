@@ -47,6 +47,8 @@ def parse_args():
     ap.add_argument("--seq-len", type=int, default=0,
                     help="override every sequence's cached length (e.g. budget + 128 for the steady-state step)")
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
+    ap.add_argument("--kv-dtype", choices=["bf16", "fp16"], default="",
+                    help="key/value dtype of the synthetic cache (default: the workload's own)")
     ap.add_argument("--two-pass", action="store_true",
                     help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
     ap.add_argument("--hook-latency", action="store_true",
@@ -218,6 +220,10 @@ def main() -> int:
     if args.seq_len > 0:
         nseq = args.sequences if args.sequences > 0 else w.num_seqs
         w = w.scaled(name=f"{w.name}_b{nseq}_len{args.seq_len}", seq_lens=(args.seq_len,) * nseq)
+    if args.kv_dtype and args.kv_dtype != w.kv_dtype:
+        if "fp8" in (args.kv_dtype, w.kv_dtype):
+            raise SystemExit("--kv-dtype switches between bf16 and fp16; the fp8 workload is --config 4")
+        w = w.scaled(name=f"{w.name}_{args.kv_dtype}", kv_dtype=args.kv_dtype)
     t_setup = time.perf_counter()
     tables = synth.make_block_tables(w)
     pool = synth.make_kv_pool(w, tables, dev)

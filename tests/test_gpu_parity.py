@@ -44,6 +44,9 @@ SCORE_CASES = {
     "d256": dict(w=small(head_dim=256, seq_lens=(140,))),
     "interleaved": dict(w=small(rope_style="interleaved")),
     "fp16": dict(w=small(kv_dtype="fp16")),
+    "fp16_interleaved_ragged": dict(w=small(kv_dtype="fp16", rope_style="interleaved", seq_lens=(300, 17, 1000, 513),
+                                            num_layers=3)),
+    "fp16_g8": dict(w=small(kv_dtype="fp16", num_q_heads=16, num_kv_heads=2, seq_lens=(700, 90))),
     "block32": dict(w=small(block_size=32, seq_lens=(500, 31))),
     "block_not_pow2": dict(w=small(block_size=24, seq_lens=(301,))),
     "kv_axis1": dict(w=small(seq_lens=(290, 64)), kv_axis=1),
@@ -450,6 +453,10 @@ RESIDENT_CASES = {
     "g8_fp8_long": dict(w=small(kv_dtype="fp8", num_q_heads=16, num_kv_heads=2, seq_lens=(9000, 2500), budget=512)),
     "interleaved": dict(w=small(rope_style="interleaved")),
     "fp16": dict(w=small(kv_dtype="fp16")),
+    "fp16_interleaved_ragged": dict(w=small(kv_dtype="fp16", rope_style="interleaved", seq_lens=(300, 17, 1000, 513),
+                                            num_layers=3)),
+    "fp16_g8": dict(w=small(kv_dtype="fp16", num_q_heads=16, num_kv_heads=2, seq_lens=(700, 90))),
+    "fp16_tile192": dict(w=small(kv_dtype="fp16", seq_lens=(3072,) * 16, budget=256, num_layers=2)),
     "fp8": dict(w=small(kv_dtype="fp8", seq_lens=(300, 45))),
     "fp8_interleaved_hkv8": dict(w=small(kv_dtype="fp8", rope_style="interleaved", num_q_heads=32, num_kv_heads=8,
                                          seq_lens=(530, 64))),
@@ -479,8 +486,6 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     rounding by mean^2/var), same kept sets away from ties."""
     case = dict(RESIDENT_CASES[name])
     w = case["w"]
-    if kernel == "mfma" and w.kv_dtype == "fp16":
-        pytest.skip("the matrix-core kernel takes bf16 and fp8 keys; fp16 runs the vector-unit kernel")
     if kernel == "mfma" and w.block_size < 16:
         pytest.skip("the matrix-core kernel needs blocks of at least 16 tokens (a step lies inside one block)")
     if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
@@ -665,6 +670,26 @@ def test_expired_wait_raises_the_status_word_and_the_step_leaves_the_cache_alone
     assert torch.equal(keep, keep2)
     for c, c2 in zip(caches, caches2):
         assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
+
+
+def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
+    """The matrix-core kernel for fp16 keys holds its coefficients as fp16 pieces; statistics
+    so large that a coefficient exceeds 65504 cannot be held, and the launch says so through
+    the status word instead of returning scores made of infinities."""
+    w = small(kv_dtype="fp16", seq_lens=(300, 200))
+    inp = build_inputs(w)
+    inp["qc"] = inp["qc"] * 1e6
+    inp["qa"] = inp["qa"] * 1e6
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    print("fp16 coefficient overflow", flush=True)
+    _, _, ws = ops.select_paged(kv, batch, sc, sel)
+    assert ws.status() != 0
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+    _, _, ws = ops.select_paged(kv, batch, sc, sel)
+    assert ws.status() == 0
 
 
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):

@@ -94,7 +94,8 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   const bool f_mfma = force && strcmp(force, "mfma") == 0;
   const bool f_off = force && strcmp(force, "off") == 0;
   // The matrix-core kernel addresses the 16 rows of a step with 32-bit offsets from a scalar base.
-  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP8_E4M3) && !f_valu &&
+  const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP16 || kv->kv_dtype == TRI_KV_FP8_E4M3) &&
+                         !f_valu &&
                          kv->stride_token > 0 && kv->stride_token < (1 << 25);
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;

@@ -29,6 +29,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
@@ -64,27 +66,73 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w 
 // product's write and another vector instruction's read of that register (three
 // instructions) and after a transcendental's write (one) is provided here: four dot
 // products, then the four square roots in the same order, then one idle cycle.
+template <int DT>
 __device__ __forceinline__ void magnitudes4(const uint32_t (&x)[4], float* m) {
-  asm("v_dot2_f32_bf16 %0, %4, %4, 0\n\t"
-      "v_dot2_f32_bf16 %1, %5, %5, 0\n\t"
-      "v_dot2_f32_bf16 %2, %6, %6, 0\n\t"
-      "v_dot2_f32_bf16 %3, %7, %7, 0\n\t"
-      "v_sqrt_f32 %0, %0\n\t"
-      "v_sqrt_f32 %1, %1\n\t"
-      "v_sqrt_f32 %2, %2\n\t"
-      "v_sqrt_f32 %3, %3\n\t"
-      "s_nop 0"
-      : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(m[3])
-      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+  if constexpr (DT == TRI_KV_FP16) {
+    asm("v_dot2_f32_f16 %0, %4, %4, 0\n\t"
+        "v_dot2_f32_f16 %1, %5, %5, 0\n\t"
+        "v_dot2_f32_f16 %2, %6, %6, 0\n\t"
+        "v_dot2_f32_f16 %3, %7, %7, 0\n\t"
+        "v_sqrt_f32 %0, %0\n\t"
+        "v_sqrt_f32 %1, %1\n\t"
+        "v_sqrt_f32 %2, %2\n\t"
+        "v_sqrt_f32 %3, %3\n\t"
+        "s_nop 0"
+        : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(m[3])
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+  } else {
+    asm("v_dot2_f32_bf16 %0, %4, %4, 0\n\t"
+        "v_dot2_f32_bf16 %1, %5, %5, 0\n\t"
+        "v_dot2_f32_bf16 %2, %6, %6, 0\n\t"
+        "v_dot2_f32_bf16 %3, %7, %7, 0\n\t"
+        "v_sqrt_f32 %0, %0\n\t"
+        "v_sqrt_f32 %1, %1\n\t"
+        "v_sqrt_f32 %2, %2\n\t"
+        "v_sqrt_f32 %3, %3\n\t"
+        "s_nop 0"
+        : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(m[3])
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+  }
 }
 
-// Two fp32 values -> packed bf16 (round to nearest even) and the fp32 remainders.
+// Two fp32 values -> packed bf16 (fp16 for fp16 keys; round to nearest even) and the fp32
+// remainders.  The packed halves are turned back into fp32 through their bit patterns, so the
+// subtraction sees exactly what was stored.
+template <int DT>
 __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, float& r1) {
   const f32x2 x = {x0, x1};
-  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
-  r0 = x0 - bf16_lo(packed);
-  r1 = x1 - bf16_hi(packed);
-  return packed;
+  if constexpr (DT == TRI_KV_FP16) {
+    const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+    r0 = x0 - (float)__builtin_bit_cast(_Float16, (unsigned short)(packed & 0xffffu));
+    r1 = x1 - (float)__builtin_bit_cast(_Float16, (unsigned short)(packed >> 16));
+    return packed;
+  } else {
+    const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    r0 = x0 - bf16_lo(packed);
+    r1 = x1 - bf16_hi(packed);
+    return packed;
+  }
+}
+
+// One 16x16x32 matrix-core step in the operand type of the keys (fp8 keys are converted to bf16).
+template <int DT>
+__device__ __forceinline__ f32x4 mfma_step(const uint4& a, const uint4& b, f32x4 c) {
+  if constexpr (DT == TRI_KV_FP16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
+}
+
+// Piece `pieces` of x in the operand type: what is left of x after `pieces` roundings.
+template <int DT>
+__device__ __forceinline__ float coefficient_piece(float x, int pieces) {
+  for (int s = 0; s < pieces; ++s) {
+    if constexpr (DT == TRI_KV_FP16)
+      x = x - (float)(_Float16)x;
+    else
+      x = x - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x) << 16);
+  }
+  return x;
 }
 
 // Everything the resident kernel needs before it starts, in one launch: workgroup (l, b)
@@ -177,14 +225,15 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
             if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
             else pair = slab_elem<DT>(set, kb, e) & 63;
           }
-          float x = c[which * 64 + pair];
-          for (int s = 0; s < sp; ++s) x = x - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x) << 16);
-          v[e] = x;
+          v[e] = coefficient_piece<DT>(c[which * 64 + pair], sp);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const f32x2 x = {v[2 * e], v[2 * e + 1]};
-          out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+          if constexpr (DT == TRI_KV_FP16)
+            out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+          else
+            out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
         }
       }
       out_base[idx] = uint4{out[0], out[1], out[2], out[3]};
@@ -237,6 +286,22 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     for (int g = 0; g < QG; ++g)
 #pragma unroll
       for (int o = 0; o < 6; ++o) B[g][o] = p[(g * 6 + o) * 64];
+    if constexpr (DT == TRI_KV_FP16) {
+      // A coefficient beyond fp16's range (65504) arrives as an infinity: the scores of this
+      // launch would be meaningless, so the status word is raised (the caller repeats the
+      // step on the vector-unit kernels) and every wait of the launch gives up.
+      uint32_t bad = 0;
+#pragma unroll
+      for (int g = 0; g < QG; ++g)
+#pragma unroll
+        for (int o = 0; o < 6; ++o) {
+          const uint32_t w4[4] = {B[g][o].x, B[g][o].y, B[g][o].z, B[g][o].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            bad |= (uint32_t)((w4[i] & 0x7c00u) == 0x7c00u) | (uint32_t)((w4[i] & 0x7c000000u) == 0x7c000000u);
+        }
+      if (__any(bad != 0) && lane == 0) atomicExch(a.status, 2u);
+    }
   };
 
   // A step is 16 consecutive tokens starting at a multiple of 16, so with blocks of at
@@ -329,7 +394,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s)
-        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(d.c[s]), as_bf16x8(B[g][s]), acc[g], 0, 0, 0);
+        acc[g] = mfma_step<DT>(d.c[s], B[g][s], acc[g]);
       acc_e[g] = acc[g];   // the magnitude MFMAs continue the sum (the key MFMAs are long done by then)
     }
 #pragma unroll
@@ -353,23 +418,23 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
             x[2 * i + 1] = __builtin_amdgcn_perm(im, re, 0x07060302u);
           }
         }
-        magnitudes4(x, &mag[4 * h]);
+        magnitudes4<DT>(x, &mag[4 * h]);
       }
       uint4 hi, lo;
       float r[8];
-      hi.x = split_pair(mag[0], mag[1], r[0], r[1]);
-      hi.y = split_pair(mag[2], mag[3], r[2], r[3]);
-      hi.z = split_pair(mag[4], mag[5], r[4], r[5]);
-      hi.w = split_pair(mag[6], mag[7], r[6], r[7]);
+      hi.x = split_pair<DT>(mag[0], mag[1], r[0], r[1]);
+      hi.y = split_pair<DT>(mag[2], mag[3], r[2], r[3]);
+      hi.z = split_pair<DT>(mag[4], mag[5], r[4], r[5]);
+      hi.w = split_pair<DT>(mag[6], mag[7], r[6], r[7]);
       float unused0, unused1;
-      lo.x = split_pair(r[0], r[1], unused0, unused1);
-      lo.y = split_pair(r[2], r[3], unused0, unused1);
-      lo.z = split_pair(r[4], r[5], unused0, unused1);
-      lo.w = split_pair(r[6], r[7], unused0, unused1);
+      lo.x = split_pair<DT>(r[0], r[1], unused0, unused1);
+      lo.y = split_pair<DT>(r[2], r[3], unused0, unused1);
+      lo.z = split_pair<DT>(r[4], r[5], unused0, unused1);
+      lo.w = split_pair<DT>(r[6], r[7], unused0, unused1);
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
-        acc_e[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(hi), as_bf16x8(B[g][4 + set]), acc_e[g], 0, 0, 0);
-        acc_e[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(lo), as_bf16x8(B[g][4 + set]), acc_e[g], 0, 0, 0);
+        acc_e[g] = mfma_step<DT>(hi, B[g][4 + set], acc_e[g]);
+        acc_e[g] = mfma_step<DT>(lo, B[g][4 + set], acc_e[g]);
       }
     }
     const int tl = t + 4 * kb + rsel;
@@ -684,7 +749,8 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
   const int QG = a.G > 4 ? 2 : 1;
   const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
-  if (a.kv_dtype != TRI_KV_BF16 && !fp8) return hipErrorInvalidValue;
+  const bool fp16 = a.kv_dtype == TRI_KV_FP16;
+  if (a.kv_dtype != TRI_KV_BF16 && !fp8 && !fp16) return hipErrorInvalidValue;
   if (a.NO <= 0 || a.NO > kMaxOffsets || a.D != 128) return hipErrorInvalidValue;
   auto prep_launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)a.L, (unsigned)a.B), dim3(kPrepThreads), 0, s, a.folded, a.omega,
@@ -693,6 +759,9 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   if (fp8) {
     if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, true>);
     else prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, false>);
+  } else if (fp16) {
+    if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true>);
+    else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false>);
   } else {
     if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true>);
     else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false>);
@@ -702,6 +771,9 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   if (fp8)
     return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
               : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+  if (fp16)
+    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
   return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
             : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
 }
