@@ -268,7 +268,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
       for (int q = 0; q < 4; ++q)
         if (chead_ok && q < a.G) {
           mean[q] = st[(chead * a.G + q) * 2];
-          sd[q] = st[(chead * a.G + q) * 2 + 1];
+          sd[q] = __fdiv_rn(1.f, st[(chead * a.G + q) * 2 + 1]);   // the tokens multiply by the reciprocal
         }
     }
 #pragma unroll
@@ -282,12 +282,12 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
         v = -INFINITY;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          if (q < a.G) v = fmaxf(v, __fdiv_rn(__fsub_rn(xs[q], mean[q]), sd[q]));
+          if (q < a.G) v = fmaxf(v, __fmul_rn(__fsub_rn(xs[q], mean[q]), sd[q]));
       } else {
         v = 0.f;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          if (q < a.G) v = __fadd_rn(v, __fdiv_rn(__fsub_rn(xs[q], mean[q]), sd[q]));
+          if (q < a.G) v = __fadd_rn(v, __fmul_rn(__fsub_rn(xs[q], mean[q]), sd[q]));
         v = __fdiv_rn(v, (float)a.G);
       }
       const int n = wstart + tl;
