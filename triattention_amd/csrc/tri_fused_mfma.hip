@@ -214,15 +214,18 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           int which, pair;   // which: 0 = P, 1 = R, 2 = E
+          constexpr bool kRegrouped = DT == TRI_KV_FP8_E4M3 && !IL;   // see compute_step
           if (o < 4) {
             const int el = slab_elem<DT>(o, kb, e);
-            if (IL) { which = el & 1; pair = el >> 1; }
+            if (kRegrouped) { which = e & 1; pair = kb * 16 + 4 * o + (e >> 1); }
+            else if (IL) { which = el & 1; pair = el >> 1; }
             else { which = el >= 64 ? 1 : 0; pair = el & 63; }
           } else {
             which = 2;
             const int set = o - 4;
             // interleaved: pairs of MFMAs 2*set and 2*set + 1; half: real parts of MFMA `set`
-            if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
+            if (kRegrouped) pair = kb * 16 + 4 * (2 * set + (e >> 2)) + (e & 3);
+            else if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
             else pair = slab_elem<DT>(set, kb, e) & 63;
           }
           v[e] = coefficient_piece<DT>(c[which * 64 + pair], sp);
@@ -368,7 +371,26 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     // The four bf16 A operands of the step as dwords (two elements each): the loaded
     // registers for bf16 keys, one conversion per dword (exact) for fp8 keys.
     uint32_t w[4][4];
-    if constexpr (FP8) {
+    // One-byte keys in the half-split layout: lane block kb holds the real parts of pairs
+    // 16*kb .. 16*kb + 15 in c[0] and their imaginary parts in c[1].  Two byte permutes per
+    // dword pair put (real, imaginary) next to each other before the conversion, so every
+    // converted dword is a pair: operand s holds pairs 16*kb + 4*s .. + 3, the magnitudes need
+    // no regrouping (8 permutes per step instead of 16 after the conversion), and the
+    // coefficient slabs are laid out to match.
+    constexpr bool kRegrouped = FP8 && !IL;
+    if constexpr (kRegrouped) {
+      const uint32_t re[4] = {raw.c[0].x, raw.c[0].y, raw.c[0].z, raw.c[0].w};
+      const uint32_t im[4] = {raw.c[1].x, raw.c[1].y, raw.c[1].z, raw.c[1].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = __builtin_amdgcn_perm(im[i], re[i], 0x05010400u);   // (re0, im0, re1, im1)
+        const uint32_t hi = __builtin_amdgcn_perm(im[i], re[i], 0x07030602u);   // (re2, im2, re3, im3)
+        w[i][0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false));
+        w[i][1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true));
+        w[i][2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false));
+        w[i][3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true));
+      }
+    } else if constexpr (FP8) {
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const uint32_t r[4] = {raw.c[s].x, raw.c[s].y, raw.c[s].z, raw.c[s].w};
@@ -407,7 +429,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         uint32_t x[4];
-        if constexpr (IL) {
+        if constexpr (IL || kRegrouped) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) x[i] = w[2 * set + h][i];
         } else {
