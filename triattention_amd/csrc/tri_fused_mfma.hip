@@ -245,6 +245,8 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
 }
 
 // QG: groups of four query heads per KV head (1 or 2).
+__device__ __forceinline__ int nsteps_of(int ntok) { return (ntok + 15) >> 4; }
+
 template <int DT, bool IL, int TW, int SL, int QG, int NB>
 __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   static_assert(SL % (16 * NB) == 0, "the slack must hold whole rotations of the step buffers");
@@ -338,7 +340,43 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       lb.scale = table_entry(reinterpret_cast<const void* const*>(a.k_scale_layers), l) + head * 4;
     return lb;
   };
+  // One-byte keys: with eight step buffers and a scale per row the scalar registers do not
+  // hold the strides, masks and sizes of the address arithmetic any more (the compiler kept
+  // them in lanes of a vector register and fetched 16 of them back per step with v_readlane,
+  // a tenth of the step's vector instructions).  For them the arithmetic is done once per
+  // tile instead: lane i keeps the byte offset of step i's first row from the head's base
+  // (the same in every layer) and the index of its first token slot.
+  uint32_t step_off_lo = 0, step_off_hi = 0;
+  int step_slot = 0;
+  if constexpr (FP8) {
+    const int nt = min(n0 + 16 * lane, (nsteps_of(ntok) - 1) * 16 + n0);
+    const int in_blk = nt & bs_mask;
+    const int64_t off = ((int64_t)step_blk * a.stride_block + (int64_t)in_blk * a.stride_token) * ES;
+    step_off_lo = (uint32_t)off;
+    step_off_hi = (uint32_t)((uint64_t)off >> 32);
+    step_slot = step_blk * a.block_size + in_blk;
+  }
   auto load_step = [&](StepData<DT>& d, const LayerBase& lb, int t) __attribute__((always_inline)) {
+    if constexpr (FP8) {
+      const int step = t >> 4;
+      const uint32_t rows_left = (uint32_t)(last_tok - (n0 + t));
+      const uint64_t row_off = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)step_off_hi, step) << 32) |
+                               (uint32_t)__builtin_amdgcn_readlane((int)step_off_lo, step);
+      const char* base = reinterpret_cast<const char*>(uniform_ptr(lb.k + row_off));
+      const uint32_t off = min(lane_row, rows_left * tok_bytes) + lane_col;
+      GlobalBytes p = (GlobalBytes)(uintptr_t)base + off;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const u32x4 v = *(GlobalU4)(p + s * 64);
+        d.c[s] = uint4{v.x, v.y, v.z, v.w};
+      }
+      const uint32_t hkv4 = (uint32_t)a.Hkv * 4u;
+      const uint64_t slot_off = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(step_slot, step) * hkv4;
+      const char* sc = reinterpret_cast<const char*>(uniform_ptr(lb.scale + slot_off));
+      const uint32_t soff = min(lane_scale_row, rows_left * hkv4);
+      d.scale = *(GlobalF32)((GlobalBytes)(uintptr_t)sc + soff);
+      return;
+    }
     const int blk = __builtin_amdgcn_readlane(step_blk, t >> 4);
     const int nt = n0 + t;
     const int in_blk = nt & bs_mask;
