@@ -114,6 +114,17 @@ __device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, fl
   }
 }
 
+// Two fp32 values -> packed fp16 and the fp32 remainders, the remainders by the
+// mixed-precision fused multiply-add, which reads the halves of the packed register as they
+// are (x - half is exact): four instructions per two values where the bf16 route needs six.
+__device__ __forceinline__ uint32_t split_pair_f16(float x0, float x1, float& r0, float& r1) {
+  const f32x2 x = {x0, x1};
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+  asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(packed), "v"(x0));
+  asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(packed), "v"(x1));
+  return packed;
+}
+
 // One 16x16x32 matrix-core step in the operand type of the keys (fp8 keys are converted to bf16).
 template <int DT>
 __device__ __forceinline__ f32x4 mfma_step(const uint4& a, const uint4& b, f32x4 c) {
@@ -228,12 +239,16 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
             else if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
             else pair = slab_elem<DT>(set, kb, e) & 63;
           }
-          v[e] = coefficient_piece<DT>(c[which * 64 + pair], sp);
+          // One-byte keys: their magnitudes go through the fp16 matrix-core instruction (see
+          // compute_step), so the magnitude slabs are fp16 pieces.
+          const bool half_slab = DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= 4);
+          v[e] = half_slab ? coefficient_piece<TRI_KV_FP16>(c[which * 64 + pair], sp)
+                           : coefficient_piece<TRI_KV_BF16>(c[which * 64 + pair], sp);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const f32x2 x = {v[2 * e], v[2 * e + 1]};
-          if constexpr (DT == TRI_KV_FP16)
+          if (DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= 4))
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
           else
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
@@ -291,15 +306,16 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
     for (int g = 0; g < QG; ++g)
 #pragma unroll
       for (int o = 0; o < 6; ++o) B[g][o] = p[(g * 6 + o) * 64];
-    if constexpr (DT == TRI_KV_FP16) {
+    if constexpr (DT == TRI_KV_FP16 || DT == TRI_KV_FP8_E4M3) {
       // A coefficient beyond fp16's range (65504) arrives as an infinity: the scores of this
       // launch would be meaningless, so the status word is raised (the caller repeats the
-      // step on the vector-unit kernels) and every wait of the launch gives up.
+      // step on the vector-unit kernels) and every wait of the launch gives up.  fp16 keys:
+      // all slabs; one-byte keys: the magnitude slabs.
       uint32_t bad = 0;
 #pragma unroll
       for (int g = 0; g < QG; ++g)
 #pragma unroll
-        for (int o = 0; o < 6; ++o) {
+        for (int o = (DT == TRI_KV_FP16 ? 0 : 4); o < 6; ++o) {
           const uint32_t w4[4] = {B[g][o].x, B[g][o].y, B[g][o].z, B[g][o].w};
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -482,19 +498,34 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
       }
       uint4 hi, lo;
       float r[8];
-      hi.x = split_pair<DT>(mag[0], mag[1], r[0], r[1]);
-      hi.y = split_pair<DT>(mag[2], mag[3], r[2], r[3]);
-      hi.z = split_pair<DT>(mag[4], mag[5], r[4], r[5]);
-      hi.w = split_pair<DT>(mag[6], mag[7], r[6], r[7]);
-      float unused0, unused1;
-      lo.x = split_pair<DT>(r[0], r[1], unused0, unused1);
-      lo.y = split_pair<DT>(r[2], r[3], unused0, unused1);
-      lo.z = split_pair<DT>(r[4], r[5], unused0, unused1);
-      lo.w = split_pair<DT>(r[6], r[7], unused0, unused1);
+      if constexpr (FP8) {
+        // The magnitudes of one-byte codes lie in [2^-9, 634]: fp16 holds them, and the fp16
+        // split is two instructions per pair cheaper (this kernel is bound by the vector unit).
+        hi.x = split_pair_f16(mag[0], mag[1], r[0], r[1]);
+        hi.y = split_pair_f16(mag[2], mag[3], r[2], r[3]);
+        hi.z = split_pair_f16(mag[4], mag[5], r[4], r[5]);
+        hi.w = split_pair_f16(mag[6], mag[7], r[6], r[7]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const f32x2 x = {r[2 * i], r[2 * i + 1]};
+          (&lo.x)[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+        }
+      } else {
+        hi.x = split_pair<DT>(mag[0], mag[1], r[0], r[1]);
+        hi.y = split_pair<DT>(mag[2], mag[3], r[2], r[3]);
+        hi.z = split_pair<DT>(mag[4], mag[5], r[4], r[5]);
+        hi.w = split_pair<DT>(mag[6], mag[7], r[6], r[7]);
+        float unused0, unused1;
+        lo.x = split_pair<DT>(r[0], r[1], unused0, unused1);
+        lo.y = split_pair<DT>(r[2], r[3], unused0, unused1);
+        lo.z = split_pair<DT>(r[4], r[5], unused0, unused1);
+        lo.w = split_pair<DT>(r[6], r[7], unused0, unused1);
+      }
+      constexpr int MT = FP8 ? TRI_KV_FP16 : DT;     // operand type of the magnitude MFMAs
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
-        acc_e[g] = mfma_step<DT>(hi, B[g][4 + set], acc_e[g]);
-        acc_e[g] = mfma_step<DT>(lo, B[g][4 + set], acc_e[g]);
+        acc_e[g] = mfma_step<MT>(hi, B[g][4 + set], acc_e[g]);
+        acc_e[g] = mfma_step<MT>(lo, B[g][4 + set], acc_e[g]);
       }
     }
     const int tl = t + 4 * kb + rsel;
