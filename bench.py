@@ -49,6 +49,8 @@ def parse_args():
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
     ap.add_argument("--kv-dtype", choices=["bf16", "fp16"], default="",
                     help="key/value dtype of the synthetic cache (default: the workload's own)")
+    ap.add_argument("--aggregation", choices=["mean", "max"], default="mean",
+                    help="aggregation of the score over the position offsets (the reference's default: mean)")
     ap.add_argument("--two-pass", action="store_true",
                     help="time the score_paged + select pair (raw scores through HBM) instead of select_paged")
     ap.add_argument("--hook-latency", action="store_true",
@@ -235,7 +237,8 @@ def main() -> int:
         kv = ops.PagedKV.from_kv_caches(caches, w.rope_style)
     qc, qa = synth.make_stats(w, dev)
     fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2, device=dev)
-    sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev))
+    sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev),
+                         args.aggregation)
     sel = ops.SelectConfig(window_size=w.window_size)
     batch = ops.StepBatch(dev, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=tables)
     ws = ops.Workspace(kv, batch, sc)
