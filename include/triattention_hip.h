@@ -4,7 +4,10 @@
  *
  * Every entry point is stream ordered: it enqueues kernels on `stream`
  * (a hipStream_t passed as void*, NULL = the null stream), never synchronises the
- * device and never allocates.  All pointers are DEVICE pointers unless a comment
+ * device and never allocates device memory.  (Once per device and process the library
+ * creates an event to chain its resident launches and, for fp8 caches with per-row scales,
+ * a side stream with two events on which the scales move next to the rows; neither is
+ * used while `stream` is under graph capture.)  All pointers are DEVICE pointers unless a comment
  * says "host".  Return value: TRI_OK or a negative tri_status; a message for the
  * last failure on the calling thread is available from tri_last_error().
  * Nothing is thrown and no torch type crosses this boundary.
@@ -124,7 +127,9 @@ uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
 
 /* Byte offset inside the workspace of a 32-bit status word: tri_select_paged and
  * tri_compress_step clear it and the resident kernel sets it to non-zero if one of its
- * bounded waits on another workgroup expired (results are then invalid; the compaction
+ * bounded waits on another workgroup expired (1), or, with fp16 keys or an fp8 cache, if a
+ * coefficient does not fit the fp16 pieces the matrix-core kernel holds it in (2)
+ * (results are then invalid; the compaction
  * inside tri_compress_step sees the word and moves nothing, so the cache is intact and
  * the caller can repeat the step with TRIATTN_RESIDENT_KERNEL=off).  The caller may read
  * it after synchronising the stream.  Host-only; no counterpart in the reference. */
