@@ -49,6 +49,10 @@ def parse_args():
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
     ap.add_argument("--kv-dtype", choices=["bf16", "fp16"], default="",
                     help="key/value dtype of the synthetic cache (default: the workload's own)")
+    ap.add_argument("--layers", type=int, default=0, help="override the number of layers")
+    ap.add_argument("--q-heads", type=int, default=0, help="override the number of query heads")
+    ap.add_argument("--kv-heads", type=int, default=0, help="override the number of KV heads")
+    ap.add_argument("--head-dim", type=int, default=0, help="override the head dimension")
     ap.add_argument("--aggregation", choices=["mean", "max"], default="mean",
                     help="aggregation of the score over the position offsets (the reference's default: mean)")
     ap.add_argument("--two-pass", action="store_true",
@@ -222,6 +226,10 @@ def main() -> int:
     if args.seq_len > 0:
         nseq = args.sequences if args.sequences > 0 else w.num_seqs
         w = w.scaled(name=f"{w.name}_b{nseq}_len{args.seq_len}", seq_lens=(args.seq_len,) * nseq)
+    shape = {k: v for k, v in (("num_layers", args.layers), ("num_q_heads", args.q_heads),
+                               ("num_kv_heads", args.kv_heads), ("head_dim", args.head_dim)) if v > 0}
+    if shape:
+        w = w.scaled(name=w.name + "_" + "_".join(f"{k[4:]}{v}" for k, v in shape.items()), **shape)
     if args.kv_dtype and args.kv_dtype != w.kv_dtype:
         if "fp8" in (args.kv_dtype, w.kv_dtype):
             raise SystemExit("--kv-dtype switches between bf16 and fp16; the fp8 workload is --config 4")

@@ -477,6 +477,22 @@ RESIDENT_CASES = {
 }
 
 
+# The same machinery with eight KV heads (workgroups of eight waves; the cases above mostly have
+# two KV heads, which take workgroups of four waves, two per CU) on a device that pretends to
+# hold 24 workgroups, so that small inputs need several, device-packed launches.
+RESIDENT_CASES.update({
+    "hkv8_ragged_small_chip": dict(w=small(num_q_heads=32, num_kv_heads=8, seq_lens=(3000, 70, 6100, 900, 4500, 1, 3300),
+                                           budget=128, num_layers=2), workgroups=24),
+    "hkv8_g8_small_chip": dict(w=small(num_q_heads=64, num_kv_heads=8, seq_lens=(2500, 300, 4000), budget=128,
+                                       num_layers=2), workgroups=24),
+    "hkv2_ragged_small_chip": dict(w=small(seq_lens=(3000, 70, 6100, 900, 4500, 1, 3300), budget=128, num_layers=2),
+                                   workgroups=12),
+    "hkv4_g7": dict(w=small(num_q_heads=28, num_kv_heads=4, seq_lens=(700, 90, 2049), num_layers=3)),
+    "hkv4_g7_fp8": dict(w=small(kv_dtype="fp8", num_q_heads=28, num_kv_heads=4, seq_lens=(700, 1300))),
+    "hkv3_fp16": dict(w=small(kv_dtype="fp16", num_q_heads=12, num_kv_heads=3, seq_lens=(640, 77))),
+})
+
+
 @pytest.mark.parametrize("kernel", ["mfma", "valu"])
 @pytest.mark.parametrize("name", list(RESIDENT_CASES))
 def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
@@ -491,6 +507,8 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
         pytest.skip("the vector-unit kernel holds four query heads per KV head")
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)      # take that kernel however small the launch
+    if "workgroups" in case:
+        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", str(case["workgroups"]))
     inp = build_inputs(w, case.get("kv_axis", 0))
     print(f"case={name} kernel={kernel} workload={w}", flush=True)
     caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=case.get("prefill_lens"))
@@ -559,7 +577,7 @@ def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
              ((2176,) * 4, "two_pass"),        # 4 x 17 tiles of 128
              ((8192,) * 4, "resident_mfma"))   # 4 x 64 tiles of 128
     for seq_lens, want in cases:
-        w = small(seq_lens=seq_lens, num_layers=1)
+        w = small(seq_lens=seq_lens, num_layers=1, num_q_heads=32, num_kv_heads=8)
         tables = synth.make_block_tables(w)
         cache = torch.zeros(2, w.pool_blocks, w.block_size, w.num_kv_heads, w.head_dim, dtype=torch.bfloat16, device=DEV)
         kv = ops.PagedKV.from_kv_caches([cache])

@@ -32,6 +32,7 @@ struct FusedPlan {
   int seqs_per_launch;  // whole sequences of maximum length per launch
   int resident;         // workgroups the device holds at once
   int bs_shift;
+  int waves;            // matrix-core kernel: waves per workgroup (8, or 4 with two workgroups per CU)
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();

@@ -419,7 +419,13 @@ int fused_resident_workgroups() {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
     cached[dev] = cus > 0 ? cus : -1;
   }
-  return cached[dev] > 0 ? cached[dev] : 0;
+  int n = cached[dev] > 0 ? cached[dev] : 0;
+  // Tests: pretend the device is smaller, so that small inputs need several launches.
+  if (const char* v = std::getenv("TRIATTN_RESIDENT_WORKGROUPS")) {
+    const int want = std::atoi(v);
+    if (want > 0 && want < n) n = want;
+  }
+  return n;
 }
 
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,

@@ -262,8 +262,13 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
 // QG: groups of four query heads per KV head (1 or 2).
 __device__ __forceinline__ int nsteps_of(int ntok) { return (ntok + 15) >> 4; }
 
-template <int DT, bool IL, int TW, int SL, int QG, int NB>
-__global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
+// W: waves per workgroup.  Eight (one workgroup per CU), or four for models with at most four
+// KV heads: a workgroup of eight would leave half its waves without a head and the CU with half
+// the loads in flight, so two workgroups of four share a CU (half the LDS each; two waves per
+// SIMD either way, which the register budget of 256 is for).
+template <int DT, bool IL, int TW, int SL, int QG, int NB, int W>
+__global__ __launch_bounds__(W * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   static_assert(SL % (16 * NB) == 0, "the slack must hold whole rotations of the step buffers");
   constexpr int RING = TW + SL;
   constexpr int RQ = 4 * QG;                                   // ring floats per token
@@ -285,10 +290,10 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   const int heads_here = min(8, a.Hkv - chunk * 8);
 
   float* ring = lds + wave * (RING * RQ);                      // [RING][query heads of the KV head]
-  float* part = lds + kFusedWaves * (RING * RQ);               // [waves][64][QG][2]
-  float* stats = part + kFusedWaves * 128 * QG;                // [2][32*QG score heads][2]
+  float* part = lds + W * (RING * RQ);                         // [waves][64][QG][2]
+  float* stats = part + W * 128 * QG;                          // [2][32*QG score heads][2]
   uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128 * QG);  // arrive count, claimed, ready
-  for (int i = threadIdx.x; i < kFusedWaves * 128 * QG; i += kFusedThreads) part[i] = 0.f;
+  for (int i = threadIdx.x; i < W * 128 * QG; i += W * kWave) part[i] = 0.f;
   if (threadIdx.x < 8) ctl[threadIdx.x] = 0;
   __syncthreads();
   // From here on the waves of the workgroup run independently.
@@ -708,23 +713,24 @@ __global__ __launch_bounds__(kFusedThreads) void fused_mfma_kernel(FusedArgs a, 
   }
 }
 
-template <int TW, int SL, int QG>
-size_t mfma_lds_bytes() {
-  return ((size_t)kFusedWaves * (TW + SL) * 4 * QG + kFusedWaves * 128 * QG + 128 * QG + 8) * 4;
+template <int TW, int SL, int QG, int W>
+constexpr size_t mfma_lds_bytes() {
+  return ((size_t)W * (TW + SL) * 4 * QG + W * 128 * QG + 128 * QG + 8) * 4;
 }
 
-template <int DT, bool IL, int TW, int SL, int QG, int NB>
+template <int DT, bool IL, int TW, int SL, int QG, int NB, int W = kFusedWaves>
 hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
-  const size_t lds = mfma_lds_bytes<TW, SL, QG>();
-  if (lds > (size_t)kFusedLdsLimit) return hipErrorInvalidValue;
-  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG, NB>);
+  constexpr size_t lds = mfma_lds_bytes<TW, SL, QG, W>();
+  // 8 waves: one workgroup per CU; 4 waves: two (LDS is handed out in blocks of 1280 bytes).
+  static_assert(((lds + 1279) / 1280 * 1280) * (kFusedWaves / W) <= (size_t)kFusedLdsLimit, "LDS of a CU");
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   if (B <= seqs_per_launch) {
     k.packed = 0;
     k.seq_base = 0;
     const int n = B;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB>), dim3(n * k.tiles_per_seq * k.HC), dim3(kFusedThreads), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>), dim3(n * k.tiles_per_seq * k.HC), dim3(W * kWave), lds, s, k, bmat);
     return hipGetLastError();
   }
   // More workgroups than the device holds at once: whole sequences are packed into
@@ -738,7 +744,7 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
   const int launches = ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB>), dim3(resident), dim3(kFusedThreads), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>), dim3(resident), dim3(W * kWave), lds, s, k, bmat);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -746,7 +752,17 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
 }
 
 template <int DT, bool IL>
-hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int seqs_per_launch, int resident, int B, hipStream_t s) {
+hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int seqs_per_launch, int resident, int B,
+                          hipStream_t s) {
+  if (waves == 4) {
+    // Two workgroups per CU: the ring of the largest tile with one rotation of slack less
+    // (a smaller tile is a run-time argument inside it).
+    constexpr int NB4 = DT == TRI_KV_FP8_E4M3 ? 8 : 4;
+    if (k.G > 4) return tw == 512 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4>(k, bmat, seqs_per_launch, resident, B, s)
+                                  : hipErrorInvalidValue;
+    return tw == 1024 ? launch_mfma_t<DT, IL, 1024, 128, 1, NB4, 4>(k, bmat, seqs_per_launch, resident, B, s)
+                      : hipErrorInvalidValue;
+  }
   if (k.G > 4) {
     switch (tw) {   // eight query heads per KV head: 32 bytes of ring per token
       case 512: return launch_mfma_t<DT, IL, 512, 64, 2, 4>(k, bmat, seqs_per_launch, resident, B, s);
@@ -779,11 +795,15 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
     if ((1 << sft) == block_size) bs_shift = sft;
   if (paged && bs_shift < 4) return p;    // a 16-token step must lie inside one block
   const int HC = ceil_div(Hkv, 8);
+  // At most four KV heads: workgroups of four waves, two per CU.
+  const int waves = Hkv <= 4 ? 4 : kFusedWaves;
+  if (waves == 4) resident *= 2;
   const int tws[3] = {256, 512, 1024};
   const int ntw = G > 4 ? 2 : 3;          // the ring of a 1024-token tile fits LDS for four query heads only
   int tw = tws[ntw - 1];
-  for (int i = 0; i < ntw; ++i)
-    if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
+  if (waves == kFusedWaves)               // (four waves: one kernel instance, with the largest ring)
+    for (int i = 0; i < ntw; ++i)
+      if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   int tile = tw, tiles = ceil_div(Tmax, tw);
   if ((int64_t)tiles * HC > resident) return p;
   if ((int64_t)B * tiles * HC <= resident) {
@@ -812,6 +832,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   p.seqs_per_launch = resident / (tiles * HC);
   p.resident = resident;
   p.bs_shift = bs_shift;
+  p.waves = waves;
   return p;
 }
 
@@ -862,13 +883,13 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
-    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
   if (fp16)
-    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
-  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
 }
 
 }  // namespace tri
