@@ -229,7 +229,8 @@ def main() -> int:
     shape = {k: v for k, v in (("num_layers", args.layers), ("num_q_heads", args.q_heads),
                                ("num_kv_heads", args.kv_heads), ("head_dim", args.head_dim)) if v > 0}
     if shape:
-        w = w.scaled(name=w.name + "_" + "_".join(f"{k[4:]}{v}" for k, v in shape.items()), **shape)
+        tags = {"num_layers": "layers", "num_q_heads": "q", "num_kv_heads": "kv", "head_dim": "dim"}
+        w = w.scaled(name=w.name + "_" + "_".join(f"{tags[k]}{v}" for k, v in shape.items()), **shape)
     if args.kv_dtype and args.kv_dtype != w.kv_dtype:
         if "fp8" in (args.kv_dtype, w.kv_dtype):
             raise SystemExit("--kv-dtype switches between bf16 and fp16; the fp8 workload is --config 4")

@@ -490,6 +490,16 @@ RESIDENT_CASES.update({
     "hkv4_g7": dict(w=small(num_q_heads=28, num_kv_heads=4, seq_lens=(700, 90, 2049), num_layers=3)),
     "hkv4_g7_fp8": dict(w=small(kv_dtype="fp8", num_q_heads=28, num_kv_heads=4, seq_lens=(700, 1300))),
     "hkv3_fp16": dict(w=small(kv_dtype="fp16", num_q_heads=12, num_kv_heads=3, seq_lens=(640, 77))),
+    # head dimension 64 (GPT-OSS: 64 query / 8 KV heads)
+    "d64_g8_hkv8": dict(w=small(head_dim=64, num_q_heads=64, num_kv_heads=8, seq_lens=(700, 90, 1500), num_layers=3)),
+    "d64_g4_hkv8_ragged_small_chip": dict(w=small(head_dim=64, num_q_heads=32, num_kv_heads=8,
+                                                  seq_lens=(3000, 70, 6100, 900, 4500, 1), budget=128, num_layers=2),
+                                          workgroups=24),
+    "d64_hkv2": dict(w=small(head_dim=64, seq_lens=(300, 1000, 17))),
+    "d64_interleaved_fp16_g7": dict(w=small(head_dim=64, kv_dtype="fp16", rope_style="interleaved", num_q_heads=28,
+                                            num_kv_heads=4, seq_lens=(640, 2049))),
+    "d64_tile_refined": dict(w=small(head_dim=64, num_q_heads=32, num_kv_heads=8, seq_lens=(3072,) * 16, budget=256,
+                                     num_layers=2)),
 })
 
 
@@ -506,6 +516,8 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
         pytest.skip("the matrix-core kernel needs blocks of at least 16 tokens (a step lies inside one block)")
     if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
         pytest.skip("the vector-unit kernel holds four query heads per KV head")
+    if kernel == "valu" and w.head_dim != 128:
+        pytest.skip("the vector-unit kernel is built for a head dimension of 128")
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)      # take that kernel however small the launch
     if "workgroups" in case:
         monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", str(case["workgroups"]))
@@ -717,7 +729,7 @@ def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
 
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
-    for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=64), {}),
+    for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=256), {}), (dict(head_dim=64, kv_dtype="fp8"), {}),
                       (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
         w = small(**kw)
         inp = build_inputs(w)

@@ -42,9 +42,10 @@ constexpr int kDppRor8m = 0x128;  // row_ror:8
 // MFMA s takes chunk s).  fp8 keys: the 16-byte chunks kb and 4 + kb (16 elements each;
 // MFMA s takes half s % 2 of chunk s / 2) and the dequantisation scale of the token this
 // lane will store.
-template <int DT>
+// HD: head dimension, 128 or (two-byte keys only) 64: half the chunks, MFMAs and pairs.
+template <int DT, int HD>
 struct StepData {
-  uint4 c[DT == TRI_KV_FP8_E4M3 ? 2 : 4];
+  uint4 c[DT == TRI_KV_FP8_E4M3 ? 2 : HD / 32];
   float scale;
 };
 
@@ -162,7 +163,7 @@ constexpr int kPrepThreads = 1024;
 constexpr int kPrepHeads = 64;      // query heads whose coefficients are staged at a time
 constexpr int kPrepPitch = 193;
 
-template <int DT, bool IL>
+template <int DT, bool IL, int HD>
 __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* folded, const float* omega,
                                                                  const float* offsets, int NO,
                                                                  const int32_t* round_start, int L, int Hkv, int G,
@@ -172,6 +173,9 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
   // One buffer, used twice: the per-offset cos / sin values, then the coefficients of up to
   // kPrepHeads query heads as [head][P | R | E][64] with a row pitch of 193 floats (the four
   // query heads and four k blocks a wave reads at once then fall into 16 different banks).
+  constexpr int F = HD / 2;              // frequency pairs
+  constexpr int NS = HD / 32;            // key slabs (MFMAs) per step
+  constexpr int NSO = NS + NS / 2;       // operands per query-head group: key slabs, magnitude slabs
   __shared__ float buf[kPrepHeads * kPrepPitch];
   __shared__ float mean_cs[2][64];
   static_assert(kPrepHeads * kPrepPitch >= 2 * kMaxOffsets * 64, "the trig values must fit the buffer");
@@ -184,10 +188,10 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
   const float rs = (float)round_start[b];
   for (int i = tid; i < NO * 64; i += kPrepThreads) {
     const int j = i >> 6, f = i & 63;
-    phase_cos_sin(__fmul_rn(__fadd_rn(rs, offsets[j]), omega[f]), part[0][j][f], part[1][j][f]);
+    if (f < F) phase_cos_sin(__fmul_rn(__fadd_rn(rs, offsets[j]), omega[f]), part[0][j][f], part[1][j][f]);
   }
   __syncthreads();
-  if (tid < 128) {
+  if (tid < 128 && (tid & 63) < F) {
     const int which = tid >> 6, f = tid & 63;
     double sum = 0.0;
     for (int j = 0; j < NO; ++j) sum += part[which][j][f];
@@ -199,23 +203,23 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
     const int nh = min(heads_per_pass, Hkv - head0);
     __syncthreads();                                        // means written; buffer free
     // P = a1*C - a2*S, R = a2*C + a1*S, E, of query heads head0*G .. (head0 + nh)*G - 1
-    const float* in = folded + ((int64_t)l * A + (int64_t)head0 * G) * 3 * 64;   // [head][a1 | a2 | e][64]
-    for (int i = tid; i < nh * G * 64; i += kPrepThreads) {
-      const int q = i >> 6, f = i & 63;
-      const float a1 = in[q * 192 + f], a2 = in[q * 192 + 64 + f], e = in[q * 192 + 128 + f];
+    const float* in = folded + ((int64_t)l * A + (int64_t)head0 * G) * 3 * F;   // [head][a1 | a2 | e][F]
+    for (int i = tid; i < nh * G * F; i += kPrepThreads) {
+      const int q = i / F, f = i % F;
+      const float a1 = in[q * 3 * F + f], a2 = in[q * 3 * F + F + f], e = in[q * 3 * F + 2 * F + f];
       const float c = mean_cs[0][f], sn = mean_cs[1][f];
       buf[q * kPrepPitch + f] = fmaf(a1, c, -a2 * sn);
-      buf[q * kPrepPitch + 64 + f] = fmaf(a2, c, a1 * sn);
-      buf[q * kPrepPitch + 128 + f] = e;
+      buf[q * kPrepPitch + F + f] = fmaf(a2, c, a1 * sn);
+      buf[q * kPrepPitch + 2 * F + f] = e;
     }
     __syncthreads();
-    const int items = nh * QG * 6 * 64;                     // (head, group, operand, lane)
-    uint4* out_base = bmat + (((int64_t)b * L + l) * Hkv + head0) * QG * 6 * 64;
+    const int items = nh * QG * NSO * 64;                   // (head, group, operand, lane)
+    uint4* out_base = bmat + (((int64_t)b * L + l) * Hkv + head0) * QG * NSO * 64;
     for (int idx = tid; idx < items; idx += kPrepThreads) {
       const int lane = idx & 63;
-      const int o = (idx >> 6) % 6;
-      const int g = (idx / (64 * 6)) % QG;
-      const int head = idx / (64 * 6 * QG);
+      const int o = (idx >> 6) % NSO;
+      const int g = (idx / (64 * NSO)) % QG;
+      const int head = idx / (64 * NSO * QG);
       const int j = lane & 15, kb = lane >> 4;
       const int q = 4 * g + (j & 3), sp = j >> 2;
       uint32_t out[4] = {0, 0, 0, 0};
@@ -226,29 +230,29 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
         for (int e = 0; e < 8; ++e) {
           int which, pair;   // which: 0 = P, 1 = R, 2 = E
           constexpr bool kRegrouped = DT == TRI_KV_FP8_E4M3 && !IL;   // see compute_step
-          if (o < 4) {
+          if (o < NS) {
             const int el = slab_elem<DT>(o, kb, e);
             if (kRegrouped) { which = e & 1; pair = kb * 16 + 4 * o + (e >> 1); }
             else if (IL) { which = el & 1; pair = el >> 1; }
-            else { which = el >= 64 ? 1 : 0; pair = el & 63; }
+            else { which = el >= F ? 1 : 0; pair = el & (F - 1); }
           } else {
             which = 2;
-            const int set = o - 4;
+            const int set = o - NS;
             // interleaved: pairs of MFMAs 2*set and 2*set + 1; half: real parts of MFMA `set`
             if (kRegrouped) pair = kb * 16 + 4 * (2 * set + (e >> 2)) + (e & 3);
             else if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
-            else pair = slab_elem<DT>(set, kb, e) & 63;
+            else pair = slab_elem<DT>(set, kb, e) & (F - 1);
           }
           // One-byte keys: their magnitudes go through the fp16 matrix-core instruction (see
           // compute_step), so the magnitude slabs are fp16 pieces.
-          const bool half_slab = DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= 4);
-          v[e] = half_slab ? coefficient_piece<TRI_KV_FP16>(c[which * 64 + pair], sp)
-                           : coefficient_piece<TRI_KV_BF16>(c[which * 64 + pair], sp);
+          const bool half_slab = DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= NS);
+          v[e] = half_slab ? coefficient_piece<TRI_KV_FP16>(c[which * F + pair], sp)
+                           : coefficient_piece<TRI_KV_BF16>(c[which * F + pair], sp);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const f32x2 x = {v[2 * e], v[2 * e + 1]};
-          if (DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= 4))
+          if (DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= NS))
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
           else
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
@@ -266,9 +270,12 @@ __device__ __forceinline__ int nsteps_of(int ntok) { return (ntok + 15) >> 4; }
 // KV heads: a workgroup of eight would leave half its waves without a head and the CU with half
 // the loads in flight, so two workgroups of four share a CU (half the LDS each; two waves per
 // SIMD either way, which the register budget of 256 is for).
-template <int DT, bool IL, int TW, int SL, int QG, int NB, int W>
+template <int DT, bool IL, int TW, int SL, int QG, int NB, int W, int HD>
 __global__ __launch_bounds__(W * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
+  static_assert(HD == 128 || (HD == 64 && DT != TRI_KV_FP8_E4M3), "head dimensions with a kernel");
+  constexpr int NS = HD / 32;            // key slabs (MFMAs) per step
+  constexpr int NSO = NS + NS / 2;       // operands per query-head group
   static_assert(SL % (16 * NB) == 0, "the slack must hold whole rotations of the step buffers");
   constexpr int RING = TW + SL;
   constexpr int RQ = 4 * QG;                                   // ring floats per token
@@ -304,13 +311,13 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   const int q = j & 3, rsel = j >> 2;
 
   // Coefficient slabs of the current layer.
-  uint4 B[QG][6];
+  uint4 B[QG][NSO];
   auto load_coefs = [&](int l) __attribute__((always_inline)) {
-    const uint4* p = bmat + (((int64_t)(b * a.L + l) * a.Hkv + head) * QG * 6) * 64 + lane;
+    const uint4* p = bmat + (((int64_t)(b * a.L + l) * a.Hkv + head) * QG * NSO) * 64 + lane;
 #pragma unroll
     for (int g = 0; g < QG; ++g)
 #pragma unroll
-      for (int o = 0; o < 6; ++o) B[g][o] = p[(g * 6 + o) * 64];
+      for (int o = 0; o < NSO; ++o) B[g][o] = p[(g * NSO + o) * 64];
     if constexpr (DT == TRI_KV_FP16 || DT == TRI_KV_FP8_E4M3) {
       // A coefficient beyond fp16's range (65504) arrives as an infinity: the scores of this
       // launch would be meaningless, so the status word is raised (the caller repeats the
@@ -320,7 +327,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
 #pragma unroll
       for (int g = 0; g < QG; ++g)
 #pragma unroll
-        for (int o = (DT == TRI_KV_FP16 ? 0 : 4); o < 6; ++o) {
+        for (int o = (DT == TRI_KV_FP16 ? 0 : NS); o < NSO; ++o) {
           const uint32_t w4[4] = {B[g][o].x, B[g][o].y, B[g][o].z, B[g][o].w};
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -377,7 +384,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     step_off_hi = (uint32_t)((uint64_t)off >> 32);
     step_slot = step_blk * a.block_size + in_blk;
   }
-  auto load_step = [&](StepData<DT>& d, const LayerBase& lb, int t) __attribute__((always_inline)) {
+  auto load_step = [&](StepData<DT, HD>& d, const LayerBase& lb, int t) __attribute__((always_inline)) {
     if constexpr (FP8) {
       const int step = t >> 4;
       const uint32_t rows_left = (uint32_t)(last_tok - (n0 + t));
@@ -408,7 +415,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     GlobalBytes p = (GlobalBytes)(uintptr_t)base + off;
     d.scale = 1.f;
 #pragma unroll
-    for (int s = 0; s < (FP8 ? 2 : 4); ++s) {
+    for (int s = 0; s < (FP8 ? 2 : NS); ++s) {
       const u32x4 v = *(GlobalU4)(p + s * 64);
       d.c[s] = uint4{v.x, v.y, v.z, v.w};
     }
@@ -426,10 +433,10 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   for (int g = 0; g < QG; ++g) { s1[g] = 0.f; s2[g] = 0.f; }
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
-  auto compute_step = [&](const StepData<DT>& raw, int l, int t) __attribute__((always_inline)) {
+  auto compute_step = [&](const StepData<DT, HD>& raw, int l, int t) __attribute__((always_inline)) {
     // The four bf16 A operands of the step as dwords (two elements each): the loaded
     // registers for bf16 keys, one conversion per dword (exact) for fp8 keys.
-    uint32_t w[4][4];
+    uint32_t w[NS][4];
     // One-byte keys in the half-split layout: lane block kb holds the real parts of pairs
     // 16*kb .. 16*kb + 15 in c[0] and their imaginary parts in c[1].  Two byte permutes per
     // dword pair put (real, imaginary) next to each other before the conversion, so every
@@ -462,24 +469,24 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+      for (int s = 0; s < NS; ++s) {
         w[s][0] = raw.c[s].x; w[s][1] = raw.c[s].y; w[s][2] = raw.c[s].z; w[s][3] = raw.c[s].w;
       }
     }
-    struct { uint4 c[4]; } d;
+    struct { uint4 c[NS]; } d;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) d.c[s] = uint4{w[s][0], w[s][1], w[s][2], w[s][3]};
+    for (int s = 0; s < NS; ++s) d.c[s] = uint4{w[s][0], w[s][1], w[s][2], w[s][3]};
     f32x4 acc[QG], acc_e[QG];
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < 4; ++s)
+      for (int s = 0; s < NS; ++s)
         acc[g] = mfma_step<DT>(d.c[s], B[g][s], acc[g]);
       acc_e[g] = acc[g];   // the magnitude MFMAs continue the sum (the key MFMAs are long done by then)
     }
 #pragma unroll
-    for (int set = 0; set < 2; ++set) {
+    for (int set = 0; set < NS / 2; ++set) {
       // |k_f|^2 = k_r^2 + k_i^2 straight from the bf16 pairs (v_dot2_f32_bf16).
       // interleaved: dword e % 4 of operand 2*set + e/4 is the (real, imaginary) pair;
       // half: real parts in operand `set`, imaginary parts in operand `set + 2`, regrouped
@@ -494,7 +501,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
         } else {
 #pragma unroll
           for (int i = 0; i < 2; ++i) {
-            const uint32_t re = w[set][2 * h + i], im = w[set + 2][2 * h + i];
+            const uint32_t re = w[set][2 * h + i], im = w[set + NS / 2][2 * h + i];
             x[2 * i] = __builtin_amdgcn_perm(im, re, 0x05040100u);
             x[2 * i + 1] = __builtin_amdgcn_perm(im, re, 0x07060302u);
           }
@@ -529,8 +536,8 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       constexpr int MT = FP8 ? TRI_KV_FP16 : DT;     // operand type of the magnitude MFMAs
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
-        acc_e[g] = mfma_step<MT>(hi, B[g][4 + set], acc_e[g]);
-        acc_e[g] = mfma_step<MT>(lo, B[g][4 + set], acc_e[g]);
+        acc_e[g] = mfma_step<MT>(hi, B[g][NS + set], acc_e[g]);
+        acc_e[g] = mfma_step<MT>(lo, B[g][NS + set], acc_e[g]);
       }
     }
     const int tl = t + 4 * kb + rsel;
@@ -671,10 +678,10 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   const int nsteps = (ntok + 15) >> 4;
   const int rotations = (nsteps + NB - 1) / NB;
   const int rot_before_consume = min(SL / (16 * NB), rotations);
-  auto score = [&](const StepData<DT>& d, int l, int slot) __attribute__((always_inline)) {
+  auto score = [&](const StepData<DT, HD>& d, int l, int slot) __attribute__((always_inline)) {
     if (slot < nsteps) compute_step(d, l, slot * 16);
   };
-  StepData<DT> buf[NB];
+  StepData<DT, HD> buf[NB];
   LayerBase base_cur = layer_base(0), base_next = base_cur;
   auto rotate = [&](int l, int r0, int r1) __attribute__((always_inline)) {
     for (int r = r0; r < r1; ++r) {
@@ -718,19 +725,19 @@ constexpr size_t mfma_lds_bytes() {
   return ((size_t)W * (TW + SL) * 4 * QG + W * 128 * QG + 128 * QG + 8) * 4;
 }
 
-template <int DT, bool IL, int TW, int SL, int QG, int NB, int W = kFusedWaves>
+template <int DT, bool IL, int TW, int SL, int QG, int NB, int W = kFusedWaves, int HD = 128>
 hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
   constexpr size_t lds = mfma_lds_bytes<TW, SL, QG, W>();
   // 8 waves: one workgroup per CU; 4 waves: two (LDS is handed out in blocks of 1280 bytes).
   static_assert(((lds + 1279) / 1280 * 1280) * (kFusedWaves / W) <= (size_t)kFusedLdsLimit, "LDS of a CU");
-  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>);
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   if (B <= seqs_per_launch) {
     k.packed = 0;
     k.seq_base = 0;
     const int n = B;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>), dim3(n * k.tiles_per_seq * k.HC), dim3(W * kWave), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>), dim3(n * k.tiles_per_seq * k.HC), dim3(W * kWave), lds, s, k, bmat);
     return hipGetLastError();
   }
   // More workgroups than the device holds at once: whole sequences are packed into
@@ -744,7 +751,7 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
   const int launches = ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
-    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W>), dim3(resident), dim3(W * kWave), lds, s, k, bmat);
+    hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>), dim3(resident), dim3(W * kWave), lds, s, k, bmat);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -752,8 +759,24 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
 }
 
 template <int DT, bool IL>
-hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int seqs_per_launch, int resident, int B,
-                          hipStream_t s) {
+hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int head_dim, int seqs_per_launch,
+                          int resident, int B, hipStream_t s) {
+  if (head_dim == 64) {
+    // Half the bytes per row: eight step buffers keep as many bytes in flight (four query heads
+    // per KV head; with eight the LDS has no room for the slack that eight buffers need).  One
+    // instance per shape, with the largest ring.
+    if constexpr (DT != TRI_KV_FP8_E4M3) {
+      if (k.G > 4) {
+        if (tw != 512) return hipErrorInvalidValue;
+        return waves == 4 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4, 64>(k, bmat, seqs_per_launch, resident, B, s)
+                          : launch_mfma_t<DT, IL, 512, 64, 2, 4, 8, 64>(k, bmat, seqs_per_launch, resident, B, s);
+      }
+      if (tw != 1024) return hipErrorInvalidValue;
+      return waves == 4 ? launch_mfma_t<DT, IL, 1024, 128, 1, 8, 4, 64>(k, bmat, seqs_per_launch, resident, B, s)
+                        : launch_mfma_t<DT, IL, 1024, 128, 1, 8, 8, 64>(k, bmat, seqs_per_launch, resident, B, s);
+    }
+    return hipErrorInvalidValue;
+  }
   if (waves == 4) {
     // Two workgroups per CU: the ring of the largest tile with one rotation of slack less
     // (a smaller tile is a run-time argument inside it).
@@ -788,7 +811,8 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, in
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                           int resident, bool any_fill, int kv_dtype) {
   FusedPlan p{};
-  if (resident <= 0 || D != 128 || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
+  const bool dim_ok = D == 128 || (D == 64 && kv_dtype != TRI_KV_FP8_E4M3);
+  if (resident <= 0 || !dim_ok || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
   int bs_shift = -1;
   for (int sft = 0; sft < 31; ++sft)
@@ -801,7 +825,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   const int tws[3] = {256, 512, 1024};
   const int ntw = G > 4 ? 2 : 3;          // the ring of a 1024-token tile fits LDS for four query heads only
   int tw = tws[ntw - 1];
-  if (waves == kFusedWaves)               // (four waves: one kernel instance, with the largest ring)
+  if (waves == kFusedWaves && D == 128)   // (four waves, head dimension 64: one kernel instance, with the largest ring)
     for (int i = 0; i < ntw; ++i)
       if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   int tile = tw, tiles = ceil_div(Tmax, tw);
@@ -814,7 +838,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
     // per-layer work of a workgroup too often, and every workgroup gathers the statistics of
     // all tiles of its sequence (one sequence of 16384 tokens as 256 tiles of 64 fills the
     // chip and takes 1.14 ms; the two-pass kernels take 0.38).
-    const int granule = kv_dtype == TRI_KV_FP8_E4M3 ? 128 : 64;
+    const int granule = (kv_dtype == TRI_KV_FP8_E4M3 || (D == 64 && G <= 4)) ? 128 : 64;   // a rotation of the step buffers
     const int tiles_max = min(resident / (B * HC), 64);
     tile = ceil_div(ceil_div(Tmax, tiles_max), granule) * granule;
     tile = min(tw, max(128, tile));
@@ -865,31 +889,42 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
   const bool fp16 = a.kv_dtype == TRI_KV_FP16;
   if (a.kv_dtype != TRI_KV_BF16 && !fp8 && !fp16) return hipErrorInvalidValue;
-  if (a.NO <= 0 || a.NO > kMaxOffsets || a.D != 128) return hipErrorInvalidValue;
+  if (a.NO <= 0 || a.NO > kMaxOffsets || (a.D != 128 && a.D != 64)) return hipErrorInvalidValue;
+  if (a.D == 64 && fp8) return hipErrorInvalidValue;
   auto prep_launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)a.L, (unsigned)a.B), dim3(kPrepThreads), 0, s, a.folded, a.omega,
                        a.offsets, a.NO, a.round_start, a.L, a.Hkv, a.G, a.A, QG, bmat, a.xchg, words, a.status);
   };
   if (fp8) {
-    if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, true>);
-    else prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, false>);
+    if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, true, 128>);
+    else prep_launch(prep_mfma_kernel<TRI_KV_FP8_E4M3, false, 128>);
   } else if (fp16) {
-    if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true>);
-    else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false>);
+    if (a.D == 64) {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true, 64>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false, 64>);
+    } else {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true, 128>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false, 128>);
+    }
   } else {
-    if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true>);
-    else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false>);
+    if (a.D == 64) {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true, 64>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false, 64>);
+    } else {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true, 128>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false, 128>);
+    }
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
-    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
   if (fp16)
-    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
-  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
+            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
 }
 
 }  // namespace tri
