@@ -847,7 +847,10 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   // A launch that fills fewer than ~60 % of the CUs loses to the two-pass kernels, which
   // spread a small problem over the whole chip (16 sequences: even at 2176 tokens = 56 % of
   // the CUs, 10 % ahead at 2560 = 62 %, 21 % ahead at 3072 = 75 %).
-  if (!any_fill && (int64_t)B * tiles * HC * 10 < (int64_t)resident * 6) return p;
+  // (Workgroups of four waves: 45 %.  28 query / 4 KV heads, 16 x 2176 tokens, 272 of 512
+  // workgroups: 0.40 ms against 0.48 ms on the two-pass kernels.)
+  const int64_t need = waves == 4 ? 45 : 60;
+  if (!any_fill && (int64_t)B * tiles * HC * 100 < (int64_t)resident * need) return p;
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;
