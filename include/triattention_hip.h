@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 2
+#define TRI_ABI_VERSION 3
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -81,6 +81,9 @@ typedef struct tri_batch {
   const int32_t* round_start;   /* [num_seqs] num_computed_tokens (runtime/hook_group_pipeline.py:78) */
   const int32_t* prefill_lens;  /* [num_seqs] or NULL (=0) */
   const int32_t* budgets;       /* [num_seqs] k = min(budget_total, T) (runtime/selector_hf.py:823) */
+  const int32_t* seq_lens_host; /* HOST copy of seq_lens, or NULL.  With it a batch that needs several resident
+                                 * launches gets the tile size that fills them best and exactly as many
+                                 * launches as it needs (without: the worst case for max_seq_len). */
 } tri_batch;
 
 /* Scoring statistics, already resolved per runtime layer (layer index modulo the

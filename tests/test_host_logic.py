@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.tri_abi_version() == 2
+    assert lib.tri_abi_version() == 3
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():

@@ -46,7 +46,7 @@ class Batch(C.Structure):
         ("num_seqs", C.c_int32), ("max_seq_len", C.c_int32), ("max_budget", C.c_int32),
         ("block_table_pitch", C.c_int32),
         ("block_table", C.c_void_p), ("seq_lens", C.c_void_p), ("round_start", C.c_void_p),
-        ("prefill_lens", C.c_void_p), ("budgets", C.c_void_p),
+        ("prefill_lens", C.c_void_p), ("budgets", C.c_void_p), ("seq_lens_host", C.c_void_p),
     ]
 
 
@@ -114,8 +114,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         if fn.restype is C.c_int and name not in ("tri_abi_version",):
             fn.restype = C.c_int
-    if lib.tri_abi_version() != 2:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 2; rebuild the library")
+    if lib.tri_abi_version() != 3:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 3; rebuild the library")
     _lib = lib
     return lib
 

@@ -62,6 +62,11 @@ int check_batch(const tri_batch* b, bool need_budget) {
   if (!b->seq_lens) return fail(TRI_ERR_INVALID_ARGUMENT, "seq_lens is NULL");
   if (b->block_table && b->block_table_pitch <= 0)
     return fail(TRI_ERR_INVALID_ARGUMENT, "block_table_pitch %d", b->block_table_pitch);
+  if (b->seq_lens_host)
+    for (int i = 0; i < b->num_seqs; ++i)
+      if (b->seq_lens_host[i] < 0 || b->seq_lens_host[i] > b->max_seq_len)
+        return fail(TRI_ERR_INVALID_ARGUMENT, "seq_lens_host[%d] = %d not in [0, max_seq_len = %d]", i,
+                    b->seq_lens_host[i], b->max_seq_len);
   if (need_budget) {
     if (!b->budgets) return fail(TRI_ERR_INVALID_ARGUMENT, "budgets is NULL");
     if (b->max_budget <= 0) return fail(TRI_ERR_INVALID_ARGUMENT, "max_budget %d", b->max_budget);
@@ -103,7 +108,7 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   tri::FusedPlan fused{};
   if (want_mfma)
     fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
-                                 sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype);
+                                 sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype, b->seq_lens_host);
   if (!fused.eligible && !f_mfma)
     fused = tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged, sp->aggregation,
                             b->max_seq_len, resident, f_valu);

@@ -33,6 +33,7 @@ struct FusedPlan {
   int resident;         // workgroups the device holds at once
   int bs_shift;
   int waves;            // matrix-core kernel: waves per workgroup (8, or 4 with two workgroups per CU)
+  int launches;         // matrix-core kernel, several launches: how many (0: the worst case for the longest sequence)
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();
@@ -40,7 +41,7 @@ int fused_resident_workgroups();
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                      int resident, bool any_fill);
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill, int kv_dtype);
+                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens = nullptr);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {

@@ -20,6 +20,9 @@
 // of the vector-unit kernel's instruction count), so bf16 keys run at the key stream's pace.
 // fp8 e4m3 keys are widened to bf16 (exact) in registers and take the same route; the
 // per-(token, head) scale multiplies the finished score.
+#include <algorithm>
+#include <vector>
+
 #include "tri_common.h"
 #include "tri_score_device.h"
 #include "tri_fused_device.h"
@@ -727,6 +730,8 @@ constexpr size_t mfma_lds_bytes() {
 
 template <int DT, bool IL, int TW, int SL, int QG, int NB, int W = kFusedWaves, int HD = 128>
 hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
+  const int known_launches = k.launch_idx;   // handed over in this field (0: unknown)
+  k.launch_idx = 0;
   constexpr size_t lds = mfma_lds_bytes<TW, SL, QG, W>();
   // 8 waves: one workgroup per CU; 4 waves: two (LDS is handed out in blocks of 1280 bytes).
   static_assert(((lds + 1279) / 1280 * 1280) * (kFusedWaves / W) <= (size_t)kFusedLdsLimit, "LDS of a CU");
@@ -748,7 +753,7 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
                      const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base));
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const int launches = ceil_div(B, seqs_per_launch);
+  const int launches = known_launches > 0 ? known_launches : ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
     hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>), dim3(resident), dim3(W * kWave), lds, s, k, bmat);
@@ -806,10 +811,41 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, in
   }
 }
 
+// What fused_pack_kernel will do with these lengths, on the host: sequences by falling tile
+// count, each into the first of the eight most recently opened launches with room.  Returns the
+// number of launches.
+int host_pack_launches(const int32_t* lens, int B, int tile, int wg_mult, int capacity) {
+  std::vector<int> tiles(B);
+  for (int i = 0; i < B; ++i) tiles[i] = ceil_div(lens[i], tile);
+  std::vector<int> order(B);
+  for (int i = 0; i < B; ++i) order[i] = i;
+  if (B <= 4096)   // (the kernel sorts up to that many)
+    std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return tiles[x] > tiles[y]; });
+  int used[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  int first = 0, open = 1;
+  for (int i = 0; i < B; ++i) {
+    const int n = tiles[order[i]] * wg_mult;
+    int pick = -1;
+    for (int c = 0; c < open; ++c)
+      if (used[c] + n <= capacity) { pick = c; break; }
+    if (pick < 0) {
+      if (open == 8) {
+        for (int c = 0; c < 7; ++c) used[c] = used[c + 1];
+        ++first;
+        --open;
+      }
+      pick = open++;
+      used[pick] = 0;
+    }
+    used[pick] += n;
+  }
+  return first + open;
+}
+
 }  // namespace
 
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill, int kv_dtype) {
+                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens) {
   FusedPlan p{};
   const bool dim_ok = D == 128 || (D == 64 && kv_dtype != TRI_KV_FP8_E4M3);
   if (resident <= 0 || !dim_ok || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
@@ -860,6 +896,28 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   p.resident = resident;
   p.bs_shift = bs_shift;
   p.waves = waves;
+  p.launches = 0;
+  if (host_lens && (int64_t)B * tiles * HC > resident) {
+    // Several launches, and the lengths are known: a launch takes as long as its tiles are
+    // long, however many of its workgroups have work, so the tile size that packs the
+    // sequences into the fewest tile-lengths wins (64 sequences of 2k-32k tokens: 1120 tiles of
+    // 1024 tokens are 4.4 launches' worth and take five; tiles of 896 fill five launches).
+    const int granule = (kv_dtype == TRI_KV_FP8_E4M3 || (D == 64 && G <= 4)) ? 128 : 64;
+    int64_t best_cost = -1;
+    for (int cand = tw; cand >= tw / 2 && cand >= 128; cand -= granule) {
+      const int per_seq = ceil_div(Tmax, cand) * HC;
+      if (per_seq > resident) break;
+      const int n = host_pack_launches(host_lens, B, cand, HC, resident);
+      const int64_t cost = (int64_t)n * (cand + 32);      // 32 tokens' worth of fixed work per launch and layer
+      if (best_cost < 0 || cost < best_cost) {
+        best_cost = cost;
+        p.tile_tokens = cand;
+        p.tiles_per_seq = ceil_div(Tmax, cand);
+        p.seqs_per_launch = resident / per_seq;
+        p.launches = n;
+      }
+    }
+  }
   return p;
 }
 
@@ -885,6 +943,7 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.spin_ticks = resident_spin_ticks();
   k.seq_launch = a.pack;
   k.seq_wg_base = a.pack + a.B;
+  k.launch_idx = a.plan.launches;   // read and reset by launch_mfma_t
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
   const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);

@@ -225,11 +225,12 @@ class StepBatch:
                 raise ValueError("block table rows != number of sequences")
         self.max_seq_len = max(self.seq_lens_host)
         self.max_budget = max(self.budgets_host) if self.budgets_host else 0
+        self._lens_host = (C.c_int32 * n)(*self.seq_lens_host)     # kept alive with the batch
         self.struct = Batch(
             num_seqs=self.num_seqs, max_seq_len=self.max_seq_len, max_budget=self.max_budget,
             block_table_pitch=pitch, block_table=_ptr(self.block_table), seq_lens=_ptr(self.seq_lens),
             round_start=_ptr(self.round_start), prefill_lens=_ptr(self.prefill_lens),
-            budgets=_ptr(self.budgets))
+            budgets=_ptr(self.budgets), seq_lens_host=C.cast(self._lens_host, C.c_void_p))
 
     def check_capacity(self, block_size: int) -> None:
         """Host-side bounds check: every sequence owns enough blocks for its tokens."""
