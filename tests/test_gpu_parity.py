@@ -2,6 +2,8 @@
 reference's own outputs (golden fixtures).  All tests need an MI355X."""
 from __future__ import annotations
 
+import os
+
 import pytest
 import torch
 
@@ -349,6 +351,26 @@ def test_compaction_large_budget_and_dims():
     _compact_case(small(seq_lens=(700,), budget=300, head_dim=256, block_size=8), 0, True, False, False)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TRIATTN_TEST_RANDOM_SHAPES", "32"))))
+def test_compaction_on_random_shapes(seed):
+    """Seeded random head counts, head dimensions, block sizes, ragged lengths, budgets per
+    sequence (from a single row to all but a few) and modes, bit-exact against the oracle."""
+    import random
+    r = random.Random(1000 + seed)
+    hkv = r.choice([1, 2, 3, 4, 5, 7, 8, 9, 16])
+    nseq = r.choice([1, 2, 3, 6])
+    seq_lens = tuple(r.choice([1, 2, 15, 16, 17, 100, 257, 1000, 1500, 2176, 4100]) for _ in range(nseq))
+    budgets = [max(1, r.choice([1, 7, t // 8, t // 2, t - 1, t - 128, t, t + 5])) for t in seq_lens]
+    w = small(seq_lens=seq_lens, num_layers=r.choice([1, 2, 3]), num_q_heads=hkv, num_kv_heads=hkv,
+              head_dim=r.choice([64, 128, 128, 256]), block_size=r.choice([1, 8, 16, 16, 24, 32, 128]),
+              budget=max(budgets), index=200 + seed)
+    kv_axis, shared = r.choice([0, 1]), r.random() < 0.4
+    per_layer, full = r.random() < 0.3, r.random() < 0.25
+    print(f"compaction seed={seed} workload={w} budgets={budgets} kv_axis={kv_axis} shared={shared} "
+          f"per_layer={per_layer} full={full}", flush=True)
+    _compact_case(w, kv_axis, shared, per_layer, full, budgets=budgets)
+
+
 @pytest.mark.parametrize("heads", [3, 5, 6, 7])
 def test_shared_compaction_with_token_rows_that_do_not_divide_a_tile(heads):
     """One index list for all heads moves whole token rows; with 3, 5, 6 or 7 heads a row's
@@ -543,6 +565,42 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
         assert float((fr[finite] - ft[finite]).abs().max() if bool(finite.any()) else 0.0) <= 5e-4 * scale, (name, b)
         assert_keep_matches(keep_r[b * h:(b + 1) * h, :k].cpu().long(), keep_t[b * h:(b + 1) * h, :k].cpu().long(),
                             ft, k, tie_tol=2e-3 * scale)
+
+
+def _random_resident_case(seed: int):
+    """A seeded random shape the matrix-core kernel has an instance for."""
+    import random
+    r = random.Random(seed)
+    kv_dtype = r.choice(["bf16", "bf16", "fp16", "fp8"])
+    head_dim = 128 if kv_dtype == "fp8" else r.choice([128, 128, 64])
+    hkv = r.choice([1, 2, 3, 4, 5, 8, 8, 12])
+    g = r.choice([1, 2, 3, 4, 4, 6, 7, 8])
+    nseq = r.choice([1, 2, 3, 5, 9])
+    seq_lens = tuple(r.choice([1, 15, 16, 17, 63, 64, 65, 127, 129, 300, 511, 513, 1023, 1025, 2049, 3000])
+                     for _ in range(nseq))
+    w = small(kv_dtype=kv_dtype, head_dim=head_dim, num_q_heads=hkv * g, num_kv_heads=hkv, seq_lens=seq_lens,
+              num_layers=r.choice([1, 2, 3]), budget=r.choice([1, 16, 96, 200]), block_size=r.choice([16, 16, 32, 128]),
+              window_size=r.choice([0, 1, 12, 200]), rope_style=r.choice(["half", "interleaved"]), index=100 + seed)
+    case = dict(w=w, sel=dict(normalize=r.random() < 0.8, group_reduce=r.choice(["max", "max", "mean"]),
+                              layer_reduce=r.choice(["mean", "mean", "max"])))
+    if r.random() < 0.3:
+        case["sel"]["protect_prefill"] = True
+        case["prefill_lens"] = [r.randrange(0, t + 1) for t in seq_lens]
+    if r.random() < 0.4:
+        case["workgroups"] = r.choice([8, 16, 40])
+    return case
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TRIATTN_TEST_RANDOM_SHAPES", "32"))))
+def test_matrix_core_kernel_on_random_shapes(seed, monkeypatch):
+    """Seeded random head layouts, key types, head dimensions, ragged lengths, block sizes, guards
+    and device sizes: resident matrix-core selection against the two-pass kernels."""
+    case = _random_resident_case(seed)
+    RESIDENT_CASES[f"random{seed}"] = case
+    try:
+        test_resident_selection_matches_two_pass(f"random{seed}", "mfma", monkeypatch)
+    finally:
+        del RESIDENT_CASES[f"random{seed}"]
 
 
 @pytest.mark.parametrize("kernel", ["mfma", "valu"])
