@@ -723,15 +723,23 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   }
 }
 
+// How a batch is cut into launches (from the plan).
+struct LaunchShape {
+  int seqs_per_launch;   // whole sequences of maximum length one launch holds
+  int resident;          // workgroups the device holds at once
+  int num_seqs;
+  int launches;          // > 0: exactly this many (the planner replayed the device's packing); 0: the worst case
+};
+
 template <int TW, int SL, int QG, int W>
 constexpr size_t mfma_lds_bytes() {
   return ((size_t)W * (TW + SL) * 4 * QG + W * 128 * QG + 128 * QG + 8) * 4;
 }
 
 template <int DT, bool IL, int TW, int SL, int QG, int NB, int W = kFusedWaves, int HD = 128>
-hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, int resident, int B, hipStream_t s) {
-  const int known_launches = k.launch_idx;   // handed over in this field (0: unknown)
-  k.launch_idx = 0;
+hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, const LaunchShape& shape, hipStream_t s) {
+  const int seqs_per_launch = shape.seqs_per_launch, resident = shape.resident, B = shape.num_seqs;
+  const int known_launches = shape.launches;
   constexpr size_t lds = mfma_lds_bytes<TW, SL, QG, W>();
   // 8 waves: one workgroup per CU; 4 waves: two (LDS is handed out in blocks of 1280 bytes).
   static_assert(((lds + 1279) / 1280 * 1280) * (kFusedWaves / W) <= (size_t)kFusedLdsLimit, "LDS of a CU");
@@ -764,8 +772,8 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, int seqs_per_launch, i
 }
 
 template <int DT, bool IL>
-hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int head_dim, int seqs_per_launch,
-                          int resident, int B, hipStream_t s) {
+hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int head_dim, const LaunchShape& shape,
+                          hipStream_t s) {
   if (head_dim == 64) {
     // Half the bytes per row: eight step buffers keep as many bytes in flight (four query heads
     // per KV head; with eight the LDS has no room for the slack that eight buffers need).  One
@@ -773,12 +781,12 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, in
     if constexpr (DT != TRI_KV_FP8_E4M3) {
       if (k.G > 4) {
         if (tw != 512) return hipErrorInvalidValue;
-        return waves == 4 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4, 64>(k, bmat, seqs_per_launch, resident, B, s)
-                          : launch_mfma_t<DT, IL, 512, 64, 2, 4, 8, 64>(k, bmat, seqs_per_launch, resident, B, s);
+        return waves == 4 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4, 64>(k, bmat, shape, s)
+                          : launch_mfma_t<DT, IL, 512, 64, 2, 4, 8, 64>(k, bmat, shape, s);
       }
       if (tw != 1024) return hipErrorInvalidValue;
-      return waves == 4 ? launch_mfma_t<DT, IL, 1024, 128, 1, 8, 4, 64>(k, bmat, seqs_per_launch, resident, B, s)
-                        : launch_mfma_t<DT, IL, 1024, 128, 1, 8, 8, 64>(k, bmat, seqs_per_launch, resident, B, s);
+      return waves == 4 ? launch_mfma_t<DT, IL, 1024, 128, 1, 8, 4, 64>(k, bmat, shape, s)
+                        : launch_mfma_t<DT, IL, 1024, 128, 1, 8, 8, 64>(k, bmat, shape, s);
     }
     return hipErrorInvalidValue;
   }
@@ -786,15 +794,15 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, in
     // Two workgroups per CU: the ring of the largest tile with one rotation of slack less
     // (a smaller tile is a run-time argument inside it).
     constexpr int NB4 = DT == TRI_KV_FP8_E4M3 ? 8 : 4;
-    if (k.G > 4) return tw == 512 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4>(k, bmat, seqs_per_launch, resident, B, s)
+    if (k.G > 4) return tw == 512 ? launch_mfma_t<DT, IL, 512, 64, 2, 4, 4>(k, bmat, shape, s)
                                   : hipErrorInvalidValue;
-    return tw == 1024 ? launch_mfma_t<DT, IL, 1024, 128, 1, NB4, 4>(k, bmat, seqs_per_launch, resident, B, s)
+    return tw == 1024 ? launch_mfma_t<DT, IL, 1024, 128, 1, NB4, 4>(k, bmat, shape, s)
                       : hipErrorInvalidValue;
   }
   if (k.G > 4) {
     switch (tw) {   // eight query heads per KV head: 32 bytes of ring per token
-      case 512: return launch_mfma_t<DT, IL, 512, 64, 2, 4>(k, bmat, seqs_per_launch, resident, B, s);
-      case 256: return launch_mfma_t<DT, IL, 256, 64, 2, 4>(k, bmat, seqs_per_launch, resident, B, s);
+      case 512: return launch_mfma_t<DT, IL, 512, 64, 2, 4>(k, bmat, shape, s);
+      case 256: return launch_mfma_t<DT, IL, 256, 64, 2, 4>(k, bmat, shape, s);
       default: return hipErrorInvalidValue;
     }
   }
@@ -804,9 +812,9 @@ hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, in
   // (16 x 16384 tokens x 36 layers, bf16, warm GPU: 3.54 ms with 64, 3.49 with 128, 3.45 with 192).
   constexpr int SL = DT == TRI_KV_FP8_E4M3 ? 128 : 192;
   switch (tw) {
-    case 1024: return launch_mfma_t<DT, IL, 1024, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
-    case 512: return launch_mfma_t<DT, IL, 512, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
-    case 256: return launch_mfma_t<DT, IL, 256, SL, 1, NB>(k, bmat, seqs_per_launch, resident, B, s);
+    case 1024: return launch_mfma_t<DT, IL, 1024, SL, 1, NB>(k, bmat, shape, s);
+    case 512: return launch_mfma_t<DT, IL, 512, SL, 1, NB>(k, bmat, shape, s);
+    case 256: return launch_mfma_t<DT, IL, 256, SL, 1, NB>(k, bmat, shape, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -943,7 +951,7 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.spin_ticks = resident_spin_ticks();
   k.seq_launch = a.pack;
   k.seq_wg_base = a.pack + a.B;
-  k.launch_idx = a.plan.launches;   // read and reset by launch_mfma_t
+  const LaunchShape shape{a.plan.seqs_per_launch, a.plan.resident, a.B, a.plan.launches};
   const int64_t words = (int64_t)a.B * a.L * k.tiles_per_seq * a.A * 2;
   const bool il = a.rope_style == TRI_ROPE_INTERLEAVED;
   uint4* bmat = reinterpret_cast<uint4*>(a.bmat);
@@ -980,13 +988,13 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
-    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
   if (fp16)
-    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
-  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s)
-            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, a.plan.seqs_per_launch, a.plan.resident, a.B, s);
+    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
+  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
 }
 
 }  // namespace tri
