@@ -160,9 +160,12 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                                protect_prefill=bool(protect_prefill and prefill_len > 0),
                                group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared)
         try:
-            keep, _, _ = ops.select_paged(kv, batch, sc, sel)
+            resident = ops.select_path(kv, batch, sc, sel) != "two_pass"   # (a single request: only when forced)
+            keep, _, ws = ops.select_paged(kv, batch, sc, sel)
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
+        if resident and ws.status() != 0:
+            raise RuntimeError(f"{MARK}:score_failed:ResidentLaunchFailed")
         return mark_keep_validated(keep.to(torch.long), total_tokens)
 
     def _select_keep_indices(*, keys_dense: torch.Tensor | None = None, kv_cache: torch.Tensor | None = None,
