@@ -627,6 +627,30 @@ def test_matrix_core_kernel_on_random_shapes(seed, monkeypatch):
         del RESIDENT_CASES[f"random{seed}"]
 
 
+@pytest.mark.parametrize("kv_dtype,head_dim", [("bf16", 128), ("fp16", 128), ("fp8", 128), ("bf16", 64), ("fp16", 64)])
+def test_matrix_core_scores_carry_every_piece(kv_dtype, head_dim, monkeypatch):
+    """Without normalisation and with a layer maximum the raw scores show through: the
+    matrix-core kernel (coefficients in three pieces, magnitudes in two) agrees with the
+    two-pass kernels' fp32 arithmetic to 5e-6 of the largest score (measured: 2e-7 .. 1.5e-6);
+    a dropped second piece of the magnitudes would show as 1e-4 .. 2e-3."""
+    w = small(kv_dtype=kv_dtype, head_dim=head_dim, seq_lens=(3000, 1000), index=77)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size, normalize=False, layer_reduce="max")
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    _, fin_r, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    _, fin_t, _ = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    torch.cuda.synchronize()
+    assert ws.status() == 0
+    h = w.num_kv_heads
+    for b, t in enumerate(w.seq_lens):
+        a, c = fin_r[b * h:(b + 1) * h, :t], fin_t[b * h:(b + 1) * h, :t]
+        m = torch.isfinite(c)
+        assert float((a[m] - c[m]).abs().max()) <= 5e-6 * float(c[m].abs().max()), (kv_dtype, head_dim, b)
+
+
 @pytest.mark.parametrize("kernel", ["mfma", "valu"])
 def test_resident_selection_on_dense_keys(kernel, monkeypatch):
     """[B, H, T, D] keys without a block table (the selector's keys_dense call shape) through
