@@ -166,9 +166,10 @@ int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_
 /* tri_score_paged + tri_select in one call, without the raw scores ever being handed to
  * the caller: the device side of _select_keep_indices_for_group_per_head's paged branch
  * (runtime/selector_hf.py:813-1033) and of the per-layer selector (:473-677).  When the
- * shape allows (head_dim 128, at most four query heads per KV head, mean aggregation
- * over offsets, power-of-two block size, layer_reduce >= 0, not shared, every
- * sequence fits the GPU's LDS) one resident kernel keeps each layer's raw scores in LDS
+ * shape allows (head_dim 128, or 64 / 256 with two-byte keys; at most eight query heads
+ * per KV head; mean aggregation over offsets; power-of-two block size; layer_reduce >= 0;
+ * not shared; a batch that fills most of the GPU and whose sequences fit its LDS in
+ * tiles) one resident kernel keeps each layer's raw scores in LDS
  * and they never reach memory; otherwise the two calls above run back to back on the
  * workspace.  Outputs as tri_select; keep may be NULL when only final_scores is wanted
  * (tri_topk_rows then turns them into keep rows). */
@@ -177,7 +178,7 @@ int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_
                      uint64_t workspace_bytes, void* stream);
 
 /* Which path tri_select_paged / tri_compress_step take for these arguments on the
- * current device: 2 = resident kernel scoring on the matrix cores (bf16 and fp8 keys), 1 = resident
+ * current device: 2 = resident kernel scoring on the matrix cores (bf16, fp16 and fp8 keys), 1 = resident
  * kernel scoring on the vector unit, 0 = score then select, -1 = invalid arguments.
  * Host-only.  No counterpart in the reference (it has a single path). */
 int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,

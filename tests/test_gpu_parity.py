@@ -544,6 +544,12 @@ RESIDENT_CASES.update({
     "d64_hkv2": dict(w=small(head_dim=64, seq_lens=(300, 1000, 17))),
     "d64_interleaved_fp16_g7": dict(w=small(head_dim=64, kv_dtype="fp16", rope_style="interleaved", num_q_heads=28,
                                             num_kv_heads=4, seq_lens=(640, 2049))),
+    # head dimension 256
+    "d256_hkv8": dict(w=small(head_dim=256, num_q_heads=16, num_kv_heads=8, seq_lens=(700, 90, 1500), num_layers=3)),
+    "d256_g8_fp16_interleaved": dict(w=small(head_dim=256, kv_dtype="fp16", rope_style="interleaved", num_q_heads=16,
+                                             num_kv_heads=2, seq_lens=(640, 2049))),
+    "d256_ragged_small_chip": dict(w=small(head_dim=256, num_q_heads=8, num_kv_heads=8,
+                                           seq_lens=(3000, 70, 4100, 900, 1), budget=128, num_layers=2), workgroups=24),
     "d64_tile_refined": dict(w=small(head_dim=64, num_q_heads=32, num_kv_heads=8, seq_lens=(3072,) * 16, budget=256,
                                      num_layers=2)),
 })
@@ -562,7 +568,7 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
         pytest.skip("the matrix-core kernel needs blocks of at least 16 tokens (a step lies inside one block)")
     if kernel == "valu" and w.num_q_heads // w.num_kv_heads > 4:
         pytest.skip("the vector-unit kernel holds four query heads per KV head")
-    if kernel == "valu" and w.head_dim != 128:
+    if kernel == "valu" and w.head_dim != 128:      # (64 and 256 exist on the matrix cores only)
         pytest.skip("the vector-unit kernel is built for a head dimension of 128")
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)      # take that kernel however small the launch
     if "workgroups" in case:
@@ -596,7 +602,7 @@ def _random_resident_case(seed: int):
     import random
     r = random.Random(seed)
     kv_dtype = r.choice(["bf16", "bf16", "fp16", "fp8"])
-    head_dim = 128 if kv_dtype == "fp8" else r.choice([128, 128, 64])
+    head_dim = 128 if kv_dtype == "fp8" else r.choice([128, 128, 64, 256])
     hkv = r.choice([1, 2, 3, 4, 5, 8, 8, 12])
     g = r.choice([1, 2, 3, 4, 4, 6, 7, 8])
     nseq = r.choice([1, 2, 3, 5, 9])
@@ -627,7 +633,8 @@ def test_matrix_core_kernel_on_random_shapes(seed, monkeypatch):
         del RESIDENT_CASES[f"random{seed}"]
 
 
-@pytest.mark.parametrize("kv_dtype,head_dim", [("bf16", 128), ("fp16", 128), ("fp8", 128), ("bf16", 64), ("fp16", 64)])
+@pytest.mark.parametrize("kv_dtype,head_dim", [("bf16", 128), ("fp16", 128), ("fp8", 128), ("bf16", 64), ("fp16", 64),
+                                               ("bf16", 256), ("fp16", 256)])
 def test_matrix_core_scores_carry_every_piece(kv_dtype, head_dim, monkeypatch):
     """Without normalisation and with a layer maximum the raw scores show through: the
     matrix-core kernel (coefficients in three pieces, magnitudes in two) agrees with the
@@ -835,7 +842,7 @@ def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
 
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
-    for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=256), {}), (dict(head_dim=64, kv_dtype="fp8"), {}),
+    for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=256, kv_dtype="fp8"), {}), (dict(head_dim=64, kv_dtype="fp8"), {}),
                       (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
         w = small(**kw)
         inp = build_inputs(w)

@@ -232,6 +232,15 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.fin = fin ? fin : at<float>(ws, w.fin);
   a.plan = w.fused;
   a.bmat = at<char>(ws, w.bmat);
+  if (w.fused.eligible == 2) {
+    // The preparation launch writes one 16-byte entry per (sequence, layer, KV head, group of four
+    // query heads, slab, lane); the region planned for them must hold that.
+    const int64_t groups = a.G > 4 ? 2 : 1, slabs = a.D / 32 + a.D / 64;
+    const int64_t need = (int64_t)a.B * a.L * a.Hkv * groups * slabs * 64 * 16;
+    if (need > w.total - w.bmat)
+      return fail(TRI_ERR_WORKSPACE, "coefficient slabs need %lld bytes, %lld planned", (long long)need,
+                  (long long)(w.total - w.bmat));
+  }
   {
     // Two resident launches that run at the same time on one device would each hold part of
     // the CUs and wait for the other's workgroups until their waits expire.  Launches of this

@@ -54,7 +54,7 @@ struct Workspace {
   int64_t xchg;      // [B][L][tiles_per_seq][A][2] tagged sums exchanged by the resident kernel
   int64_t status;    // one word: non-zero when a bounded wait of the resident kernel expired
   int64_t pack;      // [2][B] int32: launch of every sequence and its first workgroup there (several launches)
-  int64_t bmat;      // [B][L][Hkv][groups of 4 query heads][6][64][8] bf16 coefficient slabs (matrix-core kernel)
+  int64_t bmat;      // [B][L][Hkv][groups of 4 query heads][slabs][64][8] bf16 coefficient slabs (matrix-core kernel)
   int64_t total;
   int32_t num_tiles; // NT
   FusedPlan fused;
@@ -75,7 +75,9 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
   w.status = take(256);
   w.pack = take(fused.eligible ? (int64_t)B * 8 : 0);
-  w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * (A / Hkv > 4 ? 2 : 1) * 6 * 64 * 16 : 0);
+  // key slabs (head_dim / 32) and magnitude slabs (half as many) per group of four query heads
+  const int slabs = max(F / 16 + F / 32, 6);
+  w.bmat = take(fused.eligible == 2 ? (int64_t)B * L * Hkv * (A / Hkv > 4 ? 2 : 1) * slabs * 64 * 16 : 0);
   w.total = off;
   return w;
 }

@@ -163,8 +163,11 @@ __device__ __forceinline__ float coefficient_piece(float x, int pieces) {
 // j / 4); element e = k index kb*8 + e of the slab.  Piece `split` of a coefficient x is
 // what is left of x after `split` roundings to bf16 (x = x1 + x2 + x3).
 constexpr int kPrepThreads = 1024;
-constexpr int kPrepHeads = 64;      // query heads whose coefficients are staged at a time
-constexpr int kPrepPitch = 193;
+// Query heads whose coefficients are staged at a time, and the pitch of a staged head
+// [P | R | E][F] in floats (odd: the four query heads and four k blocks a wave reads at once
+// then fall into 16 different banks).
+template <int HD> constexpr int prep_heads() { return HD > 128 ? 32 : 64; }
+template <int HD> constexpr int prep_pitch() { return 3 * (HD / 2) + 1; }
 
 template <int DT, bool IL, int HD>
 __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* folded, const float* omega,
@@ -174,28 +177,28 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
                                                                  unsigned long long* xchg, int64_t words,
                                                                  uint32_t* status) {
   // One buffer, used twice: the per-offset cos / sin values, then the coefficients of up to
-  // kPrepHeads query heads as [head][P | R | E][64] with a row pitch of 193 floats (the four
-  // query heads and four k blocks a wave reads at once then fall into 16 different banks).
+  // kPrepHeads query heads as [head][P | R | E][F] with a row pitch of 3F + 1 floats.
   constexpr int F = HD / 2;              // frequency pairs
   constexpr int NS = HD / 32;            // key slabs (MFMAs) per step
   constexpr int NSO = NS + NS / 2;       // operands per query-head group: key slabs, magnitude slabs
+  constexpr int kPrepHeads = prep_heads<HD>(), kPrepPitch = prep_pitch<HD>();
   __shared__ float buf[kPrepHeads * kPrepPitch];
-  __shared__ float mean_cs[2][64];
-  static_assert(kPrepHeads * kPrepPitch >= 2 * kMaxOffsets * 64, "the trig values must fit the buffer");
-  float (*part)[kMaxOffsets][64] = reinterpret_cast<float (*)[kMaxOffsets][64]>(buf);
+  __shared__ float mean_cs[2][F];
+  static_assert(kPrepHeads * kPrepPitch >= 2 * kMaxOffsets * F, "the trig values must fit the buffer");
+  float (*part)[kMaxOffsets][F] = reinterpret_cast<float (*)[kMaxOffsets][F]>(buf);
   const int l = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int64_t wg = (int64_t)b * gridDim.x + l, nwg = (int64_t)gridDim.x * gridDim.y;
   for (int64_t i = wg * kPrepThreads + tid; i < words; i += nwg * kPrepThreads) xchg[i] = 0ull;
   if (wg == 0 && tid == 0) *status = 0u;
 
   const float rs = (float)round_start[b];
-  for (int i = tid; i < NO * 64; i += kPrepThreads) {
-    const int j = i >> 6, f = i & 63;
-    if (f < F) phase_cos_sin(__fmul_rn(__fadd_rn(rs, offsets[j]), omega[f]), part[0][j][f], part[1][j][f]);
+  for (int i = tid; i < NO * F; i += kPrepThreads) {
+    const int j = i / F, f = i % F;
+    phase_cos_sin(__fmul_rn(__fadd_rn(rs, offsets[j]), omega[f]), part[0][j][f], part[1][j][f]);
   }
   __syncthreads();
-  if (tid < 128 && (tid & 63) < F) {
-    const int which = tid >> 6, f = tid & 63;
+  if (tid < 2 * F) {
+    const int which = tid / F, f = tid % F;
     double sum = 0.0;
     for (int j = 0; j < NO; ++j) sum += part[which][j][f];
     mean_cs[which][f] = (float)(sum / NO);
@@ -276,7 +279,7 @@ __device__ __forceinline__ int nsteps_of(int ntok) { return (ntok + 15) >> 4; }
 template <int DT, bool IL, int TW, int SL, int QG, int NB, int W, int HD>
 __global__ __launch_bounds__(W * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
-  static_assert(HD == 128 || (HD == 64 && DT != TRI_KV_FP8_E4M3), "head dimensions with a kernel");
+  static_assert(HD == 128 || ((HD == 64 || HD == 256) && DT != TRI_KV_FP8_E4M3), "head dimensions with a kernel");
   constexpr int NS = HD / 32;            // key slabs (MFMAs) per step
   constexpr int NSO = NS + NS / 2;       // operands per query-head group
   static_assert(SL % (16 * NB) == 0, "the slack must hold whole rotations of the step buffers");
@@ -774,6 +777,20 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, const LaunchShape& sha
 template <int DT, bool IL>
 hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int head_dim, const LaunchShape& shape,
                           hipStream_t s) {
+  if (head_dim == 256) {
+    // Twice the bytes per row: two step buffers hold as many bytes as four do for 128.
+    if constexpr (DT != TRI_KV_FP8_E4M3) {
+      if (k.G > 4) {
+        if (tw != 512) return hipErrorInvalidValue;
+        return waves == 4 ? launch_mfma_t<DT, IL, 512, 64, 2, 2, 4, 256>(k, bmat, shape, s)
+                          : launch_mfma_t<DT, IL, 512, 64, 2, 2, 8, 256>(k, bmat, shape, s);
+      }
+      if (tw != 1024) return hipErrorInvalidValue;
+      return waves == 4 ? launch_mfma_t<DT, IL, 1024, 128, 1, 2, 4, 256>(k, bmat, shape, s)
+                        : launch_mfma_t<DT, IL, 1024, 192, 1, 2, 8, 256>(k, bmat, shape, s);
+    }
+    return hipErrorInvalidValue;
+  }
   if (head_dim == 64) {
     // Half the bytes per row: eight step buffers keep as many bytes in flight (four query heads
     // per KV head; with eight the LDS has no room for the slack that eight buffers need).  One
@@ -855,7 +872,7 @@ int host_pack_launches(const int32_t* lens, int B, int tile, int wg_mult, int ca
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                           int resident, bool any_fill, int kv_dtype, const int32_t* host_lens) {
   FusedPlan p{};
-  const bool dim_ok = D == 128 || (D == 64 && kv_dtype != TRI_KV_FP8_E4M3);
+  const bool dim_ok = D == 128 || ((D == 64 || D == 256) && kv_dtype != TRI_KV_FP8_E4M3);
   if (resident <= 0 || !dim_ok || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
     return p;
   int bs_shift = -1;
@@ -869,7 +886,7 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   const int tws[3] = {256, 512, 1024};
   const int ntw = G > 4 ? 2 : 3;          // the ring of a 1024-token tile fits LDS for four query heads only
   int tw = tws[ntw - 1];
-  if (waves == kFusedWaves && D == 128)   // (four waves, head dimension 64: one kernel instance, with the largest ring)
+  if (waves == kFusedWaves && D == 128)   // (four waves, head dimensions 64 and 256: one kernel instance, with the largest ring)
     for (int i = 0; i < ntw; ++i)
       if ((int64_t)B * ceil_div(Tmax, tws[i]) * HC <= resident) { tw = tws[i]; break; }
   int tile = tw, tiles = ceil_div(Tmax, tw);
@@ -959,8 +976,8 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   const bool fp8 = a.kv_dtype == TRI_KV_FP8_E4M3;
   const bool fp16 = a.kv_dtype == TRI_KV_FP16;
   if (a.kv_dtype != TRI_KV_BF16 && !fp8 && !fp16) return hipErrorInvalidValue;
-  if (a.NO <= 0 || a.NO > kMaxOffsets || (a.D != 128 && a.D != 64)) return hipErrorInvalidValue;
-  if (a.D == 64 && fp8) return hipErrorInvalidValue;
+  if (a.NO <= 0 || a.NO > kMaxOffsets || (a.D != 128 && a.D != 64 && a.D != 256)) return hipErrorInvalidValue;
+  if (a.D != 128 && fp8) return hipErrorInvalidValue;
   auto prep_launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)a.L, (unsigned)a.B), dim3(kPrepThreads), 0, s, a.folded, a.omega,
                        a.offsets, a.NO, a.round_start, a.L, a.Hkv, a.G, a.A, QG, bmat, a.xchg, words, a.status);
@@ -972,6 +989,9 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
     if (a.D == 64) {
       if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true, 64>);
       else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false, 64>);
+    } else if (a.D == 256) {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true, 256>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false, 256>);
     } else {
       if (il) prep_launch(prep_mfma_kernel<TRI_KV_FP16, true, 128>);
       else prep_launch(prep_mfma_kernel<TRI_KV_FP16, false, 128>);
@@ -980,6 +1000,9 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
     if (a.D == 64) {
       if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true, 64>);
       else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false, 64>);
+    } else if (a.D == 256) {
+      if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true, 256>);
+      else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false, 256>);
     } else {
       if (il) prep_launch(prep_mfma_kernel<TRI_KV_BF16, true, 128>);
       else prep_launch(prep_mfma_kernel<TRI_KV_BF16, false, 128>);
