@@ -186,7 +186,7 @@ def test_group_selection_matches_oracle_on_random_shapes(seed):
     r = random.Random(2000 + seed)
     hkv, g = r.choice([1, 2, 3, 4, 8]), r.choice([1, 2, 4, 7, 8])
     seq_lens = tuple(r.choice([1, 17, 64, 97, 130, 300, 513, 700]) for _ in range(r.choice([1, 2, 3])))
-    w = small(kv_dtype=r.choice(["bf16", "bf16", "fp16", "fp8"]), head_dim=r.choice([64, 128, 128]),
+    w = small(kv_dtype=r.choice(["bf16", "bf16", "fp16", "fp8"]), head_dim=r.choice([64, 128, 128, 256]),
               num_q_heads=hkv * g, num_kv_heads=hkv, seq_lens=seq_lens, num_layers=r.choice([1, 2, 3]),
               budget=r.choice([16, 96, 200]), block_size=r.choice([8, 16, 32]), window_size=r.choice([0, 12, 40]),
               rope_style=r.choice(["half", "interleaved"]), index=300 + seed)
