@@ -55,6 +55,15 @@ SCORE_CASES = {
     "llama3": dict(w=small(rope_theta=5e5, rope_scaling="llama3")),
     "max_agg": dict(w=small(seq_lens=(300, 40)), aggregation="max"),
     "max_agg_d64": dict(w=small(head_dim=64, seq_lens=(100,)), aggregation="max"),
+    # max aggregation on the matrix cores (bf16 keys, head dimension 128)
+    "max_agg_interleaved_ragged": dict(w=small(rope_style="interleaved", seq_lens=(1300, 17, 513, 1), num_layers=3),
+                                       aggregation="max"),
+    "max_agg_g8": dict(w=small(num_q_heads=16, num_kv_heads=2, seq_lens=(700, 90)), aggregation="max"),
+    "max_agg_hkv4_g7": dict(w=small(num_q_heads=28, num_kv_heads=4, seq_lens=(333,)), aggregation="max"),
+    "max_agg_g1_hkv3": dict(w=small(num_q_heads=3, num_kv_heads=3, seq_lens=(129, 600)), aggregation="max"),
+    "max_agg_block_not_pow2": dict(w=small(block_size=24, seq_lens=(301, 1025)), aggregation="max"),
+    "max_agg_kv_axis1_block32": dict(w=small(block_size=32, seq_lens=(290, 64)), kv_axis=1, aggregation="max"),
+    "max_agg_fp16": dict(w=small(kv_dtype="fp16", seq_lens=(200,)), aggregation="max"),
     "no_mlr": dict(w=small(), disable_mlr=True),
     "no_trig": dict(w=small(), disable_trig=True),
     "no_trig_max": dict(w=small(), disable_trig=True, aggregation="max"),
@@ -89,6 +98,39 @@ def test_raw_scores_match_oracle(name):
             err = (got - want[l]).abs()
             tol = score_tolerance(want[l])                        # 1e-3 relative to per-head RMS
             assert bool((err <= tol).all()), (name, b, l, float(err.max()), float(tol.min()))
+
+
+@pytest.mark.parametrize("name", ["max_agg", "max_agg_interleaved_ragged", "max_agg_g8", "max_agg_hkv4_g7",
+                                  "max_agg_block_not_pow2"])
+def test_max_aggregation_on_matrix_cores_matches_the_vector_unit_kernel(name, monkeypatch):
+    """Keys are exact in bf16 and the coefficients enter in three bf16 pieces, so the matrix-core
+    kernel agrees with the vector-unit kernel to fp32 rounding (1e-5 of the per-head RMS, a
+    hundred times tighter than the bound against the oracle); the per-tile sums behind the
+    statistics are compared through the selection scores."""
+    case = dict(SCORE_CASES[name])
+    w = case.pop("w")
+    kv_axis = case.pop("kv_axis", 0)
+    inp = build_inputs(w, kv_axis)
+    print(f"case={name} workload={w}", flush=True)
+    out = {}
+    for kernel in ("mfma", "valu"):
+        monkeypatch.setenv("TRIATTN_MAX_KERNEL", kernel)
+        caches, kv, batch, sc = device_objects(w, inp, DEV, aggregation="max")
+        raw, ws = ops.score_paged(kv, batch, sc)
+        sel = ops.SelectConfig(window_size=w.window_size)
+        keep, fin = ops.select(kv, batch, sc, sel, raw, ws, want_scores=True)
+        torch.cuda.synchronize()
+        out[kernel] = (raw.clone(), fin.clone())
+    h = w.num_kv_heads
+    for b, t in enumerate(w.seq_lens):
+        got, want = out["mfma"][0][b, :, :t], out["valu"][0][b, :, :t]          # [L, T, A]
+        rms = want.pow(2).mean(dim=1, keepdim=True).sqrt().clamp_min(1e-30)
+        assert float(((got - want).abs() / rms).max()) <= 1e-5, (name, b)
+        fm, fv = out["mfma"][1][b * h:(b + 1) * h, :t], out["valu"][1][b * h:(b + 1) * h, :t]
+        finite = torch.isfinite(fv)
+        assert torch.equal(torch.isfinite(fm), finite)
+        if bool(finite.any()):
+            assert float((fm[finite] - fv[finite]).abs().max()) <= 5e-4 * float(fv[finite].abs().max()), (name, b)
 
 
 def test_head_major_output_layout():

@@ -21,6 +21,8 @@
 // store two different tokens with a single instruction.
 #include "tri_common.h"
 #include "tri_score_device.h"
+#include <cstdlib>
+#include <cstring>
 
 namespace tri {
 namespace {
@@ -495,6 +497,316 @@ __global__ __launch_bounds__(kScoreThreads) void score_max_kernel(ScoreArgs a) {
   }
 }
 
+// ------------------------------------------------------- max, matrix cores
+// The same scores as score_max_kernel for two-byte bf16 keys with a head dimension of 128, as
+// a matrix product: per offset j the sum over the pairs is linear in the key,
+//   raw_j = sum_f kr_f (A1_f cos_jf - A2_f sin_jf) + ki_f (A2_f cos_jf + A1_f sin_jf),
+// so 16 tokens x 128 key elements times 128 x (query heads x offsets) coefficients gives every
+// per-offset sum of a step (v_mfma_f32_16x16x32_bf16; the keys are exact in bf16, a
+// coefficient enters as three bf16 pieces accumulated into the same column).  Column tile q
+// (of four) holds offsets 0..15 of the workgroup's query head q, so the maximum over them is
+// a maximum over the 16 lanes of a row group; offsets from 16 on sit in NX further tiles as
+// column 4 (j - 16) + q, four lanes apart per head.  The magnitude term goes through the
+// matrix cores too: |k_f| in two bf16 pieces times E in three pieces, one piece per column
+// group.  A workgroup builds its operand slabs in LDS from the per-sequence tables (60 KB
+// for 17 offsets), then each wave takes 16 tokens a step.  Outputs as score_max_kernel: raw
+// rows and per-tile sums.
+typedef __bf16 mx_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float mx_f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kDppRowMirror = 0x140;   // row_mirror
+constexpr int kDppRor4 = 0x124;        // row_ror:4
+
+__device__ __forceinline__ mx_f32x4 mx_mfma(const uint4& a, const uint4& b, mx_f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mx_bf16x8, a), __builtin_bit_cast(mx_bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ uint32_t bf16_bits(float x) {
+  return (uint32_t)__builtin_bit_cast(unsigned short, (__bf16)x);
+}
+// x = p[0] + p[1] + p[2] up to 24 bits: each piece is what bf16 holds of the remainder.
+__device__ __forceinline__ void bf16_pieces(float x, uint32_t (&p)[3]) {
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    p[i] = bf16_bits(x);
+    x -= __uint_as_float(p[i] << 16);
+  }
+}
+__device__ __forceinline__ float bf16_elem(const uint4& v, int e) {   // e: compile-time
+  const uint32_t w = e < 2 ? v.x : e < 4 ? v.y : e < 6 ? v.z : v.w;
+  return (e & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+}
+
+constexpr int kMaxMfmaHeads = 4;   // query heads of one KV head per workgroup
+constexpr int kTrigPitch = 65;     // floats per offset in LDS (odd: 16 offsets read at once fall into 16 banks)
+__host__ __device__ constexpr size_t max_mfma_lds_bytes(int nx, int no) {
+  return (size_t)(kMaxMfmaHeads + nx) * 12 * 64 * 16 + 2 * 64 * 16 + 3 * kMaxMfmaHeads * 64 * 4 +
+         (size_t)2 * no * kTrigPitch * 4 + (kScoreTileTokens + 2) * 4 + 4 * kMaxMfmaHeads * 2 * 4;
+}
+
+template <int NX, bool IL>
+__global__ __launch_bounds__(kScoreThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void score_max_mfma_kernel(ScoreArgs a) {
+  constexpr int F = 64;
+  constexpr int NT = kMaxMfmaHeads + NX;
+  extern __shared__ __align__(16) char max_mfma_lds[];
+  uint4* Bk = reinterpret_cast<uint4*>(max_mfma_lds);          // [NT][4 key slabs][3 pieces][64 lanes]
+  uint4* Bm = Bk + NT * 12 * 64;                               // [2 magnitude slabs][64 lanes]
+  float* cf = reinterpret_cast<float*>(Bm + 2 * 64);           // [A1 | A2 | E][4 query heads][F]
+  float* tcos = cf + 3 * kMaxMfmaHeads * F;                    // [NO][kTrigPitch]
+  float* tsin = tcos + a.NO * kTrigPitch;                      // [NO][kTrigPitch]
+  int* lds_blk = reinterpret_cast<int*>(tsin + a.NO * kTrigPitch);   // [kScoreTileTokens + 2]
+  float* red = reinterpret_cast<float*>(lds_blk + kScoreTileTokens + 2);   // [4 waves][4 heads][2]
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x;
+  const int head = blockIdx.y / a.QC, qc = blockIdx.y % a.QC;
+  const int q0 = qc * kMaxMfmaHeads, nq = min(kMaxMfmaHeads, a.G - q0);
+  const int b = blockIdx.z / a.L, l = blockIdx.z % a.L;
+  const int seq_len = a.seq_lens[b];
+  const int n0 = tile * kScoreTileTokens;
+  if (n0 >= seq_len) return;
+  const int n1 = min(n0 + kScoreTileTokens, seq_len);
+
+  int lb0 = 0;
+  if (a.block_table_pitch >= 0) {
+    lb0 = n0 / a.block_size;
+    const int lb1 = (n1 - 1) / a.block_size;
+    for (int i = threadIdx.x; i <= lb1 - lb0; i += kScoreThreads)
+      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
+  }
+  for (int i = threadIdx.x; i < 3 * kMaxMfmaHeads * F; i += kScoreThreads) {
+    const int which = i / (kMaxMfmaHeads * F), q = (i / F) % kMaxMfmaHeads, f = i % F;
+    const int ah = head * a.G + q0 + min(q, nq - 1);
+    cf[i] = q < nq ? a.coef[(((int64_t)(b * a.L + l) * a.A + ah) * 3 + which) * F + f] : 0.f;
+  }
+  for (int i = threadIdx.x; i < a.NO * F; i += kScoreThreads) {
+    const int j = i / F, f = i % F;
+    tcos[j * kTrigPitch + f] = a.trig[((int64_t)(b * a.NO + j) * 2 + 0) * F + f];
+    tsin[j * kTrigPitch + f] = a.trig[((int64_t)(b * a.NO + j) * 2 + 1) * F + f];
+  }
+  __syncthreads();
+
+  // Operand slabs.  Lane (c16 = lane % 16, kb = lane / 16) of slab (t, s) holds one column
+  // and key elements 32 s + 8 kb + 0..7; the column is (head t, offset c16) in the first
+  // four tiles and (head c16 % 4, offset 16 + 4 (t - 4) + c16 / 4) in the others.
+  for (int i = threadIdx.x; i < NT * 4 * 64; i += kScoreThreads) {
+    const int ln = i & 63, sl = (i >> 6) & 3, t = i >> 8;
+    const int c16 = ln & 15, kb = ln >> 4;
+    const int q = t < kMaxMfmaHeads ? t : (c16 & 3);
+    const int j = t < kMaxMfmaHeads ? c16 : 16 + 4 * (t - kMaxMfmaHeads) + (c16 >> 2);
+    const bool live = q < nq && j < a.NO;
+    const int jc = live ? j : 0;
+    uint32_t w[3][4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = 32 * sl + 8 * kb + e;
+      const int f = IL ? (d >> 1) : (d & 63);
+      const bool im = IL ? (d & 1) != 0 : d >= 64;
+      const float a1 = cf[(0 * kMaxMfmaHeads + q) * F + f], a2 = cf[(1 * kMaxMfmaHeads + q) * F + f];
+      const float cs = tcos[jc * kTrigPitch + f], sn = tsin[jc * kTrigPitch + f];
+      float x = im ? fmaf(a2, cs, a1 * sn) : fmaf(a1, cs, -(a2 * sn));
+      if (!live) x = 0.f;
+      uint32_t pc[3];
+      bf16_pieces(x, pc);
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        if (e & 1) w[p][e >> 1] |= pc[p] << 16;
+        else w[p][e >> 1] = pc[p];
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < 3; ++p) Bk[((t * 4 + sl) * 3 + p) * 64 + ln] = uint4{w[p][0], w[p][1], w[p][2], w[p][3]};
+  }
+  // Magnitude slabs: column c16 = query head (c16 % 4), piece (c16 / 4) of E; element e of slab
+  // m is the pair whose magnitude the same lane forms from its key registers below.
+  for (int i = threadIdx.x; i < 2 * 64; i += kScoreThreads) {
+    const int ln = i & 63, m = i >> 6;
+    const int c16 = ln & 15, kb = ln >> 4;
+    const int q = c16 & 3, piece = c16 >> 2;
+    const bool live = piece < 3 && q < nq;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int f = IL ? 16 * (2 * m + (e >> 2)) + 4 * kb + (e & 3) : 32 * m + 8 * kb + e;
+      uint32_t pc[3];
+      bf16_pieces(live ? cf[(2 * kMaxMfmaHeads + q) * F + f] : 0.f, pc);
+      const uint32_t v = piece == 0 ? pc[0] : piece == 1 ? pc[1] : pc[2];
+      if (e & 1) w[e >> 1] |= v << 16;
+      else w[e >> 1] = v;
+    }
+    Bm[m * 64 + ln] = uint4{w[0], w[1], w[2], w[3]};
+  }
+  __syncthreads();
+
+  const int r16 = lane & 15, kb = lane >> 4;
+  const bool main_col = r16 < a.NO;             // this lane's column of the first four tiles is an offset
+  bool extra_col[NX > 0 ? NX : 1];              // ... and of the further tiles
+#pragma unroll
+  for (int x = 0; x < NX; ++x) extra_col[x] = 16 + 4 * x + (r16 >> 2) < a.NO;
+  const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
+  const int64_t lane_off = (int64_t)head * a.stride_head + 8 * kb;
+  constexpr int TW = kScoreTileTokens / 4;
+  const int wstart = n0 + wave * TW;
+  const int wend = min(wstart + TW, n1);
+  const bool out_lane = r16 < nq;
+  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer +
+                   (int64_t)(head * a.G + q0 + (out_lane ? r16 : 0)) * a.raw_stride_head;
+  float s1 = 0.f, s2 = 0.f;
+
+  // Row lane % 16 of the step that starts at token t0: four 16-byte pieces, one per key slab.
+  // Rows past the tile are clamped to its last token (loaded, never stored).
+  auto load_step = [&](int t0, uint4 (&A)[4]) __attribute__((always_inline)) {
+    const int t = min(t0 + r16, n1 - 1);
+    int64_t phys, in_off;
+    if (a.block_table_pitch < 0) {
+      phys = b; in_off = t;
+    } else {
+      const int lb = a.bs_shift >= 0 ? (t >> a.bs_shift) : (t / a.block_size);
+      phys = lds_blk[lb - lb0];
+      in_off = t - lb * a.block_size;
+    }
+    const int64_t e = phys * a.stride_block + in_off * a.stride_token + lane_off;
+    GlobalBytes p = (GlobalBytes)(uintptr_t)kbase + e * 2;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const u32x4 v = *(GlobalU4)(p + sl * 64);
+      A[sl] = uint4{v.x, v.y, v.z, v.w};
+    }
+  };
+
+  // The keys of the next two steps are in flight while a step is worked on.
+  uint4 A[4] = {}, An[4] = {}, Ann[4] = {};
+  if (wstart < wend) load_step(wstart, A);
+  if (wstart + 16 < wend) load_step(wstart + 16, An);
+  for (int t0 = wstart; t0 < wend; t0 += 16) {
+    if (t0 + 32 < wend) load_step(t0 + 32, Ann);
+
+    mx_f32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      acc[t] = mx_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl)
+#pragma unroll
+        for (int p = 2; p >= 0; --p) acc[t] = mx_mfma(A[sl], Bk[((t * 4 + sl) * 3 + p) * 64 + lane], acc[t]);
+      // One tile's operands at a time: left to itself the scheduler requests the slabs of all
+      // tiles up front and spills the keys to make room for them.
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Magnitudes of this lane's 16 pairs as two bf16 pieces each.
+    mx_f32x4 accm = mx_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      uint32_t hi[4], lo[4];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float kr, ki;
+        if (IL) {
+          kr = bf16_elem(A[2 * m + (e >> 2)], 2 * (e & 3));
+          ki = bf16_elem(A[2 * m + (e >> 2)], 2 * (e & 3) + 1);
+        } else {
+          kr = bf16_elem(A[m], e);
+          ki = bf16_elem(A[m + 2], e);
+        }
+        const float mag = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
+        const uint32_t h = bf16_bits(mag);
+        const uint32_t lw = bf16_bits(mag - __uint_as_float(h << 16));
+        if (e & 1) { hi[e >> 1] |= h << 16; lo[e >> 1] |= lw << 16; }
+        else { hi[e >> 1] = h; lo[e >> 1] = lw; }
+      }
+      const uint4 bm = Bm[m * 64 + lane];
+      accm = mx_mfma(uint4{lo[0], lo[1], lo[2], lo[3]}, bm, accm);
+      accm = mx_mfma(uint4{hi[0], hi[1], hi[2], hi[3]}, bm, accm);
+    }
+
+    // Offsets from 16 on: the maximum over this lane's columns of the further tiles, then over
+    // the four lanes of the same query head (lane % 4).
+    float far[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if constexpr (NX > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = -INFINITY;
+#pragma unroll
+        for (int x = 0; x < NX; ++x) v = extra_col[x] ? fmaxf(v, acc[kMaxMfmaHeads + x][i]) : v;
+        v = fmaxf(v, dpp<kDppRor4>(v));
+        v = fmaxf(v, dpp<kDppRor8>(v));
+        far[i] = v;
+      }
+    }
+    // Offsets 0..15 of head q: the 16 lanes of the row group; lane q keeps the result.
+    float val[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < kMaxMfmaHeads; ++q) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = main_col ? acc[q][i] : -INFINITY;
+        v = fmaxf(v, dpp<kDppXor1>(v));
+        v = fmaxf(v, dpp<kDppXor2>(v));
+        v = fmaxf(v, dpp<kDppHalfMirror>(v));
+        v = fmaxf(v, dpp<kDppRowMirror>(v));
+        if (r16 == q) val[i] = v;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float ex = accm[i] + __shfl_down(accm[i], 4, 16) + __shfl_down(accm[i], 8, 16);
+      const int tk = t0 + 4 * kb + i;
+      if (out_lane && tk < wend) {
+        const float v = fmaxf(val[i], far[i]) + ex;
+        raw_row[(int64_t)tk * a.raw_stride_token] = v;
+        s1 += v;
+        s2 = fmaf(v, v, s2);
+      }
+    }
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) { A[sl] = An[sl]; An[sl] = Ann[sl]; }
+  }
+
+  // Per-tile sums of every query head: over the four row groups of a wave, then the waves.
+  s1 += __shfl_xor(s1, 16); s1 += __shfl_xor(s1, 32);
+  s2 += __shfl_xor(s2, 16); s2 += __shfl_xor(s2, 32);
+  if (lane < kMaxMfmaHeads) {
+    red[(wave * kMaxMfmaHeads + lane) * 2 + 0] = s1;
+    red[(wave * kMaxMfmaHeads + lane) * 2 + 1] = s2;
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < nq) {
+    float t1 = 0.f, t2 = 0.f;
+    for (int w = 0; w < 4; ++w) {
+      t1 += red[(w * kMaxMfmaHeads + threadIdx.x) * 2 + 0];
+      t2 += red[(w * kMaxMfmaHeads + threadIdx.x) * 2 + 1];
+    }
+    float* out = a.partial + (((int64_t)(b * a.L + l) * a.num_tiles + tile) * a.A + head * a.G + q0 + threadIdx.x) * 2;
+    out[0] = t1;
+    out[1] = t2;
+  }
+}
+
+template <int NX>
+hipError_t launch_max_mfma_nx(const ScoreArgs& k, dim3 grid, int il, size_t lds, hipStream_t s) {
+  const void* fn = il ? reinterpret_cast<const void*>(&score_max_mfma_kernel<NX, true>)
+                      : reinterpret_cast<const void*>(&score_max_mfma_kernel<NX, false>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  if (il) hipLaunchKernelGGL((score_max_mfma_kernel<NX, true>), grid, dim3(kScoreThreads), lds, s, k);
+  else hipLaunchKernelGGL((score_max_mfma_kernel<NX, false>), grid, dim3(kScoreThreads), lds, s, k);
+  return hipGetLastError();
+}
+
+hipError_t launch_max_mfma(const ScoreArgs& k, int B, int il, hipStream_t s) {
+  const int nx = k.NO > 16 ? ceil_div(k.NO - 16, 4) : 0;
+  const size_t lds = max_mfma_lds_bytes(nx, k.NO);
+  dim3 grid(k.num_tiles, k.Hkv * k.QC, B * k.L);
+  switch (nx) {
+    case 0: return launch_max_mfma_nx<0>(k, grid, il, lds, s);
+    case 1: return launch_max_mfma_nx<1>(k, grid, il, lds, s);
+    case 2: return launch_max_mfma_nx<2>(k, grid, il, lds, s);
+    case 3: return launch_max_mfma_nx<3>(k, grid, il, lds, s);
+    case 4: return launch_max_mfma_nx<4>(k, grid, il, lds, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 // -------------------------------------------------------------- prologues
 __global__ void fold_stats_kernel(const float* qr, const float* qi, const float* qabs, const float* fs,
                                   int n_heads_total, int F, int disable_mlr, int disable_trig,
@@ -610,6 +922,12 @@ hipError_t launch_prepare(const float* folded, const float* omega, const float* 
   return hipGetLastError();
 }
 
+// TRIATTN_MAX_KERNEL=valu keeps max aggregation on the vector-unit kernel (comparison runs).
+static bool max_on_vector_unit() {
+  const char* v = std::getenv("TRIATTN_MAX_KERNEL");
+  return v && std::strcmp(v, "valu") == 0;
+}
+
 hipError_t launch_score(const ScoreLaunch& a, hipStream_t s) {
   ScoreArgs k{};
   k.k_layers = a.k_layers;
@@ -637,6 +955,10 @@ hipError_t launch_score(const ScoreLaunch& a, hipStream_t s) {
   int hpad = 1;
   while (hpad < a.Hkv) hpad <<= 1;
   k.Hpad = hpad;
+  const int il_max = a.rope_style == TRI_ROPE_INTERLEAVED;
+  if (a.aggregation == TRI_REDUCE_MAX && a.kv_dtype == TRI_KV_BF16 && a.D == 128 && a.NO <= kMaxOffsets &&
+      !max_on_vector_unit())
+    return launch_max_mfma(k, a.B, il_max, s);
   const int lph = a.D / 16;
   const int upw = kWave / lph;
   const int HC = hpad >= upw ? hpad / upw : 1;
