@@ -333,6 +333,12 @@ def main() -> int:
     score_gbs = algo["score"] / (mean(score_ms) * 1e-3) / 1e9
     compact_gbs = algo["compact"] / (mean(compact_ms) * 1e-3) / 1e9
 
+    if args.aggregation == "mean":
+        two_pass_kernel = "score_mean_kernel"
+    elif w.kv_dtype == "bf16" and w.head_dim == 128 and os.environ.get("TRIATTN_MAX_KERNEL") != "valu":
+        two_pass_kernel = "score_max_mfma_kernel"
+    else:
+        two_pass_kernel = "score_max_kernel"
     out = {
         "metric": "keys scored+compacted/sec & achieved HBM GB/s (% peak), Qwen3-8B 16k ctx",
         "value": keys_per_s,
@@ -362,10 +368,10 @@ def main() -> int:
         "timed_region_wall_s": wall_s,
         "setup_s": setup_s,
         "path": path,
-        "roofline": {"kernel": {"two_pass": "score_mean_kernel", "resident_valu": "fused_select_kernel",
+        "roofline": {"kernel": {"two_pass": two_pass_kernel, "resident_valu": "fused_select_kernel",
                                 "resident_mfma": "fused_mfma_kernel"}[path], "bound": "hbm",
                      "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, path))},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, path)) if args.aggregation == "mean" else None},
     }
     # A plain device-to-device copy of 1 GiB on the same box, for scale: bytes read + bytes
     # written per second (outside every timed region of the step).
