@@ -673,26 +673,8 @@ void score_max_mfma_kernel(ScoreArgs a) {
     }
   };
 
-  // The keys of the next two steps are in flight while a step is worked on.
-  uint4 A[4] = {}, An[4] = {}, Ann[4] = {};
-  if (wstart < wend) load_step(wstart, A);
-  if (wstart + 16 < wend) load_step(wstart + 16, An);
-  for (int t0 = wstart; t0 < wend; t0 += 16) {
-    if (t0 + 32 < wend) load_step(t0 + 32, Ann);
-
-    mx_f32x4 acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      acc[t] = mx_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int sl = 0; sl < 4; ++sl)
-#pragma unroll
-        for (int p = 2; p >= 0; --p) acc[t] = mx_mfma(A[sl], Bk[((t * 4 + sl) * 3 + p) * 64 + lane], acc[t]);
-      // One tile's operands at a time: left to itself the scheduler requests the slabs of all
-      // tiles up front and spills the keys to make room for them.
-      __builtin_amdgcn_sched_barrier(0);
-    }
-
+  // What follows the key products of one 16-token step: magnitude term, maxima, stores.
+  auto finish = [&](const uint4 (&A)[4], mx_f32x4 (&acc)[NT], int t0) __attribute__((always_inline)) {
     // Magnitudes of this lane's 16 pairs as two bf16 pieces each.
     mx_f32x4 accm = mx_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -758,8 +740,39 @@ void score_max_mfma_kernel(ScoreArgs a) {
         s2 = fmaf(v, v, s2);
       }
     }
+  };
+
+  // Two steps (32 tokens) share every read of an operand slab from LDS — those reads, 60 KB a
+  // step, are what the CU runs out of first; the keys of the next two steps are in flight
+  // meanwhile.  (A second step that lies beyond the wave's tokens works on clamped rows and
+  // stores nothing.)
+  uint4 A0[4] = {}, A1[4] = {}, N0[4] = {}, N1[4] = {};
+  if (wstart < wend) { load_step(wstart, A0); load_step(wstart + 16, A1); }
+  for (int t0 = wstart; t0 < wend; t0 += 32) {
+    if (t0 + 32 < wend) { load_step(t0 + 32, N0); load_step(t0 + 48, N1); }
+
+    mx_f32x4 acc0[NT], acc1[NT];
 #pragma unroll
-    for (int sl = 0; sl < 4; ++sl) { A[sl] = An[sl]; An[sl] = Ann[sl]; }
+    for (int t = 0; t < NT; ++t) {
+      acc0[t] = mx_f32x4{0.f, 0.f, 0.f, 0.f};
+      acc1[t] = mx_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl)
+#pragma unroll
+        for (int p = 2; p >= 0; --p) {
+          const uint4 bk = Bk[((t * 4 + sl) * 3 + p) * 64 + lane];
+          acc0[t] = mx_mfma(A0[sl], bk, acc0[t]);
+          acc1[t] = mx_mfma(A1[sl], bk, acc1[t]);
+        }
+      // One tile's operands at a time: left to itself the scheduler requests the slabs of all
+      // tiles up front and spills the keys to make room for them.
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    finish(A0, acc0, t0);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(A1, acc1, t0 + 16);
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) { A0[sl] = N0[sl]; A1[sl] = N1[sl]; }
   }
 
   // Per-tile sums of every query head: over the four row groups of a wave, then the waves.
