@@ -133,6 +133,23 @@ def test_max_aggregation_on_matrix_cores_matches_the_vector_unit_kernel(name, mo
             assert float((fm[finite] - fv[finite]).abs().max()) <= 5e-4 * float(fv[finite].abs().max()), (name, b)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TRIATTN_TEST_RANDOM_SHAPES", "32")) // 2))
+def test_max_aggregation_on_matrix_cores_on_random_shapes(seed, monkeypatch):
+    """Seeded random head layouts, ragged lengths, block sizes, RoPE pairings and cache layouts: the
+    matrix-core max-aggregation scorer against the vector-unit kernel."""
+    import random
+    r = random.Random(5000 + seed)
+    hkv, g = r.choice([1, 2, 3, 4, 8]), r.choice([1, 2, 3, 4, 5, 7, 8])
+    seq_lens = tuple(r.choice([1, 15, 16, 17, 97, 130, 511, 513, 700, 1100]) for _ in range(r.choice([1, 2, 3])))
+    w = small(num_q_heads=hkv * g, num_kv_heads=hkv, seq_lens=seq_lens, num_layers=r.choice([1, 2, 3]),
+              block_size=r.choice([8, 16, 24, 32]), rope_style=r.choice(["half", "interleaved"]), index=500 + seed)
+    SCORE_CASES[f"random_max{seed}"] = dict(w=w, kv_axis=r.choice([0, 1]), aggregation="max")
+    try:
+        test_max_aggregation_on_matrix_cores_matches_the_vector_unit_kernel(f"random_max{seed}", monkeypatch)
+    finally:
+        del SCORE_CASES[f"random_max{seed}"]
+
+
 def test_head_major_output_layout():
     w = small(seq_lens=(200, 77))
     inp = build_inputs(w)
