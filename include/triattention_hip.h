@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 3
+#define TRI_ABI_VERSION 4
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -110,6 +110,9 @@ typedef struct tri_select_params {
                                    runtime, runtime/selector_hf.py:916-989).  1: reduce first, then normalise per
                                    (layer, KV head) with torch mean / unbiased std (SGLang backend,
                                    sglang/scheduler_hooks.py:655-690, core/utils.py:466-480) */
+  int32_t no_resident;          /* 1: never take a resident kernel for this call, whatever the shape and the
+                                   TRIATTN_RESIDENT_KERNEL override say (a caller repeating a step whose resident
+                                   launch raised the status word).  No counterpart in the reference. */
 } tri_select_params;
 
 int tri_abi_version(void);
@@ -128,7 +131,9 @@ int tri_fold_stats(const float* q_mean_real, const float* q_mean_imag, const flo
 uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
                              const tri_score_params* sp);
 
-/* Byte offset inside the workspace of a 32-bit status word: tri_select_paged and
+/* Byte offset inside the workspace of a 32-bit status word (the same for every layout, batch and
+ * score parameters of one library build, so one workspace reused for steps of different shapes
+ * keeps its word in one place): tri_select_paged and
  * tri_compress_step clear it and the resident kernel sets it to non-zero if one of its
  * bounded waits on another workgroup expired (1), or, with fp16 keys or an fp8 cache, if a
  * coefficient does not fit the fp16 pieces the matrix-core kernel holds it in (2)

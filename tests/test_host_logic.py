@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.tri_abi_version() == 3
+    assert lib.tri_abi_version() == 4
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
@@ -48,6 +48,26 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.tri_compact_paged(None, None, None, 0, 0, None) == _lib.TRI_ERR_INVALID_ARGUMENT
     with pytest.raises(_lib.TriError):
         _lib.check(lib.tri_topk_rows(None, 0, 0, None, None, 1, 1, None, 1, None))
+
+
+def test_status_word_sits_at_one_offset_for_every_shape():
+    """A workspace sized for one batch is reused for smaller ones; the status word the kernels
+    write and the word the host reads must be the same for all of them."""
+    import ctypes as C
+    lib = _lib.load()
+    seen = set()
+    for layers, heads, tmax, seqs, score_heads in ((36, 8, 16384, 16, 32), (36, 8, 2176, 1, 32), (4, 2, 300, 3, 8),
+                                                   (64, 8, 32768, 8, 64), (1, 4, 17, 1, 4)):
+        kv = _lib.KvLayout(num_layers=layers, num_kv_heads=heads, head_dim=128, block_size=16, kv_dtype=0,
+                           stride_block=16 * heads * 128, stride_token=heads * 128, stride_head=128, k_layers=8)
+        batch = _lib.Batch(num_seqs=seqs, max_seq_len=tmax, block_table_pitch=4096, block_table=8, seq_lens=8)
+        sp = _lib.ScoreParams(num_score_heads=score_heads, num_offsets=17)
+        total = int(lib.tri_workspace_bytes(C.byref(kv), C.byref(batch), C.byref(sp)))
+        assert total > 0, lib.tri_last_error()
+        off = int(lib.tri_workspace_status_offset(C.byref(kv), C.byref(batch), C.byref(sp)))
+        assert off + 4 <= total
+        seen.add(off)
+    assert len(seen) == 1
 
 
 # ---------------------------------------------------------------- settings
@@ -432,7 +452,7 @@ def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
     """Host logic of ``triattention_apply_compression_batch`` with a stand-in for the kernels:
     requests with something to drop go to one batched call per KV-cache group, the others get
     the one-by-one hook's answers; block lists are truncated per request; a failed resident launch
-    sends every request of the batch through the one-by-one path."""
+    repeats that KV-cache group, and only it, on the kernels that do not wait for each other."""
     calls = {"batch": [], "single": []}
 
     def select_group(*, layer_kv_iter=None, total_tokens, budget_total, **kw):
@@ -440,14 +460,15 @@ def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
         k = min(total_tokens, budget_total)
         return {"mode": "per_head", "indices": torch.arange(k).repeat(2, 1), "semantic": "hf_aligned_global_per_head"}
 
-    def compress_batch(*, layer_kv, block_size, requests):
-        calls["batch"].append([dict(r) for r in requests])
-        if fail["now"]:
+    def compress_batch(*, layer_kv, block_size, requests, allow_resident=True):
+        calls["batch"].append([dict(r, allow_resident=allow_resident, layers=[li for li, _ in layer_kv])
+                               for r in requests])
+        if fail["now"] and allow_resident and (fail["layer"] is None or fail["layer"] in [li for li, _ in layer_kv]):
             raise hook_mod.ResidentLaunchFailed("forced")
         return [{"mode": "per_head", "indices": torch.arange(r["budget_total"]).repeat(2, 1),
                  "semantic": "hf_aligned_global_per_head"} for r in requests]
 
-    fail = {"now": False}
+    fail = {"now": False, "layer": None}
     select_group._supports_paged_group = True
     select_group._compress_batch = compress_batch
     select_layer = lambda **kw: None
@@ -498,17 +519,37 @@ def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
     runner2, reqs2, sig2, sched2 = runner_with([40, 5])
     out2 = RunnerHookCompressionExecutor(runner2).execute_batch(sig2, sched2)
     assert out2["r0"].applied and not calls["batch"] and calls["single"] == [40]
-    # failed resident launch: everything is repeated one by one, with the resident kernel switched off meanwhile
+    # failed resident launch: the group is repeated in one batched call without the resident
+    # kernel; nothing goes through the one-by-one path and the environment is left alone
     calls["batch"].clear(); calls["single"].clear(); moved.clear()
     fail["now"] = True
-    seen_env = []
-    monkeypatch.setattr(hook_mod, "compact_request_kv_in_place_per_head",
-                        lambda **kw: seen_env.append(__import__("os").environ.get("TRIATTN_RESIDENT_KERNEL")) or 8)
     runner3, reqs3, sig3, sched3 = runner_with([40, 30])
     out3 = RunnerHookCompressionExecutor(runner3).execute_batch(sig3, sched3)
-    assert len(calls["batch"]) == 1 and calls["single"] == [40, 30] and seen_env == ["off", "off"]
+    assert [[r["allow_resident"] for r in c] for c in calls["batch"]] == [[True, True], [False, False]]
+    assert not calls["single"] and not moved
     assert all(r.applied and r.cache_len_after == 8 for r in out3.values())
     assert "TRIATTN_RESIDENT_KERNEL" not in __import__("os").environ
+    # two KV-cache groups, the resident launch of the second fails: the first group is not
+    # touched again (one call), the second is repeated alone without the resident kernel
+    calls["batch"].clear()
+    fail["layer"] = 1
+    reqs4 = {f"r{i}": types.SimpleNamespace(num_computed_tokens=t, block_ids=(list(range(100 * i, 100 * i + 10)),
+                                                                           list(range(100 * i + 50, 100 * i + 60))))
+             for i, t in enumerate([40, 30])}
+    runner4 = _Runner(requests=reqs4, kv_caches=[torch.zeros(2, 400, 4, 2, 64), torch.zeros(2, 400, 4, 2, 64)],
+                      cache_config=types.SimpleNamespace(block_size=4))
+    monkeypatch.setattr(hook_mod, "resolve_group_tensors",
+                        lambda base_runner: {0: [(0, base_runner.kv_caches[0])], 1: [(1, base_runner.kv_caches[1])]})
+    install_runner_compression_hook(runner4, cfg)
+    sig4 = {rid: _signal(req_id=rid, estimated_cache_len=q.num_computed_tokens + 1, prefill_len=3)
+            for rid, q in reqs4.items()}
+    sched4 = types.SimpleNamespace(num_scheduled_tokens={rid: 1 for rid in reqs4})
+    out4 = RunnerHookCompressionExecutor(runner4).execute_batch(sig4, sched4)
+    assert [(c[0]["layers"], c[0]["allow_resident"]) for c in calls["batch"]] == [([0], True), ([1], True), ([1], False)]
+    assert all(r.applied and r.cache_len_after == 8 for r in out4.values())
+    assert reqs4["r0"].block_ids == ([0, 1], [50, 51]) and reqs4["r1"].block_ids == ([100, 101], [150, 151])
+    assert not calls["single"]
+    fail["layer"] = None
     # a runner without the batch hook: execute_batch loops over execute
     bare = _Runner(triattention_apply_compression=lambda **kw: {"applied": True, "reason": "x", "cache_len_after": 1})
     res = RunnerHookCompressionExecutor(bare).execute_batch({"a": _signal(req_id="a"), "b": _signal(req_id="b")}, sched)

@@ -13,6 +13,7 @@ import os
 # TRIATTN_HIP_LIBRARY points at another build of the same ABI (e.g. an instrumented one).
 LIB_PATH = Path(os.environ.get("TRIATTN_HIP_LIBRARY") or Path(__file__).resolve().parent / "libtriattention_hip.so")
 
+ABI_VERSION = 4
 TRI_OK = 0
 TRI_ERR_INVALID_ARGUMENT = -1
 TRI_ERR_UNSUPPORTED = -2
@@ -61,7 +62,7 @@ class SelectParams(C.Structure):
     _fields_ = [
         ("normalize", C.c_int32), ("window_size", C.c_int32), ("protect_prefill", C.c_int32),
         ("group_reduce", C.c_int32), ("layer_reduce", C.c_int32), ("shared", C.c_int32),
-        ("group_first", C.c_int32),
+        ("group_first", C.c_int32), ("no_resident", C.c_int32),
     ]
 
 
@@ -114,8 +115,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         if fn.restype is C.c_int and name not in ("tri_abi_version",):
             fn.restype = C.c_int
-    if lib.tri_abi_version() != 3:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != 3; rebuild the library")
+    if lib.tri_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != {ABI_VERSION}; rebuild the library")
     _lib = lib
     return lib
 

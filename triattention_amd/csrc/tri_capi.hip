@@ -193,7 +193,7 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
 int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
                     hipStream_t s) {
-  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first;
+  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident;
   if (!fused) {
     // The status word belongs to the resident kernel; on this path it just reads "fine".
     const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
@@ -393,7 +393,8 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first) ? w.fused.eligible : 0;
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident)
+             ? w.fused.eligible : 0;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,

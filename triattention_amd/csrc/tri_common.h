@@ -66,6 +66,9 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   int64_t off = 0;
   auto take = [&](int64_t bytes) { int64_t o = off; off = align_up(off + bytes, 256); return o; };
   w.num_tiles = ceil_div(Tmax > 0 ? Tmax : 1, kScoreTileTokens);
+  // The status word comes first, so its place does not depend on the batch: a caller that
+  // reuses one workspace for steps of different shapes always reads the same word.
+  w.status = take(256);
   w.coef = take((int64_t)B * L * A * 3 * F * 4);
   w.trig = take((int64_t)B * (NO + 1) * 2 * F * 4);
   w.partial = take((int64_t)B * L * w.num_tiles * A * 2 * 4);
@@ -73,7 +76,6 @@ inline Workspace plan_workspace(int B, int L, int A, int F, int NO, int Hkv, int
   w.raw = take((int64_t)B * L * Tmax * A * 4);
   w.fin = take((int64_t)B * L * Hkv * Tmax * 4);
   w.xchg = take(fused.eligible ? (int64_t)B * L * fused.tiles_per_seq * A * 2 * 8 : 0);
-  w.status = take(256);
   w.pack = take(fused.eligible ? (int64_t)B * 8 : 0);
   // key slabs (head_dim / 32) and magnitude slabs (half as many) per group of four query heads
   const int slabs = max(F / 16 + F / 32, 6);

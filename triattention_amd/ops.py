@@ -268,13 +268,15 @@ class SelectConfig:
     layer_reduce: str | None = "mean"    # None: one keep set per layer
     shared: bool = False
     group_first: bool = False            # reduce over the query heads of a KV head before normalising
+    allow_resident: bool = True          # False: never a resident kernel (repeat of a step whose resident launch failed)
 
     def struct(self) -> SelectParams:
         lr = REDUCE_NONE if self.layer_reduce is None else (REDUCE_MAX if self.layer_reduce == "max" else REDUCE_MEAN)
         return SelectParams(normalize=int(self.normalize), window_size=int(self.window_size),
                             protect_prefill=int(self.protect_prefill),
                             group_reduce=REDUCE_MAX if self.group_reduce == "max" else REDUCE_MEAN,
-                            layer_reduce=lr, shared=int(self.shared), group_first=int(self.group_first))
+                            layer_reduce=lr, shared=int(self.shared), group_first=int(self.group_first),
+                            no_resident=int(not self.allow_resident))
 
 
 def fold_stats(q_mean_complex: torch.Tensor, q_abs_mean: torch.Tensor, freq_scale_sq: torch.Tensor,
@@ -309,6 +311,8 @@ class Workspace:
         self.buf = torch.empty(self.bytes + 256, dtype=torch.uint8, device=kv.device)
         off = (-self.buf.data_ptr()) % 256
         self.ptr = self.buf.data_ptr() + off
+        # The library keeps the status word at one offset for every shape, so a workspace reused
+        # for another batch (fits()) still reads the word the kernels of that batch write.
         self._status_at = off + int(lib.tri_workspace_status_offset(C.byref(kv.struct), C.byref(batch.struct),
                                                                     C.byref(sp)))
 

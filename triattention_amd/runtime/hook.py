@@ -557,10 +557,15 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
             if not members:
                 continue
             try:
-                selected = compress_batch(layer_kv=group_tensors[gid], block_size=batch[0].block_size,
-                                          requests=requests)
-            except ResidentLaunchFailed:
-                raise
+                try:
+                    selected = compress_batch(layer_kv=group_tensors[gid], block_size=batch[0].block_size,
+                                              requests=requests)
+                except ResidentLaunchFailed:
+                    # The guarded compaction moved nothing of THIS group; groups handled before it
+                    # are compacted and truncated already and stay as they are.  Repeat this
+                    # group alone on the kernels that do not wait for each other.
+                    selected = compress_batch(layer_kv=group_tensors[gid], block_size=batch[0].block_size,
+                                              requests=requests, allow_resident=False)
             except Exception as exc:
                 raise RuntimeError(f"{MARK}:batch:gid={gid}:global_per_head:{type(exc).__name__}") from exc
             for (r, ids, total), res in zip(members, selected):
@@ -612,20 +617,7 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
         if len(together) == 1:
             results[together[0].req_id] = _run_single(together[0])
         elif together:
-            try:
-                results.update(_run_batch(together))
-            except ResidentLaunchFailed:
-                # Nothing was moved.  Repeat on the kernels that do not wait for each other.
-                previous = os.environ.get("TRIATTN_RESIDENT_KERNEL")
-                os.environ["TRIATTN_RESIDENT_KERNEL"] = "off"
-                try:
-                    for r in together:
-                        results[r.req_id] = _run_single(r)
-                finally:
-                    if previous is None:
-                        os.environ.pop("TRIATTN_RESIDENT_KERNEL", None)
-                    else:
-                        os.environ["TRIATTN_RESIDENT_KERNEL"] = previous
+            results.update(_run_batch(together))
         return {req_id: results[req_id] for req_id in signals if req_id in results}
 
     _hook.batch = _batch_hook

@@ -162,10 +162,14 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         try:
             resident = ops.select_path(kv, batch, sc, sel) != "two_pass"   # (a single request: only when forced)
             keep, _, ws = ops.select_paged(kv, batch, sc, sel)
+            if resident and ws.status() != 0:
+                # A wait inside the resident kernel expired (or a coefficient did not fit its operand
+                # type): the keep lists mean nothing.  Nothing has been moved yet; score again on the
+                # kernels that do not wait for each other.
+                sel.allow_resident = False
+                keep, _, ws = ops.select_paged(kv, batch, sc, sel, ws)
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
-        if resident and ws.status() != 0:
-            raise RuntimeError(f"{MARK}:score_failed:ResidentLaunchFailed")
         return mark_keep_validated(keep.to(torch.long), total_tokens)
 
     def _select_keep_indices(*, keys_dense: torch.Tensor | None = None, kv_cache: torch.Tensor | None = None,
@@ -246,7 +250,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                 "group_agg_mode": agg, "debug_group_layer_indices": list(layer_ids),
                 "debug_recent_count": _recent_count(total_tokens)}
 
-    def _compress_group_batch(*, layer_kv: list, block_size: int, requests: list) -> list:
+    def _compress_group_batch(*, layer_kv: list, block_size: int, requests: list,
+                              allow_resident: bool = True) -> list:
         """Selection **and** compaction of several requests of one KV-cache group in one launch
         sequence (no counterpart in the reference, which walks the requests one by one,
         runner_compression_actions.py:24; per request the result equals what
@@ -256,8 +261,9 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         with ``block_ids, total_tokens, prefill_len, protect_prefill, round_start, budget_total``
         and ``total_tokens > budget_total > 0``.  Returns the selector result dictionaries in
         request order; the caches then hold the kept rows in slots ``0..k-1``.  Raises
-        ``ResidentLaunchFailed`` with the caches untouched when a wait inside the resident
-        kernel expired."""
+        ``ResidentLaunchFailed`` with the caches of this group untouched when a wait inside the
+        resident kernel expired; the caller repeats the call with ``allow_resident=False``, which
+        takes the kernels that do not wait for each other."""
         if mode != "per_head" or semantics != "hf_aligned_global_per_head":
             raise RuntimeError("batched compression serves the per_head / hf_aligned_global_per_head mode only")
         agg = os.environ.get("TRIATTN_RUNTIME_DEBUG_GROUP_PERHEAD_AGG_MODE", "mean").strip().lower()
@@ -281,7 +287,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                               block_tables=[[int(x) for x in r["block_ids"]] for r in requests],
                               prefill_lens=guards)
         sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
-                               protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg)
+                               protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
+                               allow_resident=bool(allow_resident))
         resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
         try:
             keep, ws = ops.compress_step(kv, batch, sc, sel)
