@@ -31,8 +31,10 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # the same counters read for the 1 GiB copies of --copy-calibration).  Keyed by
 # (workload, path); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_qwen3_8b_36l_b16_16k", "two_pass"): 9_717_510 * 1024 * 2 + 1_184_256 * 1024,     # score_mean_kernel
-    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): 9_476_694 * 1024 * 2 + 12_800 * 1024,      # fused_mfma_kernel
+    ("c1_qwen3_8b_36l_b16_16k", "two_pass"): (9_717_510 * 1024 * 2 + 1_184_256 * 1024,       # score_mean_kernel
+                                               "profiles/c1_step_hbm_counters.txt"),
+    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_476_694 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
+                                                    "profiles/c1_step_hbm_counters.txt"),
 }
 
 
@@ -43,6 +45,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=1, help="workload index 0..4 (default 1: 36 layers, 16 x 16384 tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sustained-steps", type=int, default=400,
+                    help="back-to-back steps of the sustained (warm clocks) measurement after the timed region; 0: skip")
+    ap.add_argument("--no-parity-check", action="store_true",
+                    help="skip the keep-set comparison of the timed path with the two-pass kernels (and, with the CPU "
+                         "baseline, with the oracle on sequence 0)")
     ap.add_argument("--cpu-layers", type=int, default=36, help="layers of one sequence the CPU baseline scores")
     ap.add_argument("--seq-len", type=int, default=0,
                     help="override every sequence's cached length (e.g. budget + 128 for the steady-state step)")
@@ -68,9 +75,12 @@ def parse_args():
     return ap.parse_args()
 
 
-def cpu_baseline(w, layers: int):
-    """The CPU oracle (a port of the reference's PyTorch path) on a bounded sample:
-    one sequence, `layers` layers, same shapes and seeded distributions."""
+def cpu_baseline(w, layers: int, seq0=None):
+    """The CPU oracle (a port of the reference's PyTorch path) on a bounded sample: one sequence,
+    `layers` layers.  With ``seq0`` (the blocks of sequence 0 of the GPU run, copied to the host:
+    ``{"caches": [L x [2, nblk, bs, H, D]], "qc", "qa"}``) the oracle scores exactly what the GPU
+    scored, and its keep set is returned for comparison; otherwise same shapes and seeded
+    distributions."""
     from oracle import compaction as ocp
     from oracle import scoring as osc
     from oracle import selection as osel
@@ -79,9 +89,14 @@ def cpu_baseline(w, layers: int):
     torch.set_num_threads(os.cpu_count() or 1)
     layers = min(layers, w.num_layers)
     sample = w.scaled(seq_lens=(w.seq_lens[0],), num_layers=layers, kv_dtype="bf16" if w.kv_dtype == "fp8" else w.kv_dtype)
-    tables = synth.make_block_tables(sample)
-    caches = synth.make_kv_pool(sample, tables, "cpu")
-    qc, qa = synth.make_stats(sample, "cpu")
+    if seq0 is not None and layers == w.num_layers:
+        caches, qc, qa = seq0["caches"], seq0["qc"], seq0["qa"]
+        tables = [list(range(int(caches[0].shape[1])))]
+    else:
+        seq0 = None
+        tables = synth.make_block_tables(sample)
+        caches = synth.make_kv_pool(sample, tables, "cpu")
+        qc, qa = synth.make_stats(sample, "cpu")
     omega, offsets = synth.rope_inv_freq(sample), synth.geometric_offsets()
     fs = torch.ones(layers, sample.num_q_heads, sample.head_dim // 2)
     t = sample.seq_lens[0]
@@ -92,16 +107,38 @@ def cpu_baseline(w, layers: int):
         kc, _ = ocp.split_kv(caches[l])
         keys = ocp.gather_dense(kc, tables[0], sample.block_size, 0, t)[0].float().repeat_interleave(g, dim=0)
         raw.append(osc.raw_scores(keys, qc[l], qa[l], omega, offsets, fs[l], t))
-    keep, _ = osel.group_keep_per_head(raw, sample.num_kv_heads, sample.budget, window_size=sample.window_size,
-                                       chunk_tokens=osel.score_chunk_tokens(sample.block_size, t))
+    keep, fin = osel.group_keep_per_head(raw, sample.num_kv_heads, sample.budget, window_size=sample.window_size,
+                                         chunk_tokens=osel.score_chunk_tokens(sample.block_size, t))
     for l in range(layers):
         ocp.compact_per_head(caches[l], tables[0], sample.block_size, keep, t, full_permutation=True)
     dt = time.perf_counter() - t0
     # one "key" is one cached token across ALL layers of the model: scale the sample's layer count up
     keys_per_s = t / (dt * w.num_layers / layers)
-    return {"value": keys_per_s, "unit": "keys/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 sequence x {t} tokens x {layers} of {w.num_layers} layers, {dt:.2f} s on the host; "
-                      f"rate scaled to all {w.num_layers} layers"}
+    what = "sequence 0 of the GPU run (its own keys and statistics)" if seq0 is not None else "1 sequence"
+    out = {"value": keys_per_s, "unit": "keys/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"{what} x {t} tokens x {layers} of {w.num_layers} layers, {dt:.2f} s on the host; "
+                     f"rate scaled to all {w.num_layers} layers"}
+    return out, (keep, fin) if seq0 is not None else None
+
+
+def keep_differences(got: torch.Tensor, want: torch.Tensor, fin: torch.Tensor, ks, heads: int, tie: float = 1e-5):
+    """Kept indices of ``got`` that ``want`` does not hold (rows = sequences x heads, CPU tensors), and
+    how many of them are near-ties: selection score within ``tie`` x the largest finite score of the
+    row's sequence of the row's threshold (the k-th largest of ``fin``)."""
+    diff = near = 0
+    for r in range(got.shape[0]):
+        k = ks[r // heads]
+        a, b = set(got[r, :k].tolist()), set(want[r, :k].tolist())
+        if a == b:
+            continue
+        row = fin[r]
+        finite = row[torch.isfinite(row)]
+        scale = float(finite.abs().max()) if finite.numel() else 1.0
+        thr = float(torch.sort(row, descending=True).values[k - 1])
+        for idx in a - b:
+            diff += 1
+            near += abs(float(row[idx]) - thr) <= tie * scale
+    return diff, near
 
 
 def hook_latency(w, dev, calls: int = 30, requests: int = 1):
@@ -333,12 +370,74 @@ def main() -> int:
     score_gbs = algo["score"] / (mean(score_ms) * 1e-3) / 1e9
     compact_gbs = algo["compact"] / (mean(compact_ms) * 1e-3) / 1e9
 
+    if not two_pass and ws.status() != 0:
+        print("bench.py: the resident kernel raised its status word during the timed steps; the step did not "
+              "do its work and the timing is void", file=sys.stderr)
+        return 3
+    keep_timed = keep.clone()
+
+    # Sustained figure: the same step back to back (with the restore copies between, which keep the
+    # memory system just as busy) for a few seconds, so the GPU sits at the clocks it holds under
+    # this load; the last quarter of the steps is what is reported.
+    sustained = None
+    if args.sustained_steps > 0:
+        n = args.sustained_steps
+        tail = max(1, min(100, n // 4))
+        sev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(tail)]
+        restore()
+        torch.cuda.synchronize()
+        s0 = time.perf_counter()
+        for i in range(n):
+            j = i - (n - tail)
+            if j >= 0:
+                sev[j][0].record()
+            step()
+            if j >= 0:
+                sev[j][1].record()
+            restore()
+        torch.cuda.synchronize()
+        s_wall = time.perf_counter() - s0
+        if not two_pass and ws.status() != 0:
+            print("bench.py: status word raised during the sustained steps", file=sys.stderr)
+            return 3
+        tail_ms = sorted(a.elapsed_time(b) for a, b in sev)
+        s_ms = sum(tail_ms) / len(tail_ms)
+        sustained = {"steps": n, "wall_s": s_wall, "ms_per_step": s_ms, "ms_per_step_of": f"last {tail} steps",
+                     "step_ms_p50": tail_ms[len(tail_ms) // 2], "step_ms_max": tail_ms[-1],
+                     "value": total_keys / (s_ms * 1e-3), "achieved_gbs": algo["total"] / (s_ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": algo["total"] / (s_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    # Parity of what was timed, outside every timed region: on the pristine cache the timed path's
+    # keep rows against the two-pass kernels' (and further down against the CPU oracle on sequence 0).
+    parity = None
+    seq0 = None
+    if not args.no_parity_check and args.aggregation == "mean":
+        restore()
+        heads = w.num_kv_heads
+        ks = [min(w.budget, t) for t in w.seq_lens]
+        two = ops.SelectConfig(window_size=w.window_size, allow_resident=False)
+        ops.select_paged(kv, batch, sc, two if two_pass else sel, ws, scores_out=fin_buf, want_keep=False)
+        keep_again = ops.topk_batch(fin_buf, batch, heads)
+        keep_tp, fin_tp, _ = ops.select_paged(kv, batch, sc, two, ws, want_scores=True)
+        torch.cuda.synchronize()
+        same_as_timed = all(torch.equal(keep_again[b * heads:(b + 1) * heads, :k], keep_timed[b * heads:(b + 1) * heads, :k])
+                            for b, k in enumerate(ks))
+        diff, near = keep_differences(keep_again.cpu(), keep_tp.cpu(), fin_tp.cpu(), ks, heads)
+        parity = {"timed_path": path, "kept_indices_compared": sum(ks) * heads, "timed_keep_reproduced": same_as_timed,
+                  "vs_two_pass_diff": diff, "vs_two_pass_near_tie_swaps": near, "near_tie_bound": "1e-5 of the largest score"}
+        gpu_rows0 = keep_again[:heads, :ks[0]].cpu()
+        del keep_tp, fin_tp
+        if not args.no_cpu_baseline and w.kv_dtype != "fp8" and args.cpu_layers >= w.num_layers:
+            blocks0 = torch.tensor(tables[0], device=dev, dtype=torch.long)
+            seq0 = {"caches": [c[:, blocks0].cpu() for c in caches], "qc": qc.cpu(), "qa": qa.cpu(), "gpu_rows": gpu_rows0}
+
     if args.aggregation == "mean":
         two_pass_kernel = "score_mean_kernel"
     elif w.kv_dtype == "bf16" and w.head_dim == 128 and os.environ.get("TRIATTN_MAX_KERNEL") != "valu":
         two_pass_kernel = "score_max_mfma_kernel"
     else:
         two_pass_kernel = "score_max_kernel"
+    traffic = MEASURED_TRAFFIC_BYTES.get((w.name, path)) if args.aggregation == "mean" else None
     out = {
         "metric": "keys scored+compacted/sec & achieved HBM GB/s (% peak), Qwen3-8B 16k ctx",
         "value": keys_per_s,
@@ -371,8 +470,14 @@ def main() -> int:
         "roofline": {"kernel": {"two_pass": two_pass_kernel, "resident_valu": "fused_select_kernel",
                                 "resident_mfma": "fused_mfma_kernel"}[path], "bound": "hbm",
                      "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, path)) if args.aggregation == "mean" else None},
+                     "traffic": traffic[0] if traffic else None,
+                     "traffic_source": (traffic[1] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by "
+                                        "the same counters on a 1 GiB copy; not measured by this run)") if traffic else None},
     }
+    if sustained is not None:
+        out["sustained"] = sustained
+    if parity is not None:
+        out["parity_check"] = parity
     # A plain device-to-device copy of 1 GiB on the same box, for scale: bytes read + bytes
     # written per second (outside every timed region of the step).
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -403,7 +508,13 @@ def main() -> int:
     if not args.no_cpu_baseline:
         del saved, caches, pool
         torch.cuda.empty_cache()
-        out["cpu_baseline"] = cpu_baseline(w, args.cpu_layers)
+        out["cpu_baseline"], oracle_keep = cpu_baseline(w, args.cpu_layers, seq0)
+        if oracle_keep is not None:
+            okeep, ofin = oracle_keep
+            heads = w.num_kv_heads
+            diff, near = keep_differences(seq0["gpu_rows"], okeep, ofin, [int(okeep.shape[1])], heads)
+            out["parity_check"].update({"vs_oracle_seq0_diff": diff, "vs_oracle_seq0_near_tie_swaps": near,
+                                        "vs_oracle_seq0_compared": int(okeep.numel())})
     print(json.dumps(out))
     return 0
 

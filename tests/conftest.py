@@ -30,3 +30,17 @@ def pytest_collection_modifyitems(config, items):
 def load_golden(name: str):
     """Fixtures are plain tensor dicts this repo wrote; nothing in them executes."""
     return torch.load(GOLDEN / name, map_location="cpu", weights_only=True)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """One line for the whole run: how many kept indices differed from the oracle's (or the other
+    path's) at near-ties, over how many compared."""
+    import helpers
+    if not helpers.SWAPS:
+        return
+    swapped = sum(s for s, _ in helpers.SWAPS.values())
+    compared = sum(c for _, c in helpers.SWAPS.values())
+    cases = sorted(name for name, (s, _) in helpers.SWAPS.items() if s)
+    terminalreporter.write_line(
+        f"near-tie swaps: {swapped} of {compared} kept indices in {len(helpers.SWAPS)} comparisons"
+        + (f" (cases: {', '.join(cases)})" if cases else ""))

@@ -64,6 +64,46 @@ def score_tolerance(ref: torch.Tensor):
     return 1e-3 * ref.pow(2).mean(dim=-1, keepdim=True).sqrt()
 
 
+# The contract is "identical kept-index sets except at exact score ties".  fp32 sums taken in
+# another order move a selection score by ~1e-6 of the largest one (measured), so an index may
+# legitimately differ only when its score lies within KEEP_TIE_TOL (ten times that) of the
+# threshold score; selection scores themselves must agree to SELECT_SCORE_TOL.  Both are
+# fractions of the largest finite selection score of the rows compared.
+KEEP_TIE_TOL = 1e-5
+SELECT_SCORE_TOL = 5e-5
+
+
+
+def selection_score_tol(raw_rows) -> float:
+    """Tolerance for selection scores, as a fraction of the largest one.  The reference's streaming
+    variance, sum(x^2) - n * mean^2 in fp32 (runtime/selector_hf.py:902-909), cancels
+    kappa = mean(x^2) / var(x) leading digits, so two correct fp32 evaluations that group their sums
+    differently disagree by a few eps * kappa in the z-scores: 1.5e-5 at kappa = 130 (head_dim 128
+    with the benchmark's key distribution), 9e-5 at kappa = 430 (head_dim 256, measured).
+    ``raw_rows``: raw scores with tokens along the last dimension (a tensor or a list of tensors);
+    rows of fewer than two tokens have no variance and are left out."""
+    rows = raw_rows if isinstance(raw_rows, (list, tuple)) else [raw_rows]
+    kappa = 1.0
+    for r in rows:
+        if r.shape[-1] < 2:
+            continue
+        r = r.double()
+        var = r.var(-1)
+        ok = var > 0
+        if bool(ok.any()):
+            kappa = max(kappa, float((r.pow(2).mean(-1)[ok] / var[ok]).max()))
+    return max(SELECT_SCORE_TOL, 8 * 2.0 ** -24 * kappa)
+
+
+# test id -> (indices swapped at near-ties, indices compared); reported in one line at the end of a run
+SWAPS: dict = {}
+
+
+def record_swaps(case: str, swapped: int, compared: int) -> None:
+    have = SWAPS.get(case, (0, 0))
+    SWAPS[case] = (have[0] + int(swapped), have[1] + int(compared))
+
+
 def assert_keep_matches(keep: torch.Tensor, want: torch.Tensor, fin: torch.Tensor, k: int, tie_tol: float):
     """Kept sets equal, except indices whose oracle score is within tie_tol of the
     k-th largest oracle score (fp32 rounding of a different summation order can swap

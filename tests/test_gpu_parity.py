@@ -8,7 +8,8 @@ import pytest
 import torch
 
 from conftest import load_golden
-from helpers import assert_keep_matches, build_inputs, device_objects, oracle_raw, score_tolerance
+from helpers import (KEEP_TIE_TOL, SELECT_SCORE_TOL, assert_keep_matches, build_inputs, device_objects, oracle_raw,
+                     record_swaps, score_tolerance, selection_score_tol)
 from oracle import compaction as ocp
 from oracle import scoring as osc
 from oracle import selection as osel
@@ -130,7 +131,7 @@ def test_max_aggregation_on_matrix_cores_matches_the_vector_unit_kernel(name, mo
         finite = torch.isfinite(fv)
         assert torch.equal(torch.isfinite(fm), finite)
         if bool(finite.any()):
-            assert float((fm[finite] - fv[finite]).abs().max()) <= 5e-4 * float(fv[finite].abs().max()), (name, b)
+            assert float((fm[finite] - fv[finite]).abs().max()) <= SELECT_SCORE_TOL * float(fv[finite].abs().max()), (name, b)
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("TRIATTN_TEST_RANDOM_SHAPES", "32")) // 2))
@@ -213,7 +214,7 @@ def test_group_selection_matches_oracle(name):
     torch.cuda.synchronize()
     keep, fin = keep.cpu(), fin.cpu()
     h = w.num_kv_heads
-    total_swapped = 0
+    total_swapped = compared = 0
     for b, t in enumerate(w.seq_lens):
         k = min(w.budget, t)
         oraw = oracle_raw(w, inp, b, t)
@@ -232,9 +233,12 @@ def test_group_selection_matches_oracle(name):
         if not bool(finite.any()):        # every token guarded: any k of them is as good as another
             continue
         scale = ofin[finite].abs().max()
-        assert float((dfin[finite] - ofin[finite]).abs().max()) <= 2e-3 * float(scale)
-        total_swapped += assert_keep_matches(got, want, ofin, k, tie_tol=2e-3 * float(scale))
-    print("swapped near-tie indices:", total_swapped, flush=True)
+        assert float((dfin[finite] - ofin[finite]).abs().max()) <= selection_score_tol(oraw) * float(scale)
+        total_swapped += assert_keep_matches(got, want, ofin, k, tie_tol=KEEP_TIE_TOL * float(scale))
+        compared += h * k
+    record_swaps(f"two_pass_vs_oracle:{name}", total_swapped, compared)
+    if not name.startswith("random"):
+        assert total_swapped == 0, (name, total_swapped)
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("TRIATTN_TEST_RANDOM_SHAPES", "32")) // 2))
@@ -309,6 +313,89 @@ def test_group_selection_matches_reference_golden(tag, kw, path, fixture, monkey
     diff = sum(len(set(got[h].tolist()) ^ set(want[h].tolist())) for h in range(hkv))
     assert diff == 0, f"{diff} indices differ from the reference's keep set"
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("tag,protect", [("default", False), ("chunk64_prefill", True)])
+@pytest.mark.parametrize("path,copies,workgroups", [
+    ("two_pass", 1, None),
+    ("resident_mfma", 1, 5),        # five tiles of 1024 tokens on the eight-wave instance the benchmark times
+    ("resident_mfma", 3, 15),       # three requests in one launch, each must come out as the single one
+    ("resident_mfma", 3, 10),       # ... and in two launches (two sequences, then one)
+    ("resident_valu", 1, 5),
+])
+def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(tag, protect, path, copies,
+                                                                                workgroups, monkeypatch):
+    """The reference's keep sets for a 5000-token request of 32 query / 8 KV heads of 128 (budget
+    2048, window 128; written by tests/golden/make_c1_shape_golden.py): its variance streams over
+    two 4096-token chunks and its chunked top-k merges.  The resident matrix-core kernel is
+    pinned to the instance and tile size of the 16 x 16384-token benchmark step (tiles of 1024
+    tokens, workgroups of eight waves) by pretending the device holds only five workgroups.
+    Gate: the reference's rows, except indices whose reference score lies within KEEP_TIE_TOL of
+    the threshold score."""
+    from golden.hashed_inputs import checksum, hashed_rows
+    gold = load_golden("selector_c1_shape.pt")
+    layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
+    keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
+    assert checksum(keys) == int(gold["key_checksum"]), "the hashed keys differ from the ones the golden was written for"
+    pool = int(gold["pool_blocks"])
+    ids = gold["block_ids"]
+    tok = torch.arange(t)
+    caches = []
+    for l in range(layers):
+        kvc = torch.zeros(2, pool * copies, bs, hkv, d, dtype=torch.bfloat16)
+        for c in range(copies):
+            kvc[0, ids[tok // bs] + c * pool, tok % bs] = keys[l].transpose(0, 1)
+        caches.append(kvc.to(DEV))
+    tables = [(ids + c * pool).tolist() for c in range(copies)]
+    if path != "two_pass":
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", path.split("_")[1])
+        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", str(workgroups))
+    kv = ops.PagedKV.from_kv_caches(caches)
+    budget = int(gold["budget"])
+    batch = ops.StepBatch(DEV, [t] * copies, round_start=[int(gold["round_start"])] * copies, budgets=budget,
+                          block_tables=tables, prefill_lens=[int(gold["prefill_len"])] * copies)
+    folded = ops.fold_stats(gold["q_mean_complex"].to(DEV), gold["q_abs_mean"].to(DEV),
+                            torch.ones(layers, hq, d // 2, device=DEV))
+    sc = ops.ScoreConfig(folded, gold["omega"].to(DEV), synth.geometric_offsets(device=DEV))
+    sel = ops.SelectConfig(window_size=int(gold["window"]), protect_prefill=protect,
+                           allow_resident=path != "two_pass")
+    assert ops.select_path(kv, batch, sc, sel) == path
+    keep, _, ws = ops.select_paged(kv, batch, sc, sel)
+    assert ws.status() == 0
+    want = gold[f"group_{tag}_keep"].long()
+    okeep, ofin = _c1_shape_oracle(tag)
+    assert torch.equal(okeep, want)          # the oracle reproduces the reference's keep set exactly
+    scale = float(ofin[torch.isfinite(ofin)].abs().max())
+    got = keep.cpu().long().view(copies, hkv, budget)
+    swapped = 0
+    for c in range(copies):
+        # Identical to the reference's rows except where a score sits within KEEP_TIE_TOL of the
+        # threshold: there the reference's own fp32 rounding decides (its selection scores are
+        # 8e-6 .. 2e-5 of the largest one away from a double-precision evaluation, the kernels'
+        # 6e-6 .. 7e-6; the one pair per request that swaps lies 2e-6 .. 4e-6 from the threshold).
+        swapped += assert_keep_matches(got[c], want, ofin, budget, tie_tol=KEEP_TIE_TOL * scale)
+    record_swaps(f"reference_golden_c1_shape:{path}:{copies}x:{workgroups}:{tag}", swapped, copies * hkv * budget)
+    assert swapped <= 2 * copies, swapped
+
+
+_C1_SHAPE_ORACLE: dict = {}
+
+
+def _c1_shape_oracle(tag):
+    """Keep rows and selection scores of the CPU oracle for tests/golden/selector_c1_shape.pt."""
+    if tag not in _C1_SHAPE_ORACLE:
+        from golden.hashed_inputs import hashed_rows
+        gold = load_golden("selector_c1_shape.pt")
+        layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
+        keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
+        offs = osc.geometric_offsets(65536)
+        raw = [osc.raw_scores(keys[l].float().repeat_interleave(hq // hkv, dim=0), gold["q_mean_complex"][l],
+                              gold["q_abs_mean"][l], gold["omega"], offs, torch.ones(hq, d // 2), int(gold["round_start"]))
+               for l in range(layers)]
+        kw = dict(chunk_tokens=64, protect_prefill=True) if tag == "chunk64_prefill" else dict(chunk_tokens=4096)
+        _C1_SHAPE_ORACLE[tag] = osel.group_keep_per_head(raw, hkv, int(gold["budget"]), window_size=int(gold["window"]),
+                                                         prefill_len=int(gold["prefill_len"]), **kw)
+    return _C1_SHAPE_ORACLE[tag]
 
 
 @pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
@@ -535,8 +622,9 @@ def test_end_to_end_c0_against_oracle():
                                           chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
     got = keep.cpu().long()
     scale = float(ofin[torch.isfinite(ofin)].abs().max())
-    swapped = assert_keep_matches(got, want, ofin, k, tie_tol=2e-3 * scale)
-    print("c0 swapped near-tie indices:", swapped, "of", h * k, flush=True)
+    swapped = assert_keep_matches(got, want, ofin, k, tie_tol=KEEP_TIE_TOL * scale)
+    record_swaps("c0_vs_oracle", swapped, h * k)
+    assert swapped == 0
     # compaction is bit-exact given the device's own keep set
     ref = inp["caches"][0].clone()
     ocp.compact_per_head(ref, inp["tables"][0], w.block_size, got, t, full_permutation=False)
@@ -614,6 +702,12 @@ RESIDENT_CASES.update({
 })
 
 
+# Named cases in which the two paths keep different indices at near-ties (scores within
+# KEEP_TIE_TOL of the threshold), and how many of the case's kept indices: 16 sequences x heads x
+# 256 kept indices each, two of which sit that close to their threshold.  Everywhere else: none.
+NEAR_TIES = {("fp16_tile192", "mfma"): 2, ("d64_tile_refined", "mfma"): 2}
+
+
 @pytest.mark.parametrize("kernel", ["mfma", "valu"])
 @pytest.mark.parametrize("name", list(RESIDENT_CASES))
 def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
@@ -645,15 +739,21 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     torch.cuda.synchronize()
     assert ws.status() == 0
     h = w.num_kv_heads
+    swapped = compared = 0
     for b, t in enumerate(w.seq_lens):
         k = min(w.budget, t)
         fr, ft = fin_r[b * h:(b + 1) * h, :t].cpu(), fin_t[b * h:(b + 1) * h, :t].cpu()
         assert torch.equal(torch.isinf(fr), torch.isinf(ft))
         finite = torch.isfinite(ft)
         scale = float(ft[finite].abs().max()) if bool(finite.any()) else 1.0
-        assert float((fr[finite] - ft[finite]).abs().max() if bool(finite.any()) else 0.0) <= 5e-4 * scale, (name, b)
-        assert_keep_matches(keep_r[b * h:(b + 1) * h, :k].cpu().long(), keep_t[b * h:(b + 1) * h, :k].cpu().long(),
-                            ft, k, tie_tol=2e-3 * scale)
+        tol = selection_score_tol(raw[b, :, :t].transpose(-1, -2).cpu()) if sel.normalize else SELECT_SCORE_TOL
+        assert float((fr[finite] - ft[finite]).abs().max() if bool(finite.any()) else 0.0) <= tol * scale, (name, b)
+        swapped += assert_keep_matches(keep_r[b * h:(b + 1) * h, :k].cpu().long(),
+                                       keep_t[b * h:(b + 1) * h, :k].cpu().long(), ft, k, tie_tol=KEEP_TIE_TOL * scale)
+        compared += h * k
+    record_swaps(f"resident_{kernel}_vs_two_pass:{name}", swapped, compared)
+    if not name.startswith("random"):
+        assert swapped <= NEAR_TIES.get((name, kernel), 0), (name, kernel, swapped)
 
 
 def _random_resident_case(seed: int):
@@ -966,7 +1066,7 @@ def test_fp8_step_scores_selects_and_compacts():
             want, ofin = osel.group_keep_per_head(oraw, h, k, window_size=w.window_size,
                                                   chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
             scale = float(ofin[torch.isfinite(ofin)].abs().max())
-            assert_keep_matches(rows, want, ofin, k, tie_tol=2e-3 * scale)
+            assert assert_keep_matches(rows, want, ofin, k, tie_tol=KEEP_TIE_TOL * scale) == 0
         else:
             assert torch.equal(rows, torch.arange(t).expand(h, t))
     for l in range(w.num_layers):

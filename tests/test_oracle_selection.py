@@ -72,6 +72,28 @@ def test_layer_selection_matches_reference(tag, fixture):
     assert torch.equal(keep, want)
 
 
+@pytest.mark.parametrize("tag,kw", [("default", dict(chunk_tokens=4096)),
+                                    ("chunk64_prefill", dict(chunk_tokens=64, protect_prefill=True))])
+def test_group_selection_matches_reference_across_chunks_at_the_benchmarked_head_shape(tag, kw):
+    """32 query / 8 KV heads of 128, 5000 tokens, budget 2048: the reference's streaming variance
+    spans two 4096-token chunks (79 chunks of 64 in the second setting) and its chunked top-k
+    merges.  The keys are rebuilt from the fixture's seed and checked against its checksum."""
+    from golden.hashed_inputs import checksum, hashed_rows
+    gold = load_golden("selector_c1_shape.pt")
+    layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
+    keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
+    assert checksum(keys) == int(gold["key_checksum"])
+    offs = osc.geometric_offsets(65536)
+    raw = [osc.raw_scores(keys[l].float().repeat_interleave(hq // hkv, dim=0), gold["q_mean_complex"][l],
+                          gold["q_abs_mean"][l], gold["omega"], offs, torch.ones(hq, d // 2), int(gold["round_start"]))
+           for l in range(layers)]
+    keep, fin = osel.group_keep_per_head(raw, hkv, int(gold["budget"]), window_size=int(gold["window"]),
+                                         prefill_len=int(gold["prefill_len"]), **kw)
+    want = gold[f"group_{tag}_keep"].long()
+    _sets_equal_off_ties(keep, want, fin, int(gold["budget"]))
+    assert torch.equal(keep, want)
+
+
 def test_streaming_stats_match_torch():
     g = torch.Generator().manual_seed(3)
     x = torch.randn(6, 1000, generator=g) * 3 + 5
