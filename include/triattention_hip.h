@@ -220,6 +220,25 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
                       const tri_select_params* sel, int32_t* keep, void* workspace,
                       uint64_t workspace_bytes, void* stream);
 
+/* tri_compress_step for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the
+ * reference.  The scratch the kernels need (coefficients, trig tables, per-tile sums, raw
+ * scores, selection scores, status word) lives in a device array inside the library,
+ * TRI_STATIC_WORKSPACE_BYTES per GPU from the moment the library is loaded until the process
+ * ends; the call allocates nothing, frees nothing, creates no stream or event, and always takes
+ * the score-then-select kernels (never a resident kernel; for fp8 caches the scales follow the
+ * rows on `stream`).  A step whose scratch (tri_workspace_bytes) exceeds the array is rejected
+ * with TRI_ERR_WORKSPACE: Qwen3-8B shapes (36 layers) fit up to 4 sequences of budget + 128 = 2176
+ * tokens, or one sequence of 11400.  Every call on a GPU uses that GPU's one array, which keeps the
+ * previous call's contents (nothing in it needs to start at zero except the status word, which
+ * the call clears): calls that overlap in time on one GPU, from any streams or threads, race.
+ * Results are those of tri_compress_step with no_resident = 1.  status_out (may be NULL)
+ * receives the device address of the status word for callers that want to read it. */
+#define TRI_STATIC_WORKSPACE_BYTES (64u << 20)
+int tri_compress_step_static(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                             const tri_select_params* sel, int32_t* keep, const uint32_t** status_out,
+                             void* stream);
+
 /* Calibration: per-query-head frequency statistics of one layer's captured query states;
  * replaces the RoPE inversion and the per-head means of scripts/calibrate.py:196-224
  * (helpers :38-98; same arithmetic as triattention/methods/pruning_utils.py:40-98).

@@ -70,6 +70,22 @@ def test_status_word_sits_at_one_offset_for_every_shape():
     assert len(seen) == 1
 
 
+def test_static_scratch_entry_rejects_oversized_steps_before_touching_the_device():
+    import ctypes as C
+    lib = _lib.load()
+    kv = _lib.KvLayout(num_layers=36, num_kv_heads=8, head_dim=128, block_size=16, kv_dtype=0,
+                       stride_block=16 * 8 * 128, stride_token=8 * 128, stride_head=128, k_layers=8, v_layers=8)
+    batch = _lib.Batch(num_seqs=16, max_seq_len=16384, max_budget=2048, block_table_pitch=1024, block_table=8,
+                       seq_lens=8, round_start=8, budgets=8)
+    sp = _lib.ScoreParams(num_score_heads=32, num_offsets=17, folded=16, omega=8, offsets=8)
+    sel = _lib.SelectParams(normalize=1, window_size=128, group_reduce=1)
+    assert lib.tri_workspace_bytes(C.byref(kv), C.byref(batch), C.byref(sp)) > _lib.STATIC_WORKSPACE_BYTES
+    rc = lib.tri_compress_step_static(C.byref(kv), C.byref(batch), C.byref(sp), C.byref(sel), 8, None, None)
+    assert rc == _lib.TRI_ERR_WORKSPACE and b"static array" in lib.tri_last_error()
+    header = (ROOT / "include" / "triattention_hip.h").read_text()
+    assert f"#define TRI_STATIC_WORKSPACE_BYTES ({_lib.STATIC_WORKSPACE_BYTES >> 20}u << 20)" in header
+
+
 # ---------------------------------------------------------------- settings
 def test_runtime_config_defaults_and_env():
     c = TriAttentionRuntimeConfig.from_env(environ={})

@@ -14,6 +14,7 @@ import os
 LIB_PATH = Path(os.environ.get("TRIATTN_HIP_LIBRARY") or Path(__file__).resolve().parent / "libtriattention_hip.so")
 
 ABI_VERSION = 4
+STATIC_WORKSPACE_BYTES = 64 << 20
 TRI_OK = 0
 TRI_ERR_INVALID_ARGUMENT = -1
 TRI_ERR_UNSUPPORTED = -2
@@ -28,7 +29,7 @@ EXPORTS = (
     "tri_abi_version", "tri_last_error", "tri_fold_stats", "tri_workspace_bytes", "tri_workspace_status_offset",
     "tri_score_paged",
     "tri_select", "tri_select_paged", "tri_select_path", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
-    "tri_compact_paged_full", "tri_compress_step", "tri_qstats_workspace_bytes", "tri_qstats",
+    "tri_compact_paged_full", "tri_compress_step", "tri_compress_step_static", "tri_qstats_workspace_bytes", "tri_qstats",
 )
 
 
@@ -108,6 +109,8 @@ def load() -> C.CDLL:
     lib.tri_compact_paged_full.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), P, I32, I32, P, U64, P]
     lib.tri_compress_step.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
                                       C.POINTER(SelectParams), P, P, U64, P]
+    lib.tri_compress_step_static.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                             C.POINTER(SelectParams), P, C.POINTER(C.c_void_p), P]
     lib.tri_qstats_workspace_bytes.argtypes = [I32, I32, I32]
     lib.tri_qstats_workspace_bytes.restype = U64
     lib.tri_qstats.argtypes = [P, I64, I64, P, P, I32, I32, I32, I32, I32, C.c_float, P, P, P, P, U64, P]

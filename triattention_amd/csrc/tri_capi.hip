@@ -8,6 +8,11 @@
 
 #include "tri_common.h"
 
+// Scratch of tri_compress_step_static: one copy per GPU, loaded with the code object.  In host
+// code this name is only a handle for hipGetSymbolAddress; the address kernels are given is
+// the one that call returns on the device in question.
+static __device__ __align__(256) unsigned char scratch[TRI_STATIC_WORKSPACE_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -132,6 +137,30 @@ struct ResidentGate {
 ResidentGate& resident_gate() {
   static ResidentGate gate;
   return gate;
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+struct StaticScratch {
+  static constexpr int kMaxDevices = 64;
+  std::mutex mutex;
+  void* ptr[kMaxDevices] = {};
+};
+int static_scratch(void** out) {
+  static StaticScratch st;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return launch_status(e, "hipGetDevice");
+  if (dev < 0 || dev >= StaticScratch::kMaxDevices) return fail(TRI_ERR_UNSUPPORTED, "device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(st.mutex);
+  if (!st.ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return launch_status(e, "hipGetSymbolAddress(scratch)");
+    if (!p || !is_aligned(p, 256)) return fail(TRI_ERR_WORKSPACE, "static scratch at %p is not 256-byte aligned", p);
+    st.ptr[dev] = p;
+  }
+  *out = st.ptr[dev];
+  return TRI_OK;
 }
 
 template <typename T>
@@ -464,6 +493,42 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
   // A resident kernel whose bounded wait expired leaves meaningless keep lists and a raised
   // status word: the compaction kernels look at that word and then leave the cache alone.
   c.guard = at<uint32_t>(workspace, w.status);
+  return launch_status(tri::launch_compact(c, s), "compact");
+}
+
+int tri_compress_step_static(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                             const tri_select_params* sel, int32_t* keep, const uint32_t** status_out,
+                             void* stream) {
+  int rc = check_layout(kv, true);
+  if (rc) return rc;
+  rc = check_batch(batch, true);
+  if (rc) return rc;
+  rc = check_score(kv, sp);
+  if (rc) return rc;
+  rc = check_select(sel);
+  if (rc) return rc;
+  if (!batch->round_start) return fail(TRI_ERR_INVALID_ARGUMENT, "round_start is NULL");
+  if (!batch->block_table) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_compress_step_static needs a block table");
+  if (!keep) return fail(TRI_ERR_INVALID_ARGUMENT, "keep is NULL");
+  const tri::Workspace w = plan(kv, batch, sp);
+  if ((uint64_t)w.total > (uint64_t)TRI_STATIC_WORKSPACE_BYTES)
+    return fail(TRI_ERR_WORKSPACE, "this step needs %lld bytes of scratch, the library's static array holds %llu; "
+                "use tri_compress_step with a workspace of the caller's", (long long)w.total,
+                (unsigned long long)TRI_STATIC_WORKSPACE_BYTES);
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  if (status_out) *status_out = at<uint32_t>(ws, w.status);
+  tri_select_params two_pass = *sel;
+  two_pass.no_resident = 1;   // the resident path chains its launches with an event it creates
+  hipStream_t s = (hipStream_t)stream;
+  rc = do_select_paged(kv, batch, sp, &two_pass, nullptr, keep, ws, w, s);
+  if (rc) return rc;
+  tri::CompactLaunch c{};
+  rc = fill_compact(kv, batch, keep, sel->layer_reduce < 0, sel->shared, c);
+  if (rc) return rc;
+  c.guard = at<uint32_t>(ws, w.status);
+  c.no_side_stream = 1;
   return launch_status(tri::launch_compact(c, s), "compact");
 }
 

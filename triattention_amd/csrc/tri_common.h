@@ -173,6 +173,7 @@ struct CompactLaunch {
   int Tmax;
   void* staging;       // full-permutation mode only
   const uint32_t* guard;   // optional: a device word; the kernels move nothing when it is non-zero
+  int no_side_stream;      // 1: fp8 scales follow the rows on the caller's stream (nothing is created)
 };
 hipError_t launch_compact(const CompactLaunch& a, hipStream_t s);
 

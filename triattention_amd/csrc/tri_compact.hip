@@ -528,7 +528,7 @@ hipError_t launch_compact(const CompactLaunch& a, hipStream_t s) {
   bool forked = false;
   SideStream& side = side_stream();
   std::unique_lock<std::mutex> lock(side.mutex, std::defer_lock);
-  if (a.has_scales) {
+  if (a.has_scales && !a.no_side_stream) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < SideStream::kMaxDevices &&
         hipStreamIsCapturing(s, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone) {

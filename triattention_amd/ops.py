@@ -539,3 +539,24 @@ def compress_step(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectCon
     _lib.check(lib.tri_compress_step(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss),
                                      _ptr(keep), ws.ptr, ws.bytes, _stream()))
     return keep, ws
+
+
+def compress_step_static(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, keep: torch.Tensor):
+    """``compress_step`` on the library's own static scratch: the call allocates nothing (``keep``
+    is the caller's, int32 [rows, max_budget]), always takes the score-then-select kernels, and
+    rejects steps whose scratch exceeds ``_lib.STATIC_WORKSPACE_BYTES``.  Calls that overlap
+    in time on one GPU share that scratch and race.  Returns the device address of the status word."""
+    lib = _lib.load()
+    _check_devices(kv, sc)
+    if batch.budgets is None or batch.block_table is None:
+        raise ValueError("compress_step_static needs budgets and block tables")
+    batch.check_capacity(kv.block_size)
+    rows = batch.num_seqs * (kv.num_layers if sel.layer_reduce is None else 1) * (1 if sel.shared else kv.num_kv_heads)
+    if (keep.numel() != rows * batch.max_budget or keep.dtype != torch.int32 or not keep.is_contiguous()
+            or keep.device != kv.device):
+        raise ValueError(f"keep must be a contiguous int32 tensor with {rows} x {batch.max_budget} entries")
+    sp, ss = sc.struct(), sel.struct()
+    status = C.c_void_p()
+    _lib.check(lib.tri_compress_step_static(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss),
+                                            _ptr(keep), C.byref(status), _stream()))
+    return int(status.value or 0)
