@@ -200,6 +200,10 @@ def test_inv_freq_from_model_config_and_native_format(tmp_path):
                                           '"original_max_position_embeddings": 8192}}')
     inv = stats_mod.resolve_inv_freq({}, 128, tmp_path)
     assert torch.equal(inv, rope.llama3_inv_freq(128, 5e5))
+    # ... and that is what transformers' own llama3 routine gives (fixture written from it)
+    gold = load_golden("llama3_inv_freq.pt")
+    assert torch.equal(inv, gold["llama3_inv_freq"])
+    assert torch.equal(rope.default_inv_freq(128, 5e5), gold["default_inv_freq"])
     assert torch.equal(stats_mod.resolve_inv_freq({"rope_theta": 1e6}, 64), rope.default_inv_freq(64, 1e6))
     with pytest.raises(ValueError):
         stats_mod.resolve_inv_freq({"inv_freq": [1.0, 0.5]}, 128)

@@ -167,6 +167,20 @@ def test_llama3_inv_freq_regimes():
     assert bool((got[mid] < base[mid]).all()) and bool((got[mid] > base[mid] / 8).all())
 
 
+def test_llama3_inv_freq_equals_transformers_golden():
+    """64 frequencies written by transformers' own llama3 routine (tests/golden/make_llama3_golden.py):
+    bit for bit, all three bands."""
+    from conftest import load_golden
+    gold = load_golden("llama3_inv_freq.pt")
+    got = orope.llama3_inv_freq(int(gold["head_dim"]), float(gold["rope_theta"]), float(gold["factor"]),
+                                float(gold["low_freq_factor"]), float(gold["high_freq_factor"]),
+                                int(gold["original_max_position_embeddings"]))
+    assert torch.equal(got, gold["llama3_inv_freq"])
+    assert torch.equal(orope.default_inv_freq(128, 5e5), gold["default_inv_freq"])
+    changed = gold["llama3_inv_freq"] != gold["default_inv_freq"]
+    assert 0 < int(changed.sum()) < 64 and float(gold["attention_scaling"]) == 1.0
+
+
 def test_fp8_dequant_closed_form():
     codes = torch.tensor([[[0.5, -1.5, 448.0, 0.0]]]).to(torch.float8_e4m3fn)
     scales = torch.tensor([[0.25]])

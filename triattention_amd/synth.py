@@ -1,6 +1,9 @@
 """Seeded synthetic workloads: paged KV pools, block tables and per-head Q statistics
 of the shapes the benchmark configurations name.  Used by the tests (small sizes, CPU
 generator, copied to the device) and by bench.py (full sizes, generated on the device).
+
+Measurement and test infrastructure, not part of the product path: nothing under
+``triattention_amd.core`` or ``triattention_amd.runtime`` imports this module.
 """
 from __future__ import annotations
 
