@@ -903,6 +903,37 @@ def test_resident_launches_on_two_streams_do_not_starve_each_other():
         assert torch.equal(keep, alone[i % 2][0]) and torch.equal(fin, alone[i % 2][1])
 
 
+@pytest.mark.parametrize("case", ["fewer_launches_planned_than_needed", "device_length_beyond_max_seq_len"])
+def test_host_lengths_that_disagree_with_the_device_raise_the_status_word(case, monkeypatch):
+    """A caller of the C ABI whose host copy of the lengths is stale: the planner sizes launches
+    and rows from the host values, the kernels read the device values.  Sequences that would not
+    be scored (or lie beyond the planned rows) raise the status word (3), every workgroup still
+    runs to its end inside the planned bounds, and the step's compaction leaves the cache alone."""
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    if case == "fewer_launches_planned_than_needed":
+        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", "16")
+        w = small(seq_lens=(3000,) * 8, num_q_heads=32, num_kv_heads=8, budget=128, index=51)
+    else:
+        w = small(seq_lens=(1000, 700), num_q_heads=32, num_kv_heads=8, budget=128, index=52)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    keep, ws = ops.compress_step(kv, batch, sc, sel)            # lengths agree: a clean step
+    assert ws.status() == 0
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    pristine = [c.clone() for c in caches]
+    if case == "fewer_launches_planned_than_needed":
+        for i in range(1, w.num_seqs):
+            batch._lens_host[i] = 100          # the host believes seven sequences are short: one launch planned
+    else:
+        batch.seq_lens[1] = 1500               # the device holds more than max_seq_len = 1000
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    keep, ws = ops.compress_step(kv, batch, sc, sel)
+    assert ws.status() == 3
+    for c, p in zip(caches, pristine):
+        assert torch.equal(c.view(torch.int16), p.view(torch.int16))
+
+
 @pytest.mark.parametrize("kv_dtype", ["bf16", "fp8"])
 def test_compress_step_replays_from_a_hip_graph(kv_dtype):
     """The launch sequence of a step (no allocation, no synchronisation, no memset nodes)

@@ -33,6 +33,8 @@ __device__ __forceinline__ uint4 load_chunk(const char* p) {
   const cu32x4 v = *(GlobalChunkIn)(uintptr_t)p;
   return uint4{v.x, v.y, v.z, v.w};
 }
+// (Non-temporal stores here are slower: 1.84 against 1.74 ms for the 16 x 16384-token step's
+// compaction; non-temporal loads change nothing.)
 __device__ __forceinline__ void store_chunk(char* p, const uint4& v) {
   *(GlobalChunk)(uintptr_t)p = cu32x4{v.x, v.y, v.z, v.w};
 }
@@ -106,6 +108,7 @@ __global__ __launch_bounds__(kOrderedThreads) void compact_kernel(CompactArgs a)
   int k = a.budgets[b];
   const int T = a.seq_lens[b];
   if (k > T) k = T;
+  if (k > a.max_budget) k = a.max_budget;   // keep rows hold max_budget entries, whatever the device array says
   if (k <= 0) return;
   const int32_t* keep =
       a.keep + ((int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * all_lists + list0) * a.max_budget;
@@ -235,6 +238,7 @@ __global__ __launch_bounds__(kCompactThreads) void compact_bulk_kernel(CompactAr
   int k = a.budgets[b];
   const int T = a.seq_lens[b];
   if (k > T) k = T;
+  if (k > a.max_budget) k = a.max_budget;   // keep rows hold max_budget entries, whatever the device array says
   if (k <= 0) return;
   const int lists = a.shared ? 1 : a.Hkv;
   const int chunks_per_entry = a.heads_per_slot * a.chunks_per_row;
@@ -321,6 +325,7 @@ __global__ __launch_bounds__(256) void compact_scales_kernel(ScaleArgs a) {
   int k = a.budgets[b];
   const int T = a.seq_lens[b];
   if (k > T) k = T;
+  if (k > a.max_budget) k = a.max_budget;   // keep rows hold max_budget entries, whatever the device array says
   if (k <= 0) return;
   const int rows = a.shared ? 1 : a.Hkv;
   const int32_t* keep = a.keep + (int64_t)(a.keep_per_layer ? (b * a.L + l) : b) * rows * a.max_budget;
@@ -384,6 +389,7 @@ __global__ __launch_bounds__(256) void permute_to_staging_kernel(FullArgs f) {
   const int T = a.seq_lens[b];
   int k = a.budgets[b];
   if (k > T) k = T;
+  if (k > a.max_budget) k = a.max_budget;   // keep rows hold max_budget entries, whatever the device array says
   const int n0 = blockIdx.x * 256;
   if (n0 >= T || k <= 0 || k >= T) return;
   const int rows = a.shared ? 1 : a.Hkv;
@@ -427,6 +433,7 @@ __global__ __launch_bounds__(256) void staging_to_cache_kernel(FullArgs f) {
   const int T = a.seq_lens[b];
   int k = a.budgets[b];
   if (k > T) k = T;
+  if (k > a.max_budget) k = a.max_budget;   // keep rows hold max_budget entries, whatever the device array says
   const int n0 = blockIdx.x * 256;
   if (n0 >= T || k <= 0 || k >= T) return;
   const int32_t* bt = a.block_table + (int64_t)b * a.block_table_pitch;

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kFusedThreads) void fused_select_kernel(FusedArgs a
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int b, tile;
   if (!locate_workgroup(a, a.tiles_per_seq, 1, reinterpret_cast<int*>(lds), b, tile)) return;
-  const int T = a.seq_lens[b];
+  const int T = checked_seq_len(a.seq_lens, b, a.Tmax, a.status);
   const int n0 = tile * a.tile_tokens;
   if (n0 >= T) return;
   const int n1 = min(n0 + a.tile_tokens, T);
@@ -383,11 +383,12 @@ hipError_t launch_fused_t(FusedArgs& k, int seqs_per_launch, int resident, int B
   // launches on the device (the host does not know the individual lengths); the host
   // issues as many launches as the worst case needs, surplus ones find no work.
   k.packed = 1;
+  const int launches = ceil_div(B, seqs_per_launch);
   hipLaunchKernelGGL(fused_pack_kernel, dim3(1), dim3(256), 0, s, k.seq_lens, B, k.tile_tokens, 1, resident,
-                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base));
+                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base), launches, k.Tmax,
+                     k.status);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const int launches = ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
     hipLaunchKernelGGL((fused_select_kernel<DT, IL, TW, SL>), dim3(resident), dim3(kFusedThreads), lds, s, k);

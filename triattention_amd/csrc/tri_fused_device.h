@@ -76,9 +76,14 @@ __device__ __forceinline__ bool locate_workgroup(const FusedArgs& a, int wgs_per
 // into the first of the eight most recently opened launches that still has room.  No
 // launch holds fewer sequences than capacity / (largest sequence) allows, so the number of
 // launches never exceeds what the host provides for.  One workgroup.
+// `launches` is how many launches the host will issue and `Tmax` the length it sized everything
+// for: a sequence that lands in a later launch (the host planned with other lengths than the
+// device holds) or is longer than Tmax would never be scored, so the status word is raised (3)
+// and the step's compaction, which looks at that word, leaves the cache alone.
 __global__ __launch_bounds__(256) void fused_pack_kernel(const int32_t* seq_lens, int B, int tile_tokens,
                                                          int wg_mult, int capacity, int32_t* seq_launch,
-                                                         int32_t* seq_wg_base) {
+                                                         int32_t* seq_wg_base, int launches, int Tmax,
+                                                         uint32_t* status) {
   constexpr int kMaxSorted = 4096;
   __shared__ int order[kMaxSorted];
   const bool sorted = B <= kMaxSorted;
@@ -116,7 +121,20 @@ __global__ __launch_bounds__(256) void fused_pack_kernel(const int32_t* seq_lens
     seq_launch[s] = first + pick;
     seq_wg_base[s] = used[pick];
     used[pick] += n;
+    if (first + pick >= launches || seq_lens[s] > Tmax) atomicExch(status, 3u);
   }
+}
+
+// Length of sequence b as the kernels use it.  The host sized grids, rings and output rows for
+// Tmax; a device length beyond it (a caller whose host copy was stale) is cut there and raises
+// the status word (3), so nothing is read or written out of range and the results are flagged.
+__device__ __forceinline__ int checked_seq_len(const int32_t* seq_lens, int b, int Tmax, uint32_t* status) {
+  int T = seq_lens[b];
+  if (T > Tmax) {
+    if (threadIdx.x == 0) atomicExch(status, 3u);
+    T = Tmax;
+  }
+  return T;
 }
 
 __device__ __forceinline__ unsigned long long xchg_load(const unsigned long long* p) {
@@ -164,7 +182,7 @@ __device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, in
   const long long t_begin = wall_clock64();
   if (a.spin_ticks < 0 && !aborted) {   // set by the host to exercise the failure path: give up without waiting
     aborted = true;
-    if (lane == 0) atomicExch(a.status, 1u);
+    if (lane == 0) atomicCAS(a.status, 0u, 1u);
   }
   for (int base = 0; base < items; base += 64) {
     const int item = base + lane;
@@ -184,7 +202,7 @@ __device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, in
         if (wall_clock64() - t_begin > a.spin_ticks ||
             __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
           aborted = true;
-          if (lane == 0) atomicExch(a.status, 1u);
+          if (lane == 0) atomicCAS(a.status, 0u, 1u);   // keeps the reason another workgroup gave (2, 3)
         }
         __builtin_amdgcn_s_sleep(4);
       }

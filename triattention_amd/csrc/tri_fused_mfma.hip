@@ -293,7 +293,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   if (!locate_workgroup(a, a.HC * a.tiles_per_seq, a.HC, reinterpret_cast<int*>(lds), b, within)) return;
   const int chunk = within % a.HC;
   const int tile = within / a.HC;
-  const int T = a.seq_lens[b];
+  const int T = checked_seq_len(a.seq_lens, b, a.Tmax, a.status);
   const int n0 = tile * a.tile_tokens;
   if (n0 >= T) return;
   const int n1 = min(n0 + a.tile_tokens, T);
@@ -760,11 +760,12 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, const LaunchShape& sha
   // launches on the device (the host does not know the individual lengths); the host
   // issues as many launches as the worst case needs, surplus ones find no work.
   k.packed = 1;
+  const int launches = known_launches > 0 ? known_launches : ceil_div(B, seqs_per_launch);
   hipLaunchKernelGGL(fused_pack_kernel, dim3(1), dim3(256), 0, s, k.seq_lens, B, k.tile_tokens, k.HC, resident,
-                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base));
+                     const_cast<int32_t*>(k.seq_launch), const_cast<int32_t*>(k.seq_wg_base), launches, k.Tmax,
+                     k.status);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const int launches = known_launches > 0 ? known_launches : ceil_div(B, seqs_per_launch);
   for (int i = 0; i < launches; ++i) {
     k.launch_idx = i;
     hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>), dim3(resident), dim3(W * kWave), lds, s, k, bmat);

@@ -227,7 +227,7 @@ constexpr int kTopkThreads = 1024;
 __global__ __launch_bounds__(kTopkThreads) void topk_rows_kernel(const float* scores, int64_t row_pitch,
                                                                 const int32_t* row_lens,
                                                                 const int32_t* row_ks, int rows_per_entry,
-                                                                int32_t* keep, int keep_pitch) {
+                                                                int32_t* keep, int keep_pitch, int max_len) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t scan[256];
   __shared__ uint32_t sh_prefix, sh_remaining;
@@ -236,8 +236,10 @@ __global__ __launch_bounds__(kTopkThreads) void topk_rows_kernel(const float* sc
 
   const int row = blockIdx.x;
   const int entry = row / rows_per_entry;
-  const int T = row_lens[entry];
-  int k = row_ks[entry];
+  // Lengths and budgets live on the device; the host sized rows for max_len scores and
+  // keep_pitch indices, and neither is ever exceeded whatever the device arrays say.
+  const int T = min(row_lens[entry], max_len);
+  int k = min(row_ks[entry], keep_pitch);
   if (k > T) k = T;
   if (k <= 0 || T <= 0) return;
   const float* x = scores + (int64_t)row * row_pitch;
@@ -330,15 +332,17 @@ template <int VPT>
 __global__ __launch_bounds__(kTopkThreads) void topk_rows_reg_kernel(const float* scores, int64_t row_pitch,
                                                                     const int32_t* row_lens,
                                                                     const int32_t* row_ks, int rows_per_entry,
-                                                                    int32_t* keep, int keep_pitch) {
+                                                                    int32_t* keep, int keep_pitch, int max_len) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t sh_prefix, sh_remaining;
   __shared__ uint32_t wave_tot[kTopkThreads / 64];
 
   const int row = blockIdx.x;
   const int entry = row / rows_per_entry;
-  const int T = row_lens[entry];
-  int k = row_ks[entry];
+  // Lengths and budgets live on the device; the host sized rows for max_len scores and
+  // keep_pitch indices, and neither is ever exceeded whatever the device arrays say.
+  const int T = min(row_lens[entry], max_len);
+  int k = min(row_ks[entry], keep_pitch);
   if (k > T) k = T;
   if (k <= 0 || T <= 0) return;
   const float* x = scores + (int64_t)row * row_pitch;
@@ -449,16 +453,16 @@ hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows
   if (num_rows <= 0) return hipSuccess;
   if (max_len > 0 && max_len <= 8 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<8>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
   else if (max_len > 0 && max_len <= 16 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<16>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
   else if (max_len > 0 && max_len <= 32 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<32>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
   else
     hipLaunchKernelGGL(topk_rows_kernel, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
   return hipGetLastError();
 }
 

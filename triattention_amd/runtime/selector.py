@@ -158,14 +158,18 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                               block_tables=tables, prefill_lens=[prefill_len])
         sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
                                protect_prefill=bool(protect_prefill and prefill_len > 0),
-                               group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared)
+                               group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared,
+                               allow_resident=holder.get("resident_ok", True))
         try:
             resident = ops.select_path(kv, batch, sc, sel) != "two_pass"   # (a single request: only when forced)
             keep, _, ws = ops.select_paged(kv, batch, sc, sel)
             if resident and ws.status() != 0:
                 # A wait inside the resident kernel expired (or a coefficient did not fit its operand
                 # type): the keep lists mean nothing.  Nothing has been moved yet; score again on the
-                # kernels that do not wait for each other.
+                # kernels that do not wait for each other, and stay on them: whatever starved the
+                # launch (a shared or masked GPU) or overflowed (this model's statistics) is still
+                # there at the next step, and every failed launch costs its full wait limit.
+                holder["resident_ok"] = False
                 sel.allow_resident = False
                 keep, _, ws = ops.select_paged(kv, batch, sc, sel, ws)
         except Exception as exc:
@@ -288,13 +292,14 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                               prefill_lens=guards)
         sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
                                protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
-                               allow_resident=bool(allow_resident))
+                               allow_resident=bool(allow_resident) and holder.get("resident_ok", True))
         resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
         try:
             keep, ws = ops.compress_step(kv, batch, sc, sel)
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
         if resident and ws.status() != 0:
+            holder["resident_ok"] = False     # later steps of this selector go straight to the two-pass kernels
             raise ResidentLaunchFailed("a wait inside the resident kernel expired; the caches were left untouched")
         h = kv.num_kv_heads
         keep = keep.to(torch.long)           # one conversion; the per-request results are views
