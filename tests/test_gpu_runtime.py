@@ -407,3 +407,108 @@ def test_dense_compressor_against_oracle(tmp_path):
     with pytest.raises(ValueError):
         TriAttentionCompressor(cfg).compress(torch.zeros(2, h, 600, d, dtype=torch.bfloat16, device=DEV),
                                              torch.zeros(2, h, 600, d, dtype=torch.bfloat16, device=DEV))
+
+
+def test_scheduler_and_worker_bookkeeping_around_the_hook_over_a_decode_loop(tmp_path):
+    """A stand-in engine (block pool, per-group block manager, worker block table) drives the hook
+    through ``engine_glue`` for 80 decode steps of two requests: the scheduler's and the worker's
+    block lists stay equal, every freed block returns to the pool exactly once, the request is
+    compressed again every ``divide_length`` tokens, and the lengths the attention inputs would get
+    equal the scheduler's effective lengths."""
+    import numpy as np
+    from helpers import build_inputs
+    from triattention_amd import synth
+    from triattention_amd.runtime import RequestStateStore, engine_glue as eg
+    NS = types.SimpleNamespace
+    w = synth.Workload(name="t", num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128, seq_lens=(300, 140),
+                       budget=100, block_size=16, window_size=12, rope_theta=1e6, index=61, pool_occupancy=0.5)
+    inp = build_inputs(w)
+    _write_stats(tmp_path / "s.pt", inp["qc"], inp["qa"], inp["omega"], w.head_dim)
+    cfg = TriAttentionRuntimeConfig(kv_budget=100, divide_length=16, window_size=12, sparse_stats_path=tmp_path / "s.pt",
+                                    log_decisions=False)
+    bs = w.block_size
+    caches = [c.to(DEV) for c in inp["caches"]]
+    used = {int(x) for tb in inp["tables"] for x in tb}
+    free = [b for b in range(w.pool_blocks) if b not in used]
+    freed_log = []
+
+    class Pool:
+        def free_blocks(self, blocks):
+            for blk in blocks:
+                assert blk.block_id not in free, "a block was freed twice"
+                free.append(blk.block_id)
+                freed_log.append(blk.block_id)
+
+    rids = ["r0", "r1"]
+    manager = NS(req_to_blocks={rid: [NS(block_id=int(x), block_hash=None) for x in inp["tables"][i]]
+                                for i, rid in enumerate(rids)},
+                 num_cached_block={rid: len(inp["tables"][i]) for i, rid in enumerate(rids)}, block_pool=Pool())
+    sched_reqs = {rid: NS(num_computed_tokens=t, num_prompt_tokens=t) for rid, t in zip(rids, w.seq_lens)}
+    worker_reqs = {rid: NS(num_computed_tokens=t, block_ids=([int(x) for x in inp["tables"][i]],))
+                   for i, (rid, t) in enumerate(zip(rids, w.seq_lens))}
+    rows = NS(num_blocks_per_row=np.array([len(tb) for tb in inp["tables"]]))
+    runner = NS(requests=worker_reqs, kv_caches=caches, cache_config=NS(block_size=bs),
+                input_batch=NS(block_table=rows, req_id_to_index={"r0": 0, "r1": 1}))
+    install_runner_compression_hook(runner, cfg)
+    store = RequestStateStore()
+    runner._triattention_state_store = store
+    executor = RunnerHookCompressionExecutor(runner)
+    glue = eg.SchedulerCompressionGlue(cfg)
+    new = [NS(req_id=rid, num_computed_tokens=0, num_prompt_tokens=t) for rid, t in zip(rids, w.seq_lens)]
+    compressions = {rid: [] for rid in rids}
+    true_len = dict(zip(rids, w.seq_lens))        # tokens really held in the cache
+    for step in range(80):
+        # -- scheduler: one token per request, a block when the cache needs one more
+        for i, rid in enumerate(rids):
+            if (true_len[rid] + 1 + bs - 1) // bs > len(manager.req_to_blocks[rid]):
+                blk = free.pop(0)
+                manager.req_to_blocks[rid].append(NS(block_id=blk, block_hash=None))
+                worker_reqs[rid].block_ids[0].append(blk)
+                rows.num_blocks_per_row[i] += 1
+        out = NS(num_scheduled_tokens={rid: 1 for rid in rids}, scheduled_new_reqs=new if step == 0 else [],
+                 finished_req_ids=set(),
+                 scheduled_cached_reqs=NS(req_ids=list(rids), num_computed_tokens=[sched_reqs[r].num_computed_tokens for r in rids]))
+        signals = glue.after_schedule(out, sched_reqs)
+        # -- worker
+        eg.register_new_requests(state_store=store, scheduler_output=out, protect_prefill=cfg.protect_prefill)
+        _, signals = eg.consume_runner_signals(state_store=store, scheduler_output=out, last_step=step)
+        events = eg.execute_runner_compression_actions(executor=executor, state_store=store, scheduler_output=out,
+                                                       signals=signals, strict_no_downgrade=True)
+        eg.apply_worker_block_reclaim_events(base_runner=runner, events=events)
+        seq_bases, pos_deltas, _, _ = eg.build_effective_sparse_overrides(base_runner=runner, state_store=store,
+                                                                          scheduler_output=out, compression_events=events)
+        for e in events:
+            if e["status"] == "applied":
+                rid = e["req_id"]
+                compressions[rid].append((sched_reqs[rid].num_computed_tokens, e["cache_len_after"]))
+                assert e["details"]["effective_tokens_before"] == true_len[rid]
+                assert e["cache_len_after"] == 100 and e["block_reclaim"]["groups"][0]["gid"] == 0
+                true_len[rid] = 100
+        for i, rid in enumerate(rids):
+            st = store.get(rid)
+            if st is not None and st.compression_count > 0:
+                # the attention inputs of this step: cached length before its token, and the shift of
+                # the slot positions against the absolute ones
+                assert seq_bases[i] == true_len[rid], (step, rid)
+                assert pos_deltas[i] == true_len[rid] - sched_reqs[rid].num_computed_tokens
+            else:
+                assert not seq_bases or i not in seq_bases
+            worker_reqs[rid].num_computed_tokens += 1
+            sched_reqs[rid].num_computed_tokens += 1
+            true_len[rid] += 1
+        # -- scheduler again: the events of this step
+        glue.apply_compression_events(events, sched_reqs, [manager], bs)
+        for i, rid in enumerate(rids):
+            assert [b.block_id for b in manager.req_to_blocks[rid]] == worker_reqs[rid].block_ids[0], (step, rid)
+            assert rows.num_blocks_per_row[i] == len(worker_reqs[rid].block_ids[0])
+            assert len(worker_reqs[rid].block_ids[0]) * bs >= true_len[rid]
+    torch.cuda.synchronize()
+    # r0 (300 tokens) is due at once and then every 16 tokens; r1 (140) likewise
+    for rid, t in zip(rids, w.seq_lens):
+        ncts = [n for n, _ in compressions[rid]]
+        assert ncts[0] == t and len(ncts) >= 4, (rid, ncts)
+        assert all(15 <= b - a <= 17 for a, b in zip(ncts, ncts[1:])), (rid, ncts)      # every divide_length tokens
+    assert freed_log
+    live = [b.block_id for rid in rids for b in manager.req_to_blocks[rid]]
+    assert len(live) == len(set(live)) and not set(live) & set(free)
+    assert len(live) + len(free) == w.pool_blocks

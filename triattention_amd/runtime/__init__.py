@@ -10,6 +10,9 @@ from .kv_compaction import (build_keep_token_indices, compact_request_kv_in_plac
 from .models import (TRITON_SCORING_REQUIRED_MARKER, CompressionPlanner, CompressionSignal, KeepPlan,
                      PlacementPlan, ReclaimEvent, ReclaimGroup, RequestCompressionState, RequestStateStore)
 from .selector import build_triattention_selector
+from .engine_glue import (EffectiveCacheLenTracker, SchedulerCompressionGlue, apply_worker_block_reclaim_events,
+                          build_effective_sparse_overrides, consume_runner_signals,
+                          execute_runner_compression_actions)
 
 # Public alias, as in the reference's runtime package.
 TriAttentionConfig = TriAttentionRuntimeConfig
@@ -22,5 +25,7 @@ __all__ = [
     "gather_request_k_dense_range", "gather_request_kv_dense", "register_kv_layout_axis_hint",
     "TRITON_SCORING_REQUIRED_MARKER", "CompressionPlanner", "CompressionSignal", "KeepPlan", "PlacementPlan",
     "ReclaimEvent", "ReclaimGroup", "RequestCompressionState", "RequestStateStore",
-    "build_triattention_selector",
+    "build_triattention_selector", "EffectiveCacheLenTracker", "SchedulerCompressionGlue",
+    "apply_worker_block_reclaim_events", "build_effective_sparse_overrides", "consume_runner_signals",
+    "execute_runner_compression_actions",
 ]
