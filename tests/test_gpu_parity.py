@@ -702,6 +702,55 @@ RESIDENT_CASES.update({
 })
 
 
+@pytest.mark.parametrize("case", ["one_request_36_layers", "one_request_split_by_layer", "one_request_uneven_layer_groups",
+                                  "three_requests_split", "sixteen_requests"])
+def test_steady_state_step_matches_oracle(case, monkeypatch):
+    """The step a long generation repeats every 128 tokens: budget + 128 = 2176 cached tokens, budget
+    2048, Qwen3-8B head shape, against the CPU oracle: kept sets, and K/V compacted bit for bit.
+    One request (what the reference's runner hands over, runtime/runner_compression_actions.py:24)
+    does not fill the chip with whole-model workgroups; the resident kernel then cuts the layers
+    into groups.  Sixteen requests run as whole-model workgroups."""
+    layers, seqs, env = {
+        "one_request_36_layers": (36, 1, {}),                                   # the library's own choice
+        "one_request_split_by_layer": (4, 1, {"TRIATTN_RESIDENT_KERNEL": "mfma", "TRIATTN_RESIDENT_LAYER_SPLIT": "1"}),
+        "one_request_uneven_layer_groups": (5, 1, {"TRIATTN_RESIDENT_KERNEL": "mfma", "TRIATTN_RESIDENT_LAYER_SPLIT": "1",
+                                                   "TRIATTN_RESIDENT_WORKGROUPS": "12"}),    # groups of 2, 2, 1 layers
+        "three_requests_split": (6, 3, {"TRIATTN_RESIDENT_KERNEL": "mfma", "TRIATTN_RESIDENT_LAYER_SPLIT": "1",
+                                        "TRIATTN_RESIDENT_WORKGROUPS": "40"}),
+        "sixteen_requests": (4, 16, {}),
+    }[case]
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    w = synth.Workload("steady", layers, 32, 8, 128, (2176,) * seqs, 2048, index=70 + layers)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    _, fin, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    keep, ws = ops.compress_step(kv, batch, sc, sel, ws)
+    assert ws.status() == 0
+    keep, fin = keep.cpu().long(), fin.cpu()
+    h, k, t = w.num_kv_heads, w.budget, 2176
+    swapped = 0
+    for b in range(seqs):
+        oraw = oracle_raw(w, inp, b, t)
+        want, ofin = osel.group_keep_per_head(oraw, h, k, window_size=w.window_size,
+                                              chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
+        finite = torch.isfinite(ofin)
+        scale = float(ofin[finite].abs().max())
+        dfin = fin[b * h:(b + 1) * h, :t]
+        assert torch.equal(torch.isfinite(dfin), finite)
+        assert float((dfin[finite] - ofin[finite]).abs().max()) <= selection_score_tol(oraw) * scale
+        got = keep[b * h:(b + 1) * h, :k]
+        swapped += assert_keep_matches(got, want, ofin, k, tie_tol=KEEP_TIE_TOL * scale)
+        blk, off = ocp.token_slots(inp["tables"][b], w.block_size, torch.arange(k))
+        for l in range(0, layers, max(1, layers // 4)):
+            ref = inp["caches"][l].clone()
+            ocp.compact_per_head(ref, inp["tables"][b], w.block_size, got, t, full_permutation=False)
+            assert torch.equal(caches[l].cpu()[:, blk, off].view(torch.int16), ref[:, blk, off].view(torch.int16)), (b, l)
+    record_swaps(f"steady_state_vs_oracle:{case}", swapped, seqs * h * k)
+
+
 # Named cases in which the two paths keep different indices at near-ties (scores within
 # KEEP_TIE_TOL of the threshold), and how many of the case's kept indices: 16 sequences x heads x
 # 256 kept indices each, two of which sit that close to their threshold.  Everywhere else: none.

@@ -268,7 +268,16 @@ def test_batch_hook_equals_the_hook_called_request_by_request(tmp_path, monkeypa
     for _, _, _, _, signals in (one, two):
         signals["r3"] = _signal(req_id="r3", estimated_cache_len=514, prefill_len=40, protect_prefill=True)
     runner, reqs, caches, sched, signals = one
+    from triattention_amd.runtime import hook as hook_mod
+    monkeypatch.setattr(hook_mod, "SINGLE_REQUEST_IN_ONE_CALL", False)     # the reference-shaped pipeline, request by request
     want = {rid: RunnerHookCompressionExecutor(runner).execute(rid, sig, sched) for rid, sig in signals.items()}
+    monkeypatch.setattr(hook_mod, "SINGLE_REQUEST_IN_ONE_CALL", True)
+    three = _fake_runner(w, inp, tmp_path)
+    three[4]["r3"] = signals["r3"]
+    fused_single = {rid: RunnerHookCompressionExecutor(three[0]).execute(rid, sig, three[3]) for rid, sig in three[4].items()}
+    assert fused_single == want                                             # ... equals the one-call path per request
+    for a, b in zip(caches, three[2]):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     runner2, reqs2, caches2, sched2, signals2 = two
     got = RunnerHookCompressionExecutor(runner2).execute_batch(signals2, sched2)
     torch.cuda.synchronize()

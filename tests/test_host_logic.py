@@ -529,16 +529,25 @@ def test_batch_hook_groups_requests_and_falls_back(monkeypatch):
         first = reqs[rid].block_ids[0][0]
         assert reqs[rid].block_ids == ([first, first + 1],)
         assert out[rid].details["reclaimed_block_count"] == 8
-    # the same requests one by one give the same dictionaries
+    # the same requests one by one through the reference-shaped pipeline (selector callable, then the
+    # compaction function per layer) give the same dictionaries
+    monkeypatch.setattr(hook_mod, "SINGLE_REQUEST_IN_ONE_CALL", False)
     runner1, reqs1, sig1, sched1 = runner_with([40, 6, 30, 17])
     sig1["r2"] = sig["r2"]
     one = {rid: RunnerHookCompressionExecutor(runner1).execute(rid, s_, sched1) for rid, s_ in sig1.items()}
     assert one == out and calls["single"] == [40, 30, 17] and moved == [40, 30, 17]
-    # a single candidate does not need the batched call
+    # ... where a single candidate of a batch call takes that pipeline too
     calls["batch"].clear(); calls["single"].clear(); moved.clear()
     runner2, reqs2, sig2, sched2 = runner_with([40, 5])
     out2 = RunnerHookCompressionExecutor(runner2).execute_batch(sig2, sched2)
     assert out2["r0"].applied and not calls["batch"] and calls["single"] == [40]
+    # by default a single request takes the one-call launch sequence, from either entry point
+    monkeypatch.setattr(hook_mod, "SINGLE_REQUEST_IN_ONE_CALL", True)
+    calls["batch"].clear(); calls["single"].clear(); moved.clear()
+    runner2b, reqs2b, sig2b, sched2b = runner_with([40, 5])
+    out2b = RunnerHookCompressionExecutor(runner2b).execute_batch(sig2b, sched2b)
+    one2b = RunnerHookCompressionExecutor(runner_with([40, 5])[0]).execute("r0", sig2b["r0"], sched2b)
+    assert out2b["r0"] == out2["r0"] == one2b and len(calls["batch"]) == 2 and not calls["single"] and not moved
     # failed resident launch: the group is repeated in one batched call without the resident
     # kernel; nothing goes through the one-by-one path and the environment is left alone
     calls["batch"].clear(); calls["single"].clear(); moved.clear()

@@ -111,9 +111,14 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   const bool paged = b->block_table != nullptr;
   const int resident = f_off ? 0 : tri::fused_resident_workgroups();
   tri::FusedPlan fused{};
+  // Small batches are cut by layers as well (TRIATTN_RESIDENT_LAYER_SPLIT=0 switches that off, =1
+  // switches it on where the kernel was forced, which otherwise keeps whole-model workgroups).
+  const char* split_env = getenv("TRIATTN_RESIDENT_LAYER_SPLIT");
+  const bool split = split_env ? strcmp(split_env, "0") != 0 : !f_mfma;
   if (want_mfma)
     fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
-                                 sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype, b->seq_lens_host);
+                                 sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype, b->seq_lens_host,
+                                 kv->num_layers, split);
   if (!fused.eligible && !f_mfma)
     fused = tri::plan_fused(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged, sp->aggregation,
                             b->max_seq_len, resident, f_valu);
@@ -259,7 +264,14 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.status = at<uint32_t>(ws, w.status);
   a.pack = at<int32_t>(ws, w.pack);
   a.fin = fin ? fin : at<float>(ws, w.fin);
+  // Partial results of a layer-split launch live where the two-pass path keeps its raw scores
+  // ([B][L][Tmax][A] floats, never smaller than [groups][B][Hkv][Tmax]).
+  a.fin_part = at<float>(ws, w.raw);
   a.plan = w.fused;
+  // Nobody asked for the selection scores themselves: the groups' partial rows go straight to the
+  // top-k, which adds them while it loads (one launch less).
+  const bool split = w.fused.eligible == 2 && w.fused.layer_groups > 1;
+  a.skip_layer_reduce = split && !fin && keep && batch->max_seq_len <= tri::topk_register_row_limit();
   a.bmat = at<char>(ws, w.bmat);
   if (w.fused.eligible == 2) {
     // The preparation launch writes one 16-byte entry per (sequence, layer, KV head, group of four
@@ -297,6 +309,11 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
     }
   }
   if (!keep) return TRI_OK;   // selection scores only
+  if (a.skip_layer_reduce)
+    return launch_status(tri::launch_topk_rows(a.fin_part, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, a.Tmax,
+                                               keep, batch->max_budget, s, w.fused.layer_groups,
+                                               (int64_t)a.B * a.Hkv * a.Tmax, sel->layer_reduce == TRI_REDUCE_MAX),
+                         "topk_rows");
   return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, a.Tmax, keep,
                                              batch->max_budget, s),
                        "topk_rows");

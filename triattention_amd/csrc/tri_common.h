@@ -34,14 +34,19 @@ struct FusedPlan {
   int bs_shift;
   int waves;            // matrix-core kernel: waves per workgroup (8, or 4 with two workgroups per CU)
   int launches;         // matrix-core kernel, several launches: how many (0: the worst case for the longest sequence)
+  int layer_groups;     // matrix-core kernel, a batch too small to fill the chip with whole-model workgroups: the
+                        // layers are cut into this many groups, one workgroup per (sequence, group, tile)
+  int layers_per_group;
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();
 // any_fill: plan the resident kernel even for a launch that would leave most CUs idle.
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                      int resident, bool any_fill);
+// L > 0 and split_layers: a single launch that would leave most of the chip idle is cut by layers too.
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens = nullptr);
+                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens = nullptr,
+                          int L = 0, bool split_layers = false);
 
 // Scratch carved out of the caller's workspace.  All offsets in bytes, 256-aligned.
 struct Workspace {
@@ -126,9 +131,13 @@ struct SelectLaunch {
 };
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
 hipError_t launch_clear_status(uint32_t* status, hipStream_t s);
+// groups > 1: row r is the sum (group_max: maximum) of `groups` partial rows group_stride floats apart,
+// added while loading (rows of at most topk_register_row_limit() elements).
 hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
                             const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry, int max_len,
-                            int32_t* keep, int keep_pitch, hipStream_t s);
+                            int32_t* keep, int keep_pitch, hipStream_t s, int groups = 1, int64_t group_stride = 0,
+                            int group_max = 0);
+int topk_register_row_limit();
 
 struct FusedLaunch {
   int B, L, Hkv, D, block_size, kv_dtype, rope_style, A, G, Tmax;
@@ -148,6 +157,8 @@ struct FusedLaunch {
   int32_t* pack;                 // workspace
   void* bmat;                    // workspace (matrix-core kernel)
   float* fin;                    // [B*Hkv][Tmax]
+  float* fin_part;               // workspace: [layer groups][B*Hkv][Tmax] (layer-split launches of the matrix-core kernel)
+  int skip_layer_reduce;         // 1: leave the groups' partial rows in fin_part (the top-k adds them while loading)
   FusedPlan plan;
 };
 // Limit of the resident kernels' waits on other workgroups, in ticks of the 100 MHz wall

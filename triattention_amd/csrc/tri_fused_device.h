@@ -31,6 +31,11 @@ struct FusedArgs {
   const int32_t* seq_launch;
   const int32_t* seq_wg_base;
   int packed, launch_idx;
+  // Layers cut into groups (one launch only): num_seqs counts (sequence, group) pairs, a workgroup
+  // runs the layers of its group and leaves its sum (or maximum) over them in fin_part
+  // [group][num sequences * Hkv][Tmax]; fused_layer_reduce_kernel combines the groups.
+  int layer_groups, layers_per_group;
+  float* fin_part;
 };
 
 // Which (sequence, workgroup within the sequence) this workgroup serves; false: none.
@@ -160,6 +165,20 @@ __device__ __forceinline__ void* uniform_ptr(const void* p) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+}
+
+// Selection scores from the per-layer-group partial results of a layer-split launch: groups
+// combined in group order, then the division by the layer count of a mean over layers.
+__global__ __launch_bounds__(256) void fused_layer_reduce_kernel(const float* part, float* fin, int64_t count,
+                                                                 int groups, int layer_reduce, int L) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = part[i];
+  for (int g = 1; g < groups; ++g) {
+    const float x = part[(int64_t)g * count + i];
+    v = (layer_reduce == TRI_REDUCE_MAX) ? fmaxf(v, x) : __fadd_rn(v, x);
+  }
+  fin[i] = (layer_reduce == TRI_REDUCE_MEAN) ? __fdiv_rn(v, (float)L) : v;
 }
 
 // Clears the exchange words and the status word before a launch sequence.

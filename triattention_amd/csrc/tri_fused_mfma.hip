@@ -291,6 +291,12 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int b, within;
   if (!locate_workgroup(a, a.HC * a.tiles_per_seq, a.HC, reinterpret_cast<int*>(lds), b, within)) return;
+  // Layers of this workgroup: all of them, or one group of a layer-split launch, where `b` so far
+  // counts (sequence, group) pairs.
+  const int lgroup = b % a.layer_groups;
+  b /= a.layer_groups;
+  const int l_begin = lgroup * a.layers_per_group;
+  const int l_end = min(a.L, l_begin + a.layers_per_group);
   const int chunk = within % a.HC;
   const int tile = within / a.HC;
   const int T = checked_seq_len(a.seq_lens, b, a.Tmax, a.status);
@@ -591,7 +597,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     uint32_t prev = 0;
     if (lane == 0) prev = __hip_atomic_fetch_add(arrive_cnt, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
     prev = __builtin_amdgcn_readfirstlane(prev);
-    if (prev + 1 != (uint32_t)(l + 1) * (uint32_t)heads_here) return;
+    if (prev + 1 != (uint32_t)(l - l_begin + 1) * (uint32_t)heads_here) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     unsigned long long* out = a.xchg + (((int64_t)(b * a.L + l) * a.tiles_per_seq + tile) * a.A + ah0) * 2;
     for (int item = lane; item < items; item += 64) {
@@ -619,18 +625,19 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     if (a.normalize) {
       uint32_t won = 0;
       if (lane == 0) {
-        uint32_t expect = (uint32_t)l;
-        won = __hip_atomic_compare_exchange_strong(claimed, &expect, (uint32_t)(l + 1), __ATOMIC_ACQ_REL,
+        uint32_t expect = (uint32_t)(l - l_begin);
+        won = __hip_atomic_compare_exchange_strong(claimed, &expect, (uint32_t)(l - l_begin + 1), __ATOMIC_ACQ_REL,
                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) ? 1u : 0u;
       }
       won = __builtin_amdgcn_readfirstlane(won);
       if (won) {
         gather_layer_stats(a, b, l, seq_tiles, T, ah0, items, stats + (l & 1) * 64 * QG, lane, aborted);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        if (lane == 0) __hip_atomic_store(ready, (uint32_t)(l + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lane == 0)
+          __hip_atomic_store(ready, (uint32_t)(l - l_begin + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
       } else {
         // The claiming wave always finishes (its own waits are bounded).
-        while (__hip_atomic_load(ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)(l + 1))
+        while (__hip_atomic_load(ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)(l - l_begin + 1))
           __builtin_amdgcn_s_sleep(2);
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -669,7 +676,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       }
       const int n = n0 + tl;
       if (n >= window_from || n < prefill) v = INFINITY;
-      if (l == 0) fin[k] = v;
+      if (l == l_begin) fin[k] = v;
       else fin[k] = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(fin[k], v) : __fadd_rn(fin[k], v);
     }
   };
@@ -688,7 +695,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     if (slot < nsteps) compute_step(d, l, slot * 16);
   };
   StepData<DT, HD> buf[NB];
-  LayerBase base_cur = layer_base(0), base_next = base_cur;
+  LayerBase base_cur = layer_base(l_begin), base_next = base_cur;
   auto rotate = [&](int l, int r0, int r1) __attribute__((always_inline)) {
     for (int r = r0; r < r1; ++r) {
       const bool wrap = r + 1 >= rotations;
@@ -703,21 +710,32 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   };
   auto settle = [&]() __attribute__((always_inline)) { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
-  load_coefs(0);
+  load_coefs(l_begin);
 #pragma unroll
   for (int i = 0; i < NB; ++i) load_step(buf[i], base_cur, min(i, nsteps - 1) * 16);
-  for (int l = 0; l < a.L; ++l) {
+  for (int l = l_begin; l < l_end; ++l) {
     base_cur = base_next;
-    base_next = layer_base(min(l + 1, a.L - 1));
+    base_next = layer_base(min(l + 1, l_end - 1));
     settle();
     rotate(l, 0, rot_before_consume);
-    if (l > 0) consume(l - 1);
+    if (l > l_begin) consume(l - 1);
     rotate(l, rot_before_consume, rotations);
     if (a.normalize) arrive(l);
-    if (l + 1 < a.L) load_coefs(l + 1);
+    if (l + 1 < l_end) load_coefs(l + 1);
   }
-  consume(a.L - 1);
+  consume(l_end - 1);
 
+  if (a.layer_groups > 1) {
+    // This group's sum (or maximum) over its layers; fused_layer_reduce_kernel combines the groups.
+    const int64_t rows = (int64_t)(a.num_seqs / a.layer_groups) * a.Hkv;
+    float* out = a.fin_part + (((int64_t)lgroup * rows + (int64_t)b * a.Hkv + head) * a.Tmax) + n0;
+#pragma unroll
+    for (int k = 0; k < TW / 64; ++k) {
+      const int tl = lane + 64 * k;
+      if (tl < ntok) out[tl] = fin[k];
+    }
+    return;
+  }
   float* out = a.fin + ((int64_t)b * a.Hkv + head) * a.Tmax + n0;
 #pragma unroll
   for (int k = 0; k < TW / 64; ++k) {
@@ -752,10 +770,11 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, const LaunchShape& sha
   if (B <= seqs_per_launch) {
     k.packed = 0;
     k.seq_base = 0;
-    const int n = B;
+    const int n = B * k.layer_groups;      // (sequence, layer group) pairs; k.num_seqs counts the same
     hipLaunchKernelGGL((fused_mfma_kernel<DT, IL, TW, SL, QG, NB, W, HD>), dim3(n * k.tiles_per_seq * k.HC), dim3(W * kWave), lds, s, k, bmat);
     return hipGetLastError();
   }
+  if (k.layer_groups != 1) return hipErrorInvalidValue;   // layer groups exist in single launches only
   // More workgroups than the device holds at once: whole sequences are packed into
   // launches on the device (the host does not know the individual lengths); the host
   // issues as many launches as the worst case needs, surplus ones find no work.
@@ -871,7 +890,8 @@ int host_pack_launches(const int32_t* lens, int B, int tile, int wg_mult, int ca
 }  // namespace
 
 FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
-                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens) {
+                          int resident, bool any_fill, int kv_dtype, const int32_t* host_lens, int L,
+                          bool split_layers) {
   FusedPlan p{};
   const bool dim_ok = D == 128 || ((D == 64 || D == 256) && kv_dtype != TRI_KV_FP8_E4M3);
   if (resident <= 0 || !dim_ok || G < 1 || G > 8 || aggregation != TRI_REDUCE_MEAN || Tmax <= 0 || B <= 0)
@@ -912,7 +932,41 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   // (Workgroups of four waves: 45 %.  28 query / 4 KV heads, 16 x 2176 tokens, 272 of 512
   // workgroups: 0.40 ms against 0.48 ms on the two-pass kernels.)
   const int64_t need = waves == 4 ? 45 : 60;
-  if (!any_fill && (int64_t)B * tiles * HC * 100 < (int64_t)resident * need) return p;
+  int layer_groups = 1, layers_per_group = L;
+  if (split_layers && L > 1 && (int64_t)B * tiles * HC <= resident &&
+      (int64_t)B * tiles * HC * 100 < (int64_t)resident * need) {
+    // A few requests (the reference's runner compresses one at a time,
+    // runtime/runner_compression_actions.py:24): whole-model workgroups would use a fraction of
+    // the chip, e.g. 17 of 256 CUs for one request of 2176 tokens.  The layers are independent
+    // until the reduction over them, so they are cut into groups and a workgroup runs one
+    // (sequence, group, tile); fewest layers per group first, with tiles as long as the chip then
+    // has room for (a workgroup pays its per-layer exchange once per layer, so one layer of a
+    // long tile beats several layers of a short one): one request of 2176 tokens x 36 layers
+    // becomes 36 groups x 7 tiles of 320 tokens = 252 workgroups.
+    const int granule = (kv_dtype == TRI_KV_FP8_E4M3 || (D == 64 && G <= 4)) ? 128 : 64;
+    const int tw_max = tws[ntw - 1];                       // the longest tile any instance of this shape holds
+    const bool one_instance = !(waves == kFusedWaves && D == 128);
+    for (int lpg = 1; lpg < L; ++lpg) {
+      const int groups = ceil_div(L, lpg);
+      const int64_t units = (int64_t)B * groups * HC;
+      if (units > resident) continue;
+      const int tiles_max = (int)min((int64_t)64, resident / units);
+      int t = ceil_div(ceil_div(Tmax, tiles_max), granule) * granule;
+      t = min(tw_max, max(128, t));
+      const int nt = ceil_div(Tmax, t);
+      if (units * nt > resident) continue;
+      if (units * nt <= (int64_t)B * tiles * HC) break;      // no better than whole-model workgroups
+      layer_groups = groups;
+      layers_per_group = lpg;
+      tile = t;
+      tiles = nt;
+      if (!one_instance)
+        for (int i = 0; i < ntw; ++i)
+          if (tws[i] >= t) { tw = tws[i]; break; }           // the instance with the smallest ring that holds the tile
+      break;
+    }
+  }
+  if (!any_fill && (int64_t)B * layer_groups * tiles * HC * 100 < (int64_t)resident * need) return p;
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;
@@ -923,6 +977,9 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   p.bs_shift = bs_shift;
   p.waves = waves;
   p.launches = 0;
+  p.layer_groups = layer_groups;
+  p.layers_per_group = layers_per_group;
+  if (layer_groups > 1) p.seqs_per_launch = B;      // one launch by construction
   if (host_lens && (int64_t)B * tiles * HC > resident) {
     // Several launches, and the lengths are known: a launch takes as long as its tiles are
     // long, however many of its workgroups have work, so the tile size that packs the
@@ -963,7 +1020,11 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   k.block_size = a.block_size; k.bs_shift = a.plan.bs_shift;
   k.block_table_pitch = a.block_table ? a.block_table_pitch : -1;
   k.tiles_per_seq = a.plan.tiles_per_seq; k.tile_tokens = a.plan.tile_tokens;
-  k.seq_base = 0; k.num_seqs = a.B; k.Tmax = a.Tmax;
+  k.layer_groups = a.plan.layer_groups > 1 ? a.plan.layer_groups : 1;
+  k.layers_per_group = k.layer_groups > 1 ? a.plan.layers_per_group : a.L;
+  k.fin_part = a.fin_part;
+  if (k.layer_groups > 1 && (!a.fin_part || (int64_t)k.layer_groups * k.layers_per_group < a.L)) return hipErrorInvalidValue;
+  k.seq_base = 0; k.num_seqs = a.B * k.layer_groups; k.Tmax = a.Tmax;
   k.normalize = a.normalize; k.window_size = a.window_size; k.protect_prefill = a.protect_prefill;
   k.group_reduce = a.group_reduce; k.layer_reduce = a.layer_reduce;
   k.spin_ticks = resident_spin_ticks();
@@ -1012,13 +1073,19 @@ hipError_t launch_fused_mfma(const FusedLaunch& a, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (fp8)
-    return il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
-              : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
-  if (fp16)
-    return il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
-              : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
-  return il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
-            : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
+    e = il ? launch_mfma_tw<TRI_KV_FP8_E4M3, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+           : launch_mfma_tw<TRI_KV_FP8_E4M3, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
+  else if (fp16)
+    e = il ? launch_mfma_tw<TRI_KV_FP16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+           : launch_mfma_tw<TRI_KV_FP16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
+  else
+    e = il ? launch_mfma_tw<TRI_KV_BF16, true>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s)
+           : launch_mfma_tw<TRI_KV_BF16, false>(k, bmat, a.plan.tw, a.plan.waves, a.D, shape, s);
+  if (e != hipSuccess || k.layer_groups <= 1 || a.skip_layer_reduce) return e;
+  const int64_t count = (int64_t)a.B * a.Hkv * a.Tmax;
+  hipLaunchKernelGGL(fused_layer_reduce_kernel, dim3((unsigned)ceil_div64(count, 256)), dim3(256), 0, s, a.fin_part, a.fin,
+                     count, k.layer_groups, a.layer_reduce, a.L);
+  return hipGetLastError();
 }
 
 }  // namespace tri

@@ -332,7 +332,8 @@ template <int VPT>
 __global__ __launch_bounds__(kTopkThreads) void topk_rows_reg_kernel(const float* scores, int64_t row_pitch,
                                                                     const int32_t* row_lens,
                                                                     const int32_t* row_ks, int rows_per_entry,
-                                                                    int32_t* keep, int keep_pitch, int max_len) {
+                                                                    int32_t* keep, int keep_pitch, int max_len,
+                                                                    int groups, int64_t group_stride, int group_max) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t sh_prefix, sh_remaining;
   __shared__ uint32_t wave_tot[kTopkThreads / 64];
@@ -357,7 +358,24 @@ __global__ __launch_bounds__(kTopkThreads) void topk_rows_reg_kernel(const float
   const int c0 = tid * VPT;
   const int nvalid = min(max(T - c0, 0), VPT);
   uint32_t key[VPT];
-  if (nvalid == VPT && (reinterpret_cast<uintptr_t>(x + c0) & 15) == 0) {
+  if (groups > 1) {
+    // The row arrives as `groups` partial rows `group_stride` floats apart (a resident launch cut
+    // by layers): they are added (or maximised) in group order, exactly as
+    // fused_layer_reduce_kernel does; the division by the layer count that turns the sum into a
+    // mean does not change the order of the scores and is left out.
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      float v = 0.f;
+      if (i < nvalid) {
+        v = x[c0 + i];
+        for (int g = 1; g < groups; ++g) {
+          const float y = x[(int64_t)g * group_stride + c0 + i];
+          v = group_max ? fmaxf(v, y) : __fadd_rn(v, y);
+        }
+      }
+      key[i] = i < nvalid ? float_key(v) : 0u;
+    }
+  } else if (nvalid == VPT && (reinterpret_cast<uintptr_t>(x + c0) & 15) == 0) {
 #pragma unroll
     for (int i = 0; i < VPT; i += 4) {
       const float4 v = *reinterpret_cast<const float4*>(x + c0 + i);
@@ -449,22 +467,28 @@ __global__ __launch_bounds__(kTopkThreads) void topk_rows_reg_kernel(const float
 
 hipError_t launch_topk_rows(const float* scores, int64_t row_pitch, int num_rows,
                             const int32_t* row_lens, const int32_t* row_ks, int rows_per_entry, int max_len,
-                            int32_t* keep, int keep_pitch, hipStream_t s) {
+                            int32_t* keep, int keep_pitch, hipStream_t s, int groups, int64_t group_stride,
+                            int group_max) {
   if (num_rows <= 0) return hipSuccess;
   if (max_len > 0 && max_len <= 8 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<8>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len, groups, group_stride, group_max);
   else if (max_len > 0 && max_len <= 16 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<16>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len, groups, group_stride, group_max);
   else if (max_len > 0 && max_len <= 32 * kTopkThreads)
     hipLaunchKernelGGL(topk_rows_reg_kernel<32>, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
-                       row_ks, rows_per_entry, keep, keep_pitch, max_len);
+                       row_ks, rows_per_entry, keep, keep_pitch, max_len, groups, group_stride, group_max);
+  else if (groups > 1)
+    return hipErrorInvalidValue;      // rows beyond the register kernels are reduced by the caller first
   else
     hipLaunchKernelGGL(topk_rows_kernel, dim3(num_rows), dim3(kTopkThreads), 0, s, scores, row_pitch, row_lens,
                        row_ks, rows_per_entry, keep, keep_pitch, max_len);
   return hipGetLastError();
 }
+
+// Longest row the register top-k kernels take (they can also add partial rows while loading).
+int topk_register_row_limit() { return 32 * kTopkThreads; }
 
 __global__ void clear_word_kernel(uint32_t* word) { *word = 0u; }
 

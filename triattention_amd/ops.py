@@ -204,7 +204,8 @@ class StepBatch:
             rows = [int(x) for r in block_tables for x in (list(r) + [0] * (pitch - len(r)))]
         # One host-to-device copy for all the small integer arrays of the step.
         parts = [self.seq_lens_host, rs, pf or [], self.budgets_host or [], rows or []]
-        flat = torch.tensor([x for part in parts for x in part], dtype=torch.int32, device=device)
+        flat = torch.tensor([x for part in parts for x in part], dtype=torch.int32,
+                            pin_memory=True).to(device, non_blocking=True)
         cuts, pos = [], 0
         for part in parts:
             cuts.append(flat[pos:pos + len(part)])
@@ -317,9 +318,14 @@ class Workspace:
                                                                     C.byref(sp)))
 
     def status(self) -> int:
-        """Synchronises, then returns the resident kernel's status word (0 = fine)."""
+        """Synchronises the device, then returns the resident kernel's status word (0 = fine).
+        The word travels to pinned host memory with a copy queued on the current stream before
+        that wait, so the host waits once."""
+        if getattr(self, "_status_host", None) is None:
+            self._status_host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        self._status_host.copy_(self.buf[self._status_at:self._status_at + 4].view(torch.int32), non_blocking=True)
         torch.cuda.synchronize(self.buf.device)
-        return int(self.buf[self._status_at:self._status_at + 4].view(torch.int32).item())
+        return int(self._status_host[0])
 
     def fits(self, kv, batch, sc) -> bool:
         sp = sc.struct()

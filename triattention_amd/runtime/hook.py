@@ -408,6 +408,12 @@ def build_hook_runtime_context(*, base_runner: Any, config: TriAttentionRuntimeC
                               int(recent) if isinstance(recent, int) else None, bool(defer))
 
 
+# A single request in the default mode goes through the same one-call launch sequence as a batch
+# of requests; False sends it through the reference-shaped pipeline (selector callable, then the
+# per-head compaction function), which gives the same result dictionaries and cache contents.
+SINGLE_REQUEST_IN_ONE_CALL = True
+
+
 @dataclass
 class _Ready:
     """A triggered request that passed every check in front of the kernels."""
@@ -510,7 +516,14 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
 
     def _hook(req_id: str, signal: CompressionSignal, scheduler_output: Any) -> dict:
         ready = _prepare(req_id, signal, scheduler_output)
-        return ready if isinstance(ready, dict) else _run_single(ready)
+        if isinstance(ready, dict):
+            return ready
+        if SINGLE_REQUEST_IN_ONE_CALL and _batchable(ready):
+            # Default mode, something to drop: score, select and compact in one library call with one
+            # host synchronisation at its end (the layer-by-layer pipeline below waits for the keep
+            # indices on the host before the compaction is launched).
+            return _run_batch([ready])[req_id]
+        return _run_single(ready)
 
     def _batchable(r: "_Ready") -> bool:
         """True when the one-by-one path would take the group selector and the ordered
@@ -614,7 +627,7 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
                 together.append(ready)
             else:
                 results[req_id] = _run_single(ready)
-        if len(together) == 1:
+        if len(together) == 1 and not SINGLE_REQUEST_IN_ONE_CALL:
             results[together[0].req_id] = _run_single(together[0])
         elif together:
             results.update(_run_batch(together))
