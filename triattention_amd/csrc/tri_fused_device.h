@@ -245,5 +245,72 @@ __device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, in
   }
 }
 
+// The same statistics for the score heads of ONE KV head (`heads` of them, at most 8, starting at
+// score head ah_first), gathered by the wave that scores that KV head, with no other wave
+// involved: the 64 lanes are (item, part) pairs -- item = (head, sum | sum of squares), 16 slots of
+// which 2 * heads are used; part = a quarter of the sequence's tiles -- so the tagged words of all
+// tiles are requested in ceil(tiles / 32) rounds of eight loads per lane, where one wave gathering
+// for all eight KV heads of the workgroup needs tiles / 4 rounds (16 of them, on the critical
+// path of every layer, for 64 tiles of eight query heads per KV head).  Tile order inside a
+// part, parts in order: a fixed summation order.  mean[i] / sd[i] of head ah_first + i come back in
+// every lane.  Called by one whole wave.
+__device__ __forceinline__ void gather_head_stats(const FusedArgs& a, int b, int l, int seq_tiles, int T, int ah_first,
+                                                  int heads, float* mean, float* sd, int lane, bool& aborted) {
+  const int item = lane & 15, part = lane >> 4;
+  const bool live = item < 2 * heads;
+  const int per_part = ceil_div(seq_tiles, 4);
+  const int t_lo = part * per_part, t_hi = min(t_lo + per_part, seq_tiles);
+  const unsigned long long* in =
+      a.xchg + ((int64_t)(b * a.L + l) * a.tiles_per_seq * a.A + ah_first) * 2 + (live ? item : 0);
+  const uint32_t want = (uint32_t)(l + 1);
+  const long long t_begin = wall_clock64();
+  if (a.spin_ticks < 0 && !aborted) {
+    aborted = true;
+    if (lane == 0) atomicCAS(a.status, 0u, 1u);
+  }
+  double acc = 0.0;
+  for (int t0 = 0; t0 < per_part; t0 += 8) {       // (wave-uniform trip count; lanes past their part's end idle)
+    unsigned long long w[8];
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int t = t_lo + t0 + u;
+        const bool mine = live && t < t_hi;
+        w[u] = mine ? xchg_load(in + (int64_t)t * a.A * 2) : ((unsigned long long)want << 32);
+        ok = ok && (uint32_t)(w[u] >> 32) == want;
+      }
+      if (__all(ok) || aborted) break;
+      if (wall_clock64() - t_begin > a.spin_ticks ||
+          __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+        aborted = true;
+        if (lane == 0) atomicCAS(a.status, 0u, 1u);
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (t_lo + t0 + u < t_hi) acc += (double)__uint_as_float((uint32_t)w[u]);
+  }
+  // parts in order: ((p0 + p1) + p2) + p3, in lanes 0..15
+  double total = acc;
+  total += __shfl(acc, item + 16);
+  total += __shfl(acc, item + 32);
+  total += __shfl(acc, item + 48);
+  const float mine = (float)total;
+  const float cnt = (float)T;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float sum = __shfl(mine, 2 * i), sumsq = __shfl(mine, 2 * i + 1);
+    const float m = __fdiv_rn(sum, cnt);
+    float var = 0.f;
+    if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(m, m))), (float)(T - 1));
+    var = fmaxf(var, 0.f);
+    float s = __fsqrt_rn(var);
+    if (s < 1e-8f) s = 1.f;
+    if (i < heads) { mean[i] = m; sd[i] = s; }
+  }
+}
+
 }  // namespace
 }  // namespace tri

@@ -623,6 +623,21 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
 #pragma unroll
     for (int qq = 0; qq < RQ; ++qq) { mean[qq] = 0.f; sd[qq] = 1.f; }
     if (a.normalize) {
+      if constexpr (QG == 2) {
+        // More than four query heads per KV head: twice the words per tile and tiles half as long,
+        // so the gather is four times the work; every wave fetches the words of its own KV head
+        // (8 x 32768 tokens x 64 layers, 64 query heads: 7.55 -> 6.82 ms).  With up to four query
+        // heads the one wave's gather below hides behind the slack and this form is slower (16 x 16384
+        // tokens x 36 layers: 3.29 -> 3.30 ms; fp8 keys 1.72 -> 1.80; 16 x 2176 tokens 0.54 -> 0.62).
+        float m8[8], s8[8];
+        gather_head_stats(a, b, l, seq_tiles, T, (chunk * 8 + wave) * a.G, a.G, m8, s8, lane, aborted);
+#pragma unroll
+        for (int qq = 0; qq < RQ; ++qq)
+          if (qq < a.G) {
+            mean[qq] = m8[qq];
+            sd[qq] = __fdiv_rn(1.f, s8[qq]);
+          }
+      } else {
       uint32_t won = 0;
       if (lane == 0) {
         uint32_t expect = (uint32_t)(l - l_begin);
@@ -650,6 +665,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
           // division per score costs ten vector instructions, 7 % of the kernel's total).
           sd[qq] = __fdiv_rn(1.f, st[(wave * a.G + qq) * 2 + 1]);
         }
+      }
     }
 #pragma unroll
     for (int k = 0; k < TW / 64; ++k) {
