@@ -100,7 +100,9 @@ typedef struct tri_score_params {
 
 /* Selection semantics (runtime/selector_hf.py:813-1033 and :473-677). */
 typedef struct tri_select_params {
-  int32_t normalize;            /* sparse_normalize_scores */
+  int32_t normalize;            /* 0: raw scores; 1: sparse_normalize_scores (streaming unbiased std, std < 1e-8 -> 1,
+                                   runtime/selector_hf.py:902-909); 2: the research path's z-score (population std
+                                   clamped at 1e-6, methods/triattention.py:255-258; two-pass kernels only) */
   int32_t window_size;          /* recent tokens forced to +inf (runtime/selector_hf.py:121-130) */
   int32_t protect_prefill;      /* tokens < prefill_len forced to +inf */
   int32_t group_reduce;         /* tri_reduce over the query heads of a KV head (runtime/selector_hf.py:277-297) */

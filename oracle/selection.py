@@ -177,6 +177,37 @@ def layer_final_scores(
     return x
 
 
+def hf_final_scores(raw_by_layer: Sequence[torch.Tensor], num_kv_heads: int, decode_start: int,
+                    normalize: bool = True) -> torch.Tensor:
+    """Selection scores of the research path, over the decode tokens only
+    (triattention/methods/triattention.py:250-258 and :368-425): every (layer, head) row of
+    raw scores from token ``decode_start`` on is z-scored with the POPULATION standard deviation
+    clamped from below at 1e-6 (not the runtime's unbiased std with ``< 1e-8 -> 1``), then
+    per KV head the maximum over its query heads per layer and the mean over layers.
+    The 1e-6 uniform noise of :260-267 exists only when the object carries a generator and is
+    not part of this.  Returns [Hkv, T - decode_start]."""
+    rows = torch.stack([r[:, decode_start:].to(torch.float32) for r in raw_by_layer])       # [L, Hq, Td]
+    if normalize and rows.numel() > 0:
+        mean = rows.mean(dim=-1, keepdim=True)
+        std = rows.std(dim=-1, unbiased=False, keepdim=True).clamp_min(1e-6)
+        rows = (rows - mean) / std
+    layers, hq, td = rows.shape
+    grouped = rows.view(layers, num_kv_heads, hq // num_kv_heads, td)
+    return grouped.max(dim=2).values.mean(dim=0)
+
+
+def hf_keep_per_head(raw_by_layer, num_kv_heads: int, decode_start: int, keep_count: int, normalize: bool = True):
+    """[Hkv, decode_start + k] absolute indices, ascending: the prefill, then the top ``keep_count``
+    decode tokens per KV head (methods/triattention.py:427-448; the reference leaves the decode part
+    in top-k order, the oracle sorts it and breaks ties by the lowest index).  Also returns the
+    selection scores."""
+    fin = hf_final_scores(raw_by_layer, num_kv_heads, decode_start, normalize)
+    k = min(keep_count, fin.shape[-1])
+    dec = topk_ascending(fin, k) + decode_start
+    pre = torch.arange(decode_start, dtype=torch.long).unsqueeze(0).expand(num_kv_heads, -1)
+    return torch.cat([pre, dec], dim=1).contiguous(), fin
+
+
 def protect_window(scores: torch.Tensor, window_size: int) -> torch.Tensor:
     """core/utils.py:483-502."""
     if window_size <= 0:

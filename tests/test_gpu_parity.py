@@ -1257,3 +1257,36 @@ def test_invalid_arguments_raise():
         ops.compact(kv, batch, torch.zeros(3, 5, dtype=torch.int32, device=DEV))
     with pytest.raises(RuntimeError):
         ops.PagedKV.from_kv_caches([c.cpu() for c in caches])
+
+
+@pytest.mark.parametrize("hq,hkv,decode_start,keep_count", [(8, 2, 40, 96), (14, 2, 0, 64), (4, 4, 17, 200), (8, 2, 290, 50)])
+def test_research_path_selection_matches_oracle(hq, hkv, decode_start, keep_count):
+    """``hf_selection.select_keep_indices_per_head`` (decode tokens only, population std clamped at 1e-6,
+    group max, layer mean, no window) against ``oracle.selection.hf_keep_per_head``, whose selection is
+    pinned by the reference's own ``_select_per_head_independent`` (tests/golden/hf_select.pt)."""
+    from triattention_amd import hf_selection
+    w = small(num_layers=3, num_q_heads=hq, num_kv_heads=hkv, seq_lens=(300,), budget=keep_count, window_size=0,
+              index=80 + hq)
+    inp = build_inputs(w)
+    t = 300
+    kc = [ocp.split_kv(c, inp["kv_axis"])[0] for c in inp["caches"]]
+    dense = [ocp.gather_dense(k, inp["tables"][0], w.block_size, 0, t).to(DEV) for k in kc]         # [1, Hkv, T, D]
+    folded = ops.fold_stats(inp["qc"].to(DEV), inp["qa"].to(DEV), inp["fs"].to(DEV))
+    got = hf_selection.select_keep_indices_per_head(dense, decode_start=decode_start, keep_count=keep_count,
+                                                    folded_stats=folded, inv_freq=inp["omega"].to(DEV),
+                                                    offsets=inp["offsets"].to(DEV), round_start=t)
+    oraw = oracle_raw(w, inp, 0, t)
+    want, fin = osel.hf_keep_per_head(oraw, hkv, decode_start, keep_count)
+    got = got.cpu()
+    k = min(keep_count, t - decode_start)
+    assert got.dtype == torch.long and tuple(got.shape) == (hkv, decode_start + k)
+    assert torch.equal(got[:, :decode_start], want[:, :decode_start])
+    assert bool((got[:, 1:] > got[:, :-1]).all())
+    if k == t - decode_start:
+        assert torch.equal(got, want)
+        return
+    scale = float(fin.abs().max())
+    swapped = assert_keep_matches(got[:, decode_start:] - decode_start, want[:, decode_start:] - decode_start, fin, k,
+                                  tie_tol=KEEP_TIE_TOL * scale)
+    record_swaps(f"research_path_vs_oracle:{hq}/{hkv}:{decode_start}", swapped, hkv * k)
+    assert swapped == 0

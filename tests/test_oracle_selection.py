@@ -94,6 +94,26 @@ def test_group_selection_matches_reference_across_chunks_at_the_benchmarked_head
     assert torch.equal(keep, want)
 
 
+@pytest.mark.parametrize("case", ["gqa4", "gqa7_no_prefill", "mha"])
+def test_research_path_selection_matches_reference(case):
+    """``oracle.selection.hf_keep_per_head`` against the reference's own
+    ``_select_per_head_independent`` (fixture written by tests/golden/make_hf_select_golden.py):
+    same kept sets per KV head (the reference leaves the decode part in top-k order)."""
+    gold = load_golden("hf_select.pt")[case]
+    raw = [gold["raw"][l] for l in range(gold["raw"].shape[0])]
+    hkv, start, k = int(gold["num_kv_heads"]), int(gold["decode_start"]), int(gold["keep_count"])
+    keep, fin = osel.hf_keep_per_head(raw, hkv, start, k)
+    want = gold["keep"]
+    assert keep.shape == want.shape and bool((keep[:, 1:] > keep[:, :-1]).all())
+    assert torch.equal(keep[:, :start], want[:, :start])                     # the prefill, in order
+    assert torch.equal(keep, torch.sort(want, dim=1).values)
+    # what distinguishes it from the runtime's normalisation: population std, clamp instead of "-> 1"
+    x = gold["raw"][0][:, start:]
+    z = (x - x.mean(-1, keepdim=True)) / x.std(-1, unbiased=False, keepdim=True).clamp_min(1e-6)
+    assert float(z[1].abs().max()) < 1e-3 and abs(float(z[0].pow(2).mean()) - 1.0) < 1e-5
+    assert not torch.allclose(z[0], osel.znorm_two_pass(x)[0], atol=1e-4)
+
+
 def test_streaming_stats_match_torch():
     g = torch.Generator().manual_seed(3)
     x = torch.randn(6, 1000, generator=g) * 3 + 5

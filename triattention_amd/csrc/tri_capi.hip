@@ -201,6 +201,9 @@ int check_select(const tri_select_params* sel) {
   if (sel->layer_reduce != TRI_REDUCE_MEAN && sel->layer_reduce != TRI_REDUCE_MAX && sel->layer_reduce != -1)
     return fail(TRI_ERR_INVALID_ARGUMENT, "layer_reduce %d", sel->layer_reduce);
   if (sel->window_size < 0) return fail(TRI_ERR_INVALID_ARGUMENT, "window_size %d", sel->window_size);
+  if (sel->normalize < 0 || sel->normalize > 2) return fail(TRI_ERR_INVALID_ARGUMENT, "normalize %d", sel->normalize);
+  if (sel->normalize == 2 && sel->group_first)
+    return fail(TRI_ERR_UNSUPPORTED, "the population-std normalisation is built for the normalise-then-reduce order only");
   return TRI_OK;
 }
 
@@ -227,7 +230,8 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
 int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
                     hipStream_t s) {
-  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident;
+  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident &&
+                     sel->normalize != 2;
   if (!fused) {
     // The status word belongs to the resident kernel; on this path it just reads "fine".
     const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
@@ -439,7 +443,8 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident)
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident &&
+          sel->normalize != 2)
              ? w.fused.eligible : 0;
 }
 

@@ -41,6 +41,14 @@ __global__ void finalize_stats_kernel(const float* partial, const int32_t* seq_l
     var = fmaxf(var, 0.f);
     sd = __fsqrt_rn(var);
     if (sd < 1e-8f) sd = 1.f;
+    if (normalize == 2) {
+      // The research path's normalisation (methods/triattention.py:255-258): population standard
+      // deviation, clamped from below at 1e-6; from the double-precision sums.
+      const double m = s / (double)T;
+      const double v = q / (double)T - m * m;
+      mean = (float)m;
+      sd = fmaxf((float)sqrt(v > 0.0 ? v : 0.0), 1e-6f);
+    }
   }
   mustd[(int64_t)idx * 2] = mean;
   mustd[(int64_t)idx * 2 + 1] = sd;

@@ -262,7 +262,7 @@ class ScoreConfig:
 
 @dataclass
 class SelectConfig:
-    normalize: bool = True
+    normalize: bool | str = True         # True / False, or "population": population std clamped at 1e-6 (research path)
     window_size: int = 128
     protect_prefill: bool = False
     group_reduce: str = "max"
@@ -273,7 +273,8 @@ class SelectConfig:
 
     def struct(self) -> SelectParams:
         lr = REDUCE_NONE if self.layer_reduce is None else (REDUCE_MAX if self.layer_reduce == "max" else REDUCE_MEAN)
-        return SelectParams(normalize=int(self.normalize), window_size=int(self.window_size),
+        return SelectParams(normalize=2 if self.normalize == "population" else int(bool(self.normalize)),
+                            window_size=int(self.window_size),
                             protect_prefill=int(self.protect_prefill),
                             group_reduce=REDUCE_MAX if self.group_reduce == "max" else REDUCE_MEAN,
                             layer_reduce=lr, shared=int(self.shared), group_first=int(self.group_first),
