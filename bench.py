@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 MEASURED_TRAFFIC_BYTES = {
     ("c1_qwen3_8b_36l_b16_16k", "two_pass"): (9_717_510 * 1024 * 2 + 1_184_256 * 1024,       # score_mean_kernel
                                                "profiles/c1_step_hbm_counters.txt"),
-    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_476_694 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
+    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_477_735 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
                                                     "profiles/c1_step_hbm_counters.txt"),
 }
 
