@@ -329,6 +329,8 @@ class Workspace:
         return int(self._status_host[0])
 
     def fits(self, kv, batch, sc) -> bool:
+        if self.buf.device != kv.device:
+            return False
         sp = sc.struct()
         need = int(_lib.load().tri_workspace_bytes(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp)))
         return 0 < need <= self.bytes

@@ -294,8 +294,16 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                                protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
                                allow_resident=bool(allow_resident) and holder.get("resident_ok", True))
         resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
+        # Scratch and keep rows of the previous step are reused when they fit (steady state: every
+        # call has the shape of the last one); the results handed out below are fresh tensors.
+        rows = len(requests) * kv.num_kv_heads
+        keep_buf = holder.get("keep")
+        if keep_buf is None or keep_buf.device != kv.device or keep_buf.numel() < rows * batch.max_budget:
+            keep_buf = holder["keep"] = torch.empty(rows * batch.max_budget, dtype=torch.int32, device=kv.device)
         try:
-            keep, ws = ops.compress_step(kv, batch, sc, sel)
+            keep, ws = ops.compress_step(kv, batch, sc, sel, holder.get("ws"),
+                                         keep_buf[:rows * batch.max_budget].view(rows, batch.max_budget))
+            holder["ws"] = ws
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
         if resident and ws.status() != 0:
