@@ -336,6 +336,62 @@ def test_batch_hook_on_the_resident_kernel(tmp_path, monkeypatch):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+@pytest.mark.parametrize("resident", [False, True])
+def test_repeated_shape_replays_a_graph_with_the_same_results(tmp_path, monkeypatch, resident):
+    """A decoding request comes back to the hook with the same lengths every ``divide_length``
+    tokens: from the second visit on the selector replays a captured launch sequence.  Eight steps
+    with fresh cache contents, other block lists, other round starts and a prefill guard that comes
+    and goes, next to a selector that never replays: equal results, bit-identical caches after every
+    step (the program's own eager work and synchronisations lie between the replays)."""
+    from helpers import build_inputs
+    from triattention_amd import synth
+    from triattention_amd.runtime import selector as selector_mod
+    if not resident:
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    w = synth.Workload(name="t", num_layers=3, num_q_heads=8, num_kv_heads=2, head_dim=128,
+                       seq_lens=(1184,) * (16 if resident else 1), budget=160, block_size=16, window_size=12,
+                       rope_theta=1e6, index=41)
+    inp = build_inputs(w)
+    monkeypatch.setattr(selector_mod, "GRAPH_REPLAY", True)
+    # (the cache is refilled by hand below; the guard against a cache that grew back is for real decoding)
+    replay = _fake_runner(w, inp, tmp_path, fail_on_effective_len_regression=False)
+    monkeypatch.setattr(selector_mod, "GRAPH_REPLAY", False)
+    eager = _fake_runner(w, inp, tmp_path, fail_on_effective_len_regression=False)
+    before = dict(selector_mod.GRAPH_COUNTS)
+    gen = torch.Generator().manual_seed(5)
+    pool = inp["caches"][0].shape[1]
+    need = len(inp["tables"][0])
+    for step in range(8):
+        fresh = [torch.randn(c.shape, generator=gen).to(c.dtype) for c in inp["caches"]]
+        perm = torch.randperm(pool, generator=gen).tolist()
+        tables = [perm[b * need:(b + 1) * need] for b in range(w.num_seqs)]
+        results = []
+        for flag, (runner, reqs, caches, sched, _) in ((True, replay), (False, eager)):
+            monkeypatch.setattr(selector_mod, "GRAPH_REPLAY", flag)
+            for c, f in zip(caches, fresh):
+                c.copy_(f)
+            signals = {}
+            for b, rid in enumerate(reqs):
+                reqs[rid].num_computed_tokens = 1184
+                reqs[rid].block_ids = (list(tables[b]),)
+                guard = step in (2, 3, 4) or not resident
+                signals[rid] = _signal(req_id=rid, estimated_cache_len=1185, prefill_len=30 + step + b if guard else 0,
+                                       protect_prefill=guard, step=step + 1)
+            ex = RunnerHookCompressionExecutor(runner)
+            results.append(ex.execute_batch(signals, sched) if resident else
+                           {rid: ex.execute(rid, sig, sched) for rid, sig in signals.items()})
+        torch.cuda.synchronize()
+        assert results[0] == results[1], f"step {step}"
+        assert all(r.applied and r.cache_len_after == 160 for r in results[0].values()), f"step {step}"
+        for a, b in zip(replay[2], eager[2]):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}: caches differ"
+        for rid in replay[1]:
+            assert replay[1][rid].block_ids == eager[1][rid].block_ids
+    # resident: two shapes (with and without the guard), 5 + 3 visits; otherwise one shape, 8 visits
+    assert selector_mod.GRAPH_COUNTS["captured"] - before["captured"] == (2 if resident else 1)
+    assert selector_mod.GRAPH_COUNTS["replayed"] - before["replayed"] == (4 if resident else 6)
+
+
 def test_runner_hook_on_an_fp8_cache_kept_in_uint8_tensors(tmp_path):
     """vLLM keeps an fp8 KV cache as uint8 tensors with one scale per tensor: the hook scores
     the codes as they are and moves rows only.  Same result dictionary and the same bytes as

@@ -210,6 +210,7 @@ class StepBatch:
         for part in parts:
             cuts.append(flat[pos:pos + len(part)])
             pos += len(part)
+        self._flat, self._sizes, self._table_in_flat = flat, [len(part) for part in parts], rows is not None
         self.seq_lens, self.round_start = cuts[0], cuts[1]
         self.prefill_lens = cuts[2] if pf is not None else None
         self.budgets = cuts[3] if self.budgets_host is not None else None
@@ -232,6 +233,36 @@ class StepBatch:
             block_table_pitch=pitch, block_table=_ptr(self.block_table), seq_lens=_ptr(self.seq_lens),
             round_start=_ptr(self.round_start), prefill_lens=_ptr(self.prefill_lens),
             budgets=_ptr(self.budgets), seq_lens_host=C.cast(self._lens_host, C.c_void_p))
+
+    def refill(self, round_start, block_tables, prefill_lens=None) -> None:
+        """New round starts, block tables and prefill lengths for the SAME sequence lengths and
+        budgets, written into the device arrays this batch already owns (their addresses do not
+        change: a launch sequence captured into a HIP graph with this batch can be replayed).
+        One pinned host-to-device copy, stream ordered."""
+        n = self.num_seqs
+        if not self._table_in_flat:
+            raise ValueError("this batch was not built from host lists with block tables")
+        pitch = int(self.block_table.shape[1])
+        rows = []
+        for r in block_tables:
+            if len(r) > pitch:
+                raise ValueError(f"a block table of {len(r)} entries does not fit the batch's pitch of {pitch}")
+            rows.extend(int(x) for x in r)
+            rows.extend([0] * (pitch - len(r)))
+        pf = [int(x) for x in prefill_lens] if prefill_lens is not None else [0] * n
+        parts = [self.seq_lens_host, [int(x) for x in round_start], pf if self.prefill_lens is not None else [],
+                 self.budgets_host or [], rows]
+        if [len(p) for p in parts] != self._sizes or len(block_tables) != n:
+            raise ValueError("refill needs the shapes the batch was built with")
+        staging = getattr(self, "_staging", None)
+        if staging is None:
+            staging = self._staging = torch.empty(self._flat.numel(), dtype=torch.int32, pin_memory=True)
+            self._staged = torch.cuda.Event()
+        else:
+            self._staged.synchronize()          # the previous copy out of the staging buffer has finished
+        staging.copy_(torch.tensor([x for part in parts for x in part], dtype=torch.int32))
+        self._flat.copy_(staging, non_blocking=True)
+        self._staged.record()
 
     def check_capacity(self, block_size: int) -> None:
         """Host-side bounds check: every sequence owns enough blocks for its tokens."""

@@ -75,6 +75,11 @@ class _DeviceStats:
         return out
 
 
+# Steady-state steps (a shape seen before) replay their launch sequence from a HIP graph.
+GRAPH_REPLAY = True
+GRAPH_COUNTS = {"captured": 0, "replayed": 0}     # process-wide, for tests and diagnostics
+
+
 class ResidentLaunchFailed(RuntimeError):
     """The resident kernel gave up waiting for its other workgroups (the GPU was shared with
     another workload for seconds); nothing was compacted, the step can be repeated."""
@@ -287,23 +292,55 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         if any(k <= 0 or k >= t for k, t in zip(ks, totals)):
             raise RuntimeError("batched compression expects total_tokens > budget_total > 0")
         guards = [int(r["prefill_len"]) if r["protect_prefill"] and int(r["prefill_len"]) > 0 else 0 for r in requests]
-        batch = ops.StepBatch(kv.device, totals, round_start=[int(r["round_start"]) for r in requests], budgets=ks,
-                              block_tables=[[int(x) for x in r["block_ids"]] for r in requests],
-                              prefill_lens=guards)
-        sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
-                               protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
-                               allow_resident=bool(allow_resident) and holder.get("resident_ok", True))
-        resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
-        # Scratch and keep rows of the previous step are reused when they fit (steady state: every
-        # call has the shape of the last one); the results handed out below are fresh tensors.
+        rounds = [int(r["round_start"]) for r in requests]
+        tables = [[int(x) for x in r["block_ids"]] for r in requests]
+        use_resident = bool(allow_resident) and holder.get("resident_ok", True)
         rows = len(requests) * kv.num_kv_heads
-        keep_buf = holder.get("keep")
-        if keep_buf is None or keep_buf.device != kv.device or keep_buf.numel() < rows * batch.max_budget:
-            keep_buf = holder["keep"] = torch.empty(rows * batch.max_budget, dtype=torch.int32, device=kv.device)
+        # A long generation repeats one shape (budget + divide_length tokens down to budget) every
+        # divide_length tokens.  The second time a shape is seen its launch sequence is captured into
+        # a HIP graph over device arrays that stay put; from then on a step is one small pinned copy
+        # of the step's integers and one graph launch.  (The first time runs eagerly: most shapes,
+        # e.g. the first compression after a long prompt, never come back.)
+        key = (id(kv), layer_ids, tuple(totals), tuple(ks), tuple(len(t) for t in tables), any(g > 0 for g in guards),
+               agg, use_resident)
+        entry = holder.setdefault("graphs", {}).get(key) if GRAPH_REPLAY else None
         try:
-            keep, ws = ops.compress_step(kv, batch, sc, sel, holder.get("ws"),
-                                         keep_buf[:rows * batch.max_budget].view(rows, batch.max_budget))
-            holder["ws"] = ws
+            if entry is not None and entry.get("graph") is not None:
+                batch, ws, keep, resident = entry["batch"], entry["ws"], entry["keep"], entry["resident"]
+                batch.refill(rounds, tables, guards)
+                entry["graph"].replay()
+                GRAPH_COUNTS["replayed"] += 1
+            else:
+                batch = ops.StepBatch(kv.device, totals, round_start=rounds, budgets=ks, block_tables=tables,
+                                      prefill_lens=guards)
+                sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
+                                       protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
+                                       allow_resident=use_resident)
+                resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
+                if entry is None:
+                    # Scratch and keep rows of the previous step are reused when they fit; the results
+                    # handed out below are fresh tensors.
+                    keep_buf = holder.get("keep")
+                    if keep_buf is None or keep_buf.device != kv.device or keep_buf.numel() < rows * batch.max_budget:
+                        keep_buf = holder["keep"] = torch.empty(rows * batch.max_budget, dtype=torch.int32,
+                                                                device=kv.device)
+                    keep, ws = ops.compress_step(kv, batch, sc, sel, holder.get("ws"),
+                                                 keep_buf[:rows * batch.max_budget].view(rows, batch.max_budget))
+                    holder["ws"] = ws
+                    if GRAPH_REPLAY:
+                        if len(holder["graphs"]) >= 8:
+                            holder["graphs"].pop(next(iter(holder["graphs"])))
+                        holder["graphs"][key] = {"graph": None}
+                else:
+                    # Second visit: buffers of the entry's own, capture (nothing runs), then replay.
+                    ws = ops.Workspace(kv, batch, sc)
+                    keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        ops.compress_step(kv, batch, sc, sel, ws, keep)
+                    entry.update(graph=graph, batch=batch, ws=ws, keep=keep, resident=resident, kv=kv, sc=sc)
+                    graph.replay()
+                    GRAPH_COUNTS["captured"] += 1
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
         if resident and ws.status() != 0:
