@@ -1079,6 +1079,43 @@ def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
     assert ws.status() == 0
 
 
+@pytest.mark.parametrize("what", ["key", "coefficient"])
+def test_magnitudes_beyond_half_range_raise_the_status_word(monkeypatch, what):
+    """Whatever the key type, the matrix-core kernel carries the magnitudes |k_f| and their
+    coefficients as fp16 pieces.  A bf16 key whose magnitude exceeds 65504, or statistics that make a
+    magnitude coefficient that large, cannot be held: the launch raises the status word (2), the step
+    moves nothing, and the same step on the other kernels gives the oracle's keep set."""
+    w = small(seq_lens=(300, 200))
+    inp = build_inputs(w)
+    if what == "key":
+        inp["caches"][1][0, int(inp["tables"][1][3]), 5, 1, 40] = 1.0e5     # K plane, one element of one row
+    else:
+        inp["qa"] = inp["qa"] * 1e6
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    print(f"magnitude overflow: {what}", flush=True)
+    before = [c.clone() for c in caches]
+    _, ws = ops.compress_step(kv, batch, sc, sel)
+    assert ws.status() == 2
+    for c, c0 in zip(caches, before):
+        assert torch.equal(c.view(torch.int16), c0.view(torch.int16))
+    for kernel in ("valu", "off"):
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+        keep, fin, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+        assert ws.status() == 0 and bool(torch.isfinite(fin[0, :50]).all())
+    keep = keep.cpu().long()
+    h = w.num_kv_heads
+    for b, t in enumerate(w.seq_lens):
+        k = min(w.budget, t)
+        oraw = oracle_raw(w, inp, b, t)
+        want, ofin = osel.group_keep_per_head(oraw, h, w.budget, window_size=w.window_size,
+                                              chunk_tokens=osel.score_chunk_tokens(w.block_size, t))
+        scale = float(ofin[torch.isfinite(ofin)].abs().max())
+        assert_keep_matches(keep[b * h:(b + 1) * h, :k], want, ofin, k, tie_tol=KEEP_TIE_TOL * scale)
+
+
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
     monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
     for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=256, kv_dtype="fp8"), {}), (dict(head_dim=64, kv_dtype="fp8"), {}),

@@ -480,7 +480,21 @@ CompactArgs make_args(const CompactLaunch& a) {
   // One list per workgroup: the ordered pass is a chain of dependent tiles per workgroup, so
   // with few sequences its run time is the chain length, and a chain over one head is
   // Hkv times shorter than one over whole token rows; with many sequences it is bound by
-  // the memory system either way (measured: same time).
+  // the memory system either way (16 x 16384 tokens x 36 layers, compaction alone, one process:
+  // 1.965 ms with one list, 2.02 with all eight).
+  // Tried and not kept, measured the same way (ordered + bulk, budget 2048 of 16384 tokens / 12000
+  // of 32768 / fp8 rows):
+  //  - the ordered pass cut into levels: with t0 = k and t(i+1) = entries below t(i), the
+  //    positions [t(i+1), t(i)) take their rows from [t(i), t(i-1)), disjoint ranges, so each level
+  //    is a flat gather without barriers between its tiles and only the last remainder needs the
+  //    tile order (levels deepest first, a workgroup barrier between them): 1.966 / 10.12 / 0.955
+  //    ms against 1.965 / 10.01 / 0.952.  The tile-by-tile order is not what bounds the pass.
+  //  - workgroups ordered so that all sequences of one layer's K (or V) tensor run next to each
+  //    other (a smaller set of pages in use at any time): 1.97 / 10.19 / 1.017 against
+  //    1.96 / 9.96 / 0.98, and 1.89 against 1.74 in a second process.
+  // What does move these figures is where the cache lies physically: the same virtual range freed
+  // and allocated again runs the same compaction in 1.69 to 1.98 ms (one box, one process), and
+  // physically contiguous allocations (hipDeviceMallocContiguous) show the same spread.
   c.lists_per_wg = 1;
   c.chunks_per_row = a.D * a.elem_bytes / 16;
   c.heads_per_slot = a.shared ? a.Hkv : 1;

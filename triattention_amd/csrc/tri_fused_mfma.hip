@@ -12,7 +12,8 @@
 // (query head, split): every fp32 coefficient is carried as three bf16 pieces
 // c = c1 + c2 + c3, so the products are exact and the sum is an fp32 accumulation of the
 // same terms the vector-unit kernel adds.  The magnitudes are evaluated on the vector unit
-// in fp32 (sqrt(k_r^2 + k_i^2)), cut into two bf16 pieces and contracted the same way.
+// in fp32 (sqrt(k_r^2 + k_i^2)), cut into two fp16 pieces and contracted the same way
+// (v_mfma_f32_16x16x32_f16 against fp16 pieces of the magnitude coefficients).
 // The three column groups of a query head are added with row rotations, which leaves every
 // token's four scores spread over the lanes exactly as the ring in LDS wants them.
 //
@@ -99,28 +100,9 @@ __device__ __forceinline__ void magnitudes4(const uint32_t (&x)[4], float* m) {
   }
 }
 
-// Two fp32 values -> packed bf16 (fp16 for fp16 keys; round to nearest even) and the fp32
-// remainders.  The packed halves are turned back into fp32 through their bit patterns, so the
-// subtraction sees exactly what was stored.
-template <int DT>
-__device__ __forceinline__ uint32_t split_pair(float x0, float x1, float& r0, float& r1) {
-  const f32x2 x = {x0, x1};
-  if constexpr (DT == TRI_KV_FP16) {
-    const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
-    r0 = x0 - (float)__builtin_bit_cast(_Float16, (unsigned short)(packed & 0xffffu));
-    r1 = x1 - (float)__builtin_bit_cast(_Float16, (unsigned short)(packed >> 16));
-    return packed;
-  } else {
-    const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
-    r0 = x0 - bf16_lo(packed);
-    r1 = x1 - bf16_hi(packed);
-    return packed;
-  }
-}
-
 // Two fp32 values -> packed fp16 and the fp32 remainders, the remainders by the
 // mixed-precision fused multiply-add, which reads the halves of the packed register as they
-// are (x - half is exact): four instructions per two values where the bf16 route needs six.
+// are (x - half is exact): four instructions per two values where a bf16 split needs six.
 __device__ __forceinline__ uint32_t split_pair_f16(float x0, float x1, float& r0, float& r1) {
   const f32x2 x = {x0, x1};
   const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
@@ -249,16 +231,16 @@ __global__ __launch_bounds__(kPrepThreads) void prep_mfma_kernel(const float* fo
             else if (IL) pair = slab_elem<DT>(2 * set + (e >> 2), kb, 2 * (e & 3)) >> 1;
             else pair = slab_elem<DT>(set, kb, e) & (F - 1);
           }
-          // One-byte keys: their magnitudes go through the fp16 matrix-core instruction (see
+          // The magnitudes go through the fp16 matrix-core instruction whatever the key type (see
           // compute_step), so the magnitude slabs are fp16 pieces.
-          const bool half_slab = DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= NS);
+          const bool half_slab = DT == TRI_KV_FP16 || o >= NS;
           v[e] = half_slab ? coefficient_piece<TRI_KV_FP16>(c[which * F + pair], sp)
                            : coefficient_piece<TRI_KV_BF16>(c[which * F + pair], sp);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const f32x2 x = {v[2 * e], v[2 * e + 1]};
-          if (DT == TRI_KV_FP16 || (DT == TRI_KV_FP8_E4M3 && o >= NS))
+          if (DT == TRI_KV_FP16 || o >= NS)
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
           else
             out[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
@@ -330,11 +312,11 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     for (int g = 0; g < QG; ++g)
 #pragma unroll
       for (int o = 0; o < NSO; ++o) B[g][o] = p[(g * NSO + o) * 64];
-    if constexpr (DT == TRI_KV_FP16 || DT == TRI_KV_FP8_E4M3) {
+    {
       // A coefficient beyond fp16's range (65504) arrives as an infinity: the scores of this
       // launch would be meaningless, so the status word is raised (the caller repeats the
       // step on the vector-unit kernels) and every wait of the launch gives up.  fp16 keys:
-      // all slabs; one-byte keys: the magnitude slabs.
+      // all slabs; otherwise the magnitude slabs.
       uint32_t bad = 0;
 #pragma unroll
       for (int g = 0; g < QG; ++g)
@@ -522,30 +504,22 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       }
       uint4 hi, lo;
       float r[8];
-      if constexpr (FP8) {
-        // The magnitudes of one-byte codes lie in [2^-9, 634]: fp16 holds them, and the fp16
-        // split is two instructions per pair cheaper (this kernel is bound by the vector unit).
-        hi.x = split_pair_f16(mag[0], mag[1], r[0], r[1]);
-        hi.y = split_pair_f16(mag[2], mag[3], r[2], r[3]);
-        hi.z = split_pair_f16(mag[4], mag[5], r[4], r[5]);
-        hi.w = split_pair_f16(mag[6], mag[7], r[6], r[7]);
+      // The magnitudes are cut into two fp16 pieces (22 bits; two bf16 pieces would carry 16) and
+      // go through the fp16 matrix-core instruction whatever the key type: the fp16 split is two
+      // instructions per pair cheaper than the bf16 one.  Magnitudes of one-byte codes lie in
+      // [2^-9, 634]; a two-byte key beyond fp16's range turns its scores into infinities or NaNs,
+      // which the check after every layer finds (status word 2: the caller repeats the step on the
+      // vector-unit kernels).
+      hi.x = split_pair_f16(mag[0], mag[1], r[0], r[1]);
+      hi.y = split_pair_f16(mag[2], mag[3], r[2], r[3]);
+      hi.z = split_pair_f16(mag[4], mag[5], r[4], r[5]);
+      hi.w = split_pair_f16(mag[6], mag[7], r[6], r[7]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const f32x2 x = {r[2 * i], r[2 * i + 1]};
-          (&lo.x)[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
-        }
-      } else {
-        hi.x = split_pair<DT>(mag[0], mag[1], r[0], r[1]);
-        hi.y = split_pair<DT>(mag[2], mag[3], r[2], r[3]);
-        hi.z = split_pair<DT>(mag[4], mag[5], r[4], r[5]);
-        hi.w = split_pair<DT>(mag[6], mag[7], r[6], r[7]);
-        float unused0, unused1;
-        lo.x = split_pair<DT>(r[0], r[1], unused0, unused1);
-        lo.y = split_pair<DT>(r[2], r[3], unused0, unused1);
-        lo.z = split_pair<DT>(r[4], r[5], unused0, unused1);
-        lo.w = split_pair<DT>(r[6], r[7], unused0, unused1);
+      for (int i = 0; i < 4; ++i) {
+        const f32x2 x = {r[2 * i], r[2 * i + 1]};
+        (&lo.x)[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
       }
-      constexpr int MT = FP8 ? TRI_KV_FP16 : DT;     // operand type of the magnitude MFMAs
+      constexpr int MT = TRI_KV_FP16;                // operand type of the magnitude MFMAs
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
         acc_e[g] = mfma_step<MT>(hi, B[g][NS + set], acc_e[g]);
@@ -736,6 +710,14 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     rotate(l, 0, rot_before_consume);
     if (l > l_begin) consume(l - 1);
     rotate(l, rot_before_consume, rotations);
+    if constexpr (!FP8) {
+      // A magnitude beyond fp16's range (or a key that is not finite) has left an infinity or a NaN
+      // in this layer's sums.
+      bool bad = false;
+#pragma unroll
+      for (int g = 0; g < QG; ++g) bad = bad || !(s2[g] < INFINITY);
+      if (__any(bad) && lane == 0) atomicExch(a.status, 2u);
+    }
     if (a.normalize) arrive(l);
     if (l + 1 < l_end) load_coefs(l + 1);
   }
