@@ -40,6 +40,8 @@ struct FusedPlan {
 };
 // Workgroups of the resident kernel the current device can hold at once (0: none).
 int fused_resident_workgroups();
+// The occupancy calculator's answer for the largest resident instance on the current device.
+bool fused_mfma_fits_device();
 // any_fill: plan the resident kernel even for a launch that would leave most CUs idle.
 FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, int aggregation, int Tmax,
                      int resident, bool any_fill);

@@ -418,6 +418,12 @@ int fused_resident_workgroups() {
   if (cached[dev] == 0) {
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
+    // The workgroups of a launch wait for each other, so all of them must be on the chip at once.
+    // That is assumed only where it can be checked: the occupancy calculator must place one
+    // workgroup of the largest instance on a CU, and no CU mask may be in force for the process
+    // (the CU count above does not show one); otherwise the two-pass kernels are used.
+    const bool masked = std::getenv("HSA_CU_MASK") || std::getenv("ROC_GLOBAL_CU_MASK");
+    if (masked || !fused_mfma_fits_device()) cus = 0;
     cached[dev] = cus > 0 ? cus : -1;
   }
   int n = cached[dev] > 0 ? cached[dev] : 0;

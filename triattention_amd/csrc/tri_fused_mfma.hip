@@ -792,6 +792,30 @@ hipError_t launch_mfma_t(FusedArgs& k, const uint4* bmat, const LaunchShape& sha
   return hipSuccess;
 }
 
+}  // namespace
+
+// Does the current device hold one resident workgroup per CU?  Asked once per device of the
+// runtime's occupancy calculator, for the instance with the largest ring (1024 + 192 tokens, eight
+// waves, 256 registers a lane): a part with less LDS per CU, or a runtime that gives the kernel
+// fewer resources than this file assumes, then takes the two-pass kernels instead of launching
+// workgroups that would wait for others that cannot start.
+bool fused_mfma_fits_device() {
+  const void* fn = reinterpret_cast<const void*>(&fused_mfma_kernel<TRI_KV_BF16, false, 1024, 192, 1, 4, kFusedWaves, 128>);
+  constexpr size_t lds = mfma_lds_bytes<1024, 192, 1, kFusedWaves>();
+  if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, kFusedWaves * kWave, lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return per_cu >= 1;
+}
+
+namespace {
+
 template <int DT, bool IL>
 hipError_t launch_mfma_tw(FusedArgs& k, const uint4* bmat, int tw, int waves, int head_dim, const LaunchShape& shape,
                           hipStream_t s) {
