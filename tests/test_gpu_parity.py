@@ -952,6 +952,39 @@ def test_resident_launches_on_two_streams_do_not_starve_each_other():
         assert torch.equal(keep, alone[i % 2][0]) and torch.equal(fin, alone[i % 2][1])
 
 
+def test_resident_launch_next_to_another_streams_kernels():
+    """A serving process keeps the GPU busy with its own kernels on other streams.  The resident
+    launch assumes that all its workgroups reach a CU; another stream's kernels only delay that
+    (they end), so steps issued while a second stream runs a queue of large matrix products finish
+    with a clean status and the same keep rows and caches as on an idle GPU."""
+    sel = ops.SelectConfig(window_size=12)
+    w, inp, caches, kv, batch, sc = _resident_batch(13)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    pristine = [c.clone() for c in caches]
+    keep0, ws = ops.compress_step(kv, batch, sc, sel)
+    assert ws.status() == 0
+    want = [c.clone() for c in caches]
+    side = torch.cuda.Stream()
+    a = torch.randn(6144, 6144, device=DEV, dtype=torch.bfloat16)
+    out = torch.empty_like(a)
+    torch.cuda.synchronize()
+    print("steps next to a queue of matrix products", flush=True)
+    for rep in range(4):
+        for c, p in zip(caches, pristine):
+            c.copy_(p)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for _ in range(60):
+                torch.matmul(a, a, out=out)
+        keep = torch.empty_like(keep0)
+        ops.compress_step(kv, batch, sc, sel, ws, keep)      # queued while the products run
+        torch.cuda.synchronize()
+        assert ws.status() == 0, f"repetition {rep}"
+        assert torch.equal(keep, keep0)
+        for c, x in zip(caches, want):
+            assert torch.equal(c.view(torch.int16), x.view(torch.int16))
+
+
 @pytest.mark.parametrize("case", ["fewer_launches_planned_than_needed", "device_length_beyond_max_seq_len"])
 def test_host_lengths_that_disagree_with_the_device_raise_the_status_word(case, monkeypatch):
     """A caller of the C ABI whose host copy of the lengths is stale: the planner sizes launches

@@ -77,6 +77,10 @@ class _DeviceStats:
 
 # Steady-state steps (a shape seen before) replay their launch sequence from a HIP graph.
 GRAPH_REPLAY = True
+# ... for steps whose scratch stays below this many bytes: every captured shape keeps scratch and keep
+# rows of its own (up to eight shapes a selector), and the steps that repeat are the small ones
+# (budget + divide_length tokens a request).
+GRAPH_MAX_SCRATCH_BYTES = 64 << 20
 GRAPH_COUNTS = {"captured": 0, "replayed": 0}     # process-wide, for tests and diagnostics
 
 
@@ -327,7 +331,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                     keep, ws = ops.compress_step(kv, batch, sc, sel, holder.get("ws"),
                                                  keep_buf[:rows * batch.max_budget].view(rows, batch.max_budget))
                     holder["ws"] = ws
-                    if GRAPH_REPLAY:
+                    if GRAPH_REPLAY and ws.bytes <= GRAPH_MAX_SCRATCH_BYTES:
                         if len(holder["graphs"]) >= 8:
                             holder["graphs"].pop(next(iter(holder["graphs"])))
                         holder["graphs"][key] = {"graph": None}
