@@ -31,9 +31,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # the same counters read for the 1 GiB copies of --copy-calibration).  Keyed by
 # (workload, path); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_qwen3_8b_36l_b16_16k", "two_pass"): (9_717_510 * 1024 * 2 + 1_184_256 * 1024,       # score_mean_kernel
-                                               "profiles/c1_step_hbm_counters.txt"),
-    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_477_735 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
+    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_482_130 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
                                                     "profiles/c1_step_hbm_counters.txt"),
 }
 
@@ -54,6 +52,12 @@ def parse_args():
     ap.add_argument("--seq-len", type=int, default=0,
                     help="override every sequence's cached length (e.g. budget + 128 for the steady-state step)")
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
+    ap.add_argument("--no-exact-pool", "--no-scattered-pool", dest="no_exact_pool", action="store_true",
+                    help="skip the second leg: the same step on a pool that holds exactly the live blocks")
+    ap.add_argument("--pool-occupancy", type=float, default=0.0,
+                    help="live blocks / blocks of the shared pool.  Default: the workload's own where it names one "
+                         "(config 3: 0.8), otherwise a pool four times the live blocks (at most 160 GiB): a serving "
+                         "engine's cache spans most of the HBM and a batch's blocks lie scattered over it")
     ap.add_argument("--kv-dtype", choices=["bf16", "fp16"], default="",
                     help="key/value dtype of the synthetic cache (default: the workload's own)")
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers")
@@ -245,6 +249,97 @@ def query_stats_leg(dev, heads: int = 32, tokens: int = 32768, dim: int = 128, c
             "query_bytes": nbytes, "gbs": nbytes / (med * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
+def pool_bytes_per_block(w) -> int:
+    return 2 * w.block_size * w.num_kv_heads * w.head_dim * (1 if w.kv_dtype == "fp8" else 2) * w.num_layers
+
+
+def default_pool_blocks(w) -> int:
+    """Four times the live blocks, at most 160 GiB over all layers."""
+    live = sum(w.blocks_per_seq)
+    return max(live, min(4 * live, (160 << 30) // pool_bytes_per_block(w)))
+
+
+def second_pool_leg(w2, args, dev, sc, sel, two_pass: bool):
+    """The same workload on a pool of another size (same sequences, same kernels, same algorithmic
+    bytes, other physical addresses): events around the whole step and its stages, restores outside
+    them."""
+    from triattention_amd import ops, synth
+    live = sum(w2.blocks_per_seq)
+    per_block = pool_bytes_per_block(w2)
+    tables = synth.make_block_tables(w2)
+    pool = synth.make_kv_pool(w2, tables, dev)
+    k_scales = v_scales = None
+    if w2.kv_dtype == "fp8":
+        caches, k_scales, v_scales = pool
+        kv = ops.PagedKV([c[0] for c in caches], [c[1] for c in caches], w2.rope_style, k_scales, v_scales)
+    else:
+        caches = pool
+        kv = ops.PagedKV.from_kv_caches(caches, w2.rope_style)
+    batch = ops.StepBatch(dev, w2.seq_lens, round_start=w2.seq_lens, budgets=w2.budget, block_tables=tables)
+    ws = ops.Workspace(kv, batch, sc)
+    rows = w2.num_seqs * w2.num_kv_heads
+    keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=dev)
+    fin_buf = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=dev)
+    raw_buf = None
+    if two_pass:
+        raw_buf = torch.empty(w2.num_seqs, w2.num_layers, batch.max_seq_len, w2.num_q_heads, dtype=torch.float32,
+                              device=dev)
+    nkeep_blocks = (w2.budget + w2.block_size - 1) // w2.block_size
+    ids = torch.tensor([b for tbl in tables for b in tbl[:nkeep_blocks]], device=dev, dtype=torch.long)
+    saved = [c[:, ids].clone() for c in caches]
+    saved_scales = None
+    if k_scales is not None:
+        slot = (ids.unsqueeze(1) * w2.block_size + torch.arange(w2.block_size, device=dev)).flatten()
+        saved_scales = [(ks[slot].clone(), vs[slot].clone()) for ks, vs in zip(k_scales, v_scales)]
+
+    def restore():
+        for i, c in enumerate(caches):
+            c[:, ids] = saved[i]
+            if saved_scales is not None:
+                k_scales[i][slot] = saved_scales[i][0]
+                v_scales[i][slot] = saved_scales[i][1]
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        if two_pass:
+            raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
+            if ev is not None:
+                ev[1].record()
+            ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
+        else:
+            ops.select_paged(kv, batch, sc, sel, ws, scores_out=fin_buf, want_keep=False)
+            if ev is not None:
+                ev[1].record()
+            ops.topk_batch(fin_buf, batch, w2.num_kv_heads, keep)
+        if ev is not None:
+            ev[2].record()
+        ops.compact(kv, batch, keep)
+        if ev is not None:
+            ev[3].record()
+
+    for _ in range(args.warmup):
+        step()
+        restore()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    for i in range(args.steps):
+        step(evs[i])
+        restore()
+    torch.cuda.synchronize()
+    if not two_pass and ws.status() != 0:
+        return {"error": "status word raised"}
+    mean = lambda xs: sum(xs) / len(xs)
+    ms = mean([e[0].elapsed_time(e[3]) for e in evs])
+    algo = w2.algorithmic_bytes()
+    gbs = algo["total"] / (ms * 1e-3) / 1e9
+    return {"pool_blocks_per_layer": w2.pool_blocks, "pool_occupancy": round(live / w2.pool_blocks, 4),
+            "pool_gib": round(w2.pool_blocks * per_block / 2**30, 1), "steps": args.steps, "ms_per_step": ms,
+            "stage_ms": {"score": mean([e[0].elapsed_time(e[1]) for e in evs]),
+                         "select" if two_pass else "topk": mean([e[1].elapsed_time(e[2]) for e in evs]),
+                         "compact": mean([e[2].elapsed_time(e[3]) for e in evs])},
+            "value": sum(w2.seq_lens) / (ms * 1e-3), "achieved_gbs": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -272,6 +367,20 @@ def main() -> int:
         if "fp8" in (args.kv_dtype, w.kv_dtype):
             raise SystemExit("--kv-dtype switches between bf16 and fp16; the fp8 workload is --config 4")
         w = w.scaled(name=f"{w.name}_{args.kv_dtype}", kv_dtype=args.kv_dtype)
+    # The shared pool.  A workload that names its own occupancy keeps it; otherwise the live blocks are
+    # scattered over a pool four times their number, and a second leg (below) runs the same step on a
+    # pool that holds exactly the live blocks.
+    w_exact = None
+    if args.pool_occupancy > 0:
+        if not 0.0 < args.pool_occupancy <= 1.0:
+            raise SystemExit("--pool-occupancy is a fraction in (0, 1]")
+        w = w.scaled(pool_occupancy=args.pool_occupancy)
+    elif w.pool_occupancy == 1.0:
+        live = sum(w.blocks_per_seq)
+        blocks = default_pool_blocks(w)
+        if blocks > live:
+            w_exact = w
+            w = w.scaled(pool_occupancy=live / blocks)
     t_setup = time.perf_counter()
     tables = synth.make_block_tables(w)
     pool = synth.make_kv_pool(w, tables, dev)
@@ -454,7 +563,9 @@ def main() -> int:
         "config": {"workload": w.name, "layers": w.num_layers, "sequences": w.num_seqs,
                    "tokens_per_sequence": max(w.seq_lens), "budget": w.budget, "kv_heads": w.num_kv_heads,
                    "q_heads": w.num_q_heads, "head_dim": w.head_dim, "block_size": w.block_size,
-                   "kv_dtype": w.kv_dtype},
+                   "kv_dtype": w.kv_dtype, "pool_blocks_per_layer": w.pool_blocks,
+                   "pool_occupancy": round(sum(w.blocks_per_seq) / w.pool_blocks, 4),
+                   "pool_gib": round(w.pool_blocks * pool_bytes_per_block(w) / 2**30, 1)},
         "achieved_gbs": step_gbs,
         "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "algorithmic_bytes": algo,
@@ -505,9 +616,12 @@ def main() -> int:
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
         out["hook_batch_call"] = hook_latency(w, dev, calls=20, requests=len(w.seq_lens))
-    if not args.no_cpu_baseline:
-        del saved, caches, pool
+    del saved, caches, pool, kv, restore, step
+    torch.cuda.empty_cache()
+    if w_exact is not None and not args.no_exact_pool:
+        out["exact_pool"] = second_pool_leg(w_exact, args, dev, sc, sel, two_pass)
         torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
         out["cpu_baseline"], oracle_keep = cpu_baseline(w, args.cpu_layers, seq0)
         if oracle_keep is not None:
             okeep, ofin = oracle_keep
