@@ -666,3 +666,52 @@ def test_keep_tensors_from_the_selector_are_remembered_by_identity():
     del keep
     gc.collect()
     assert key not in kc._VALIDATED_KEEP
+
+
+def test_header_is_plain_c_and_a_c_program_links_the_library(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 with warnings as errors, and a C program
+    that includes it links against the library, reads the ABI version, takes the struct sizes the
+    Python mirror uses and gets the documented refusal (no compute call: there is no GPU here)."""
+    import ctypes as C
+    import shutil
+    import subprocess
+    from triattention_amd import build as tri_build
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    _lib.load()
+    root = Path(__file__).resolve().parents[1]
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "triattention_hip.h"
+int main(void) {
+  tri_kv_layout kv; tri_batch b; tri_score_params sp; tri_select_params sel;
+  memset(&kv, 0, sizeof kv); memset(&b, 0, sizeof b); memset(&sp, 0, sizeof sp); memset(&sel, 0, sizeof sel);
+  printf("abi %d %d\n", tri_abi_version(), TRI_ABI_VERSION);
+  printf("sizes %zu %zu %zu %zu\n", sizeof kv, sizeof b, sizeof sp, sizeof sel);
+  printf("bytes %llu\n", (unsigned long long)tri_workspace_bytes(&kv, &b, &sp));
+  int rc = tri_compress_step(&kv, &b, &sp, &sel, NULL, NULL, 0, NULL);
+  printf("rc %d msg %s\n", rc, tri_last_error());
+  rc = tri_compress_step_static(NULL, &b, &sp, &sel, NULL, NULL, NULL);
+  printf("rc %d msg %s\n", rc, tri_last_error());
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    libdir = tri_build.LIB_PATH.parent
+    cmd = [gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{root / 'include'}", str(src), "-o", str(exe),
+           f"-L{libdir}", "-ltriattention_hip", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib",
+           "-Wl,--allow-shlib-undefined"]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.splitlines()
+    assert lines[0] == f"abi {_lib.ABI_VERSION} {_lib.ABI_VERSION}"
+    sizes = [int(x) for x in lines[1].split()[1:]]
+    assert sizes == [C.sizeof(_lib.KvLayout), C.sizeof(_lib.Batch), C.sizeof(_lib.ScoreParams), C.sizeof(_lib.SelectParams)]
+    assert lines[2] == "bytes 0"
+    assert lines[3].startswith("rc -") and "bad layer/head count" in lines[3]
+    assert lines[4].startswith("rc -") and "kv layout is NULL" in lines[4]
