@@ -139,7 +139,8 @@ uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
  * tri_compress_step clear it and the resident kernel sets it to non-zero if one of its
  * bounded waits on another workgroup expired (1), or if a magnitude coefficient (with fp16
  * keys: any coefficient) or a key's magnitude does not fit the fp16 pieces the matrix-core
- * kernel holds it in, i.e. exceeds 65504 (2)
+ * kernel holds it in, i.e. exceeds 65504, or if the keys of a layer are so small throughout
+ * (no magnitude of 2^-9 among those looked at) that the pieces would be subnormals (2)
  * (results are then invalid; the compaction
  * inside tri_compress_step sees the word and moves nothing, so the cache is intact and
  * the caller can repeat the step with TRIATTN_RESIDENT_KERNEL=off).  The caller may read

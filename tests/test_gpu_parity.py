@@ -1112,16 +1112,19 @@ def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
     assert ws.status() == 0
 
 
-@pytest.mark.parametrize("what", ["key", "coefficient"])
+@pytest.mark.parametrize("what", ["key", "coefficient", "tiny_keys"])
 def test_magnitudes_beyond_half_range_raise_the_status_word(monkeypatch, what):
     """Whatever the key type, the matrix-core kernel carries the magnitudes |k_f| and their
-    coefficients as fp16 pieces.  A bf16 key whose magnitude exceeds 65504, or statistics that make a
-    magnitude coefficient that large, cannot be held: the launch raises the status word (2), the step
+    coefficients as fp16 pieces.  A bf16 key whose magnitude exceeds 65504, statistics that make a
+    magnitude coefficient that large, or keys so small throughout that their magnitudes are fp16
+    subnormals (scaled by 2^-14) cannot be held: the launch raises the status word (2), the step
     moves nothing, and the same step on the other kernels gives the oracle's keep set."""
     w = small(seq_lens=(300, 200))
     inp = build_inputs(w)
     if what == "key":
         inp["caches"][1][0, int(inp["tables"][1][3]), 5, 1, 40] = 1.0e5     # K plane, one element of one row
+    elif what == "tiny_keys":
+        inp["caches"] = [(c.float() * 2.0 ** -14).to(c.dtype) for c in inp["caches"]]
     else:
         inp["qa"] = inp["qa"] * 1e6
     caches, kv, batch, sc = device_objects(w, inp, DEV)

@@ -425,6 +425,9 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   float s1[QG], s2[QG];
 #pragma unroll
   for (int g = 0; g < QG; ++g) { s1[g] = 0.f; s2[g] = 0.f; }
+  // Largest of a sample of the layer's magnitudes (their first fp16 pieces), per lane; see the check
+  // after every layer.
+  f16x2 mag_seen = {(_Float16)0.f, (_Float16)0.f};
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
   auto compute_step = [&](const StepData<DT, HD>& raw, int l, int t) __attribute__((always_inline)) {
@@ -519,6 +522,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
         const f32x2 x = {r[2 * i], r[2 * i + 1]};
         (&lo.x)[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
       }
+      if constexpr (!FP8) mag_seen = __builtin_elementwise_max(mag_seen, __builtin_bit_cast(f16x2, hi.x));
       constexpr int MT = TRI_KV_FP16;                // operand type of the magnitude MFMAs
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
@@ -716,7 +720,15 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       bool bad = false;
 #pragma unroll
       for (int g = 0; g < QG; ++g) bad = bad || !(s2[g] < INFINITY);
-      if (__any(bad) && lane == 0) atomicExch(a.status, 2u);
+      // The other end of fp16's range: below 2^-14 the first piece is a subnormal and below 2^-3 the
+      // second one is, so magnitudes carry an absolute error of up to 2^-25 whatever their size.
+      // Against keys of ordinary size that is nothing (scaled by 2^-10, magnitudes around 2^-9, the
+      // selection scores are as close to the fp64 ones as unscaled); keys that are all tiny (scaled by
+      // 2^-14: errors of 2e-4 of the largest score) are left to the other kernels: no lane of the
+      // wave has seen a magnitude of 2^-9 in this layer (one pair in eight is looked at).
+      const bool seen = (float)mag_seen[0] >= 0x1p-9f || (float)mag_seen[1] >= 0x1p-9f;
+      mag_seen = f16x2{(_Float16)0.f, (_Float16)0.f};
+      if ((__any(bad) || !__any(seen)) && lane == 0) atomicExch(a.status, 2u);
     }
     if (a.normalize) arrive(l);
     if (l + 1 < l_end) load_coefs(l + 1);
