@@ -154,6 +154,25 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         return ops.PagedKV.for_kv_caches(caches, rope_style=_stats().rope_style,
                                           kv_axis=hints.pop() if len(hints) == 1 else None)
 
+    def _resident_failed(status: int) -> bool:
+        """Book-keeping after a resident launch.  An expired wait (1) means the launch was starved
+        of CUs (a shared or masked GPU): that is still so at the next step and every such launch costs
+        its full wait limit, so the selector stays on the two-pass kernels from then on.  A value
+        outside fp16's range (2) ends a launch at once; it may be this model's statistics (every
+        step) or one odd key (this step), so the selector gives up on the resident kernels after
+        three such steps in a row.  A disagreement between host and device lengths (3) concerns one
+        step."""
+        if status == 0:
+            holder["range_failures"] = 0
+            return False
+        if status == 1:
+            holder["resident_ok"] = False
+        elif status == 2:
+            holder["range_failures"] = holder.get("range_failures", 0) + 1
+            if holder["range_failures"] >= 3:
+                holder["resident_ok"] = False
+        return True
+
     def _score_and_select(kv: ops.PagedKV, layer_ids: tuple, block_ids, total_tokens: int, prefill_len: int,
                           protect_prefill: bool, round_start: int, k: int, layer_reduce, group_reduce: str,
                           score_heads: int, shared: bool) -> torch.Tensor:
@@ -172,13 +191,9 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         try:
             resident = ops.select_path(kv, batch, sc, sel) != "two_pass"   # (a single request: only when forced)
             keep, _, ws = ops.select_paged(kv, batch, sc, sel)
-            if resident and ws.status() != 0:
-                # A wait inside the resident kernel expired (or a coefficient did not fit its operand
-                # type): the keep lists mean nothing.  Nothing has been moved yet; score again on the
-                # kernels that do not wait for each other, and stay on them: whatever starved the
-                # launch (a shared or masked GPU) or overflowed (this model's statistics) is still
-                # there at the next step, and every failed launch costs its full wait limit.
-                holder["resident_ok"] = False
+            if resident and _resident_failed(ws.status()):
+                # The keep lists mean nothing.  Nothing has been moved yet; score again on the
+                # kernels that do not wait for each other.
                 sel.allow_resident = False
                 keep, _, ws = ops.select_paged(kv, batch, sc, sel, ws)
         except Exception as exc:
@@ -347,8 +362,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                     GRAPH_COUNTS["captured"] += 1
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
-        if resident and ws.status() != 0:
-            holder["resident_ok"] = False     # later steps of this selector go straight to the two-pass kernels
+        if resident and _resident_failed(ws.status()):
             raise ResidentLaunchFailed("a wait inside the resident kernel expired; the caches were left untouched")
         h = kv.num_kv_heads
         keep = keep.to(torch.long)           # one conversion; the per-request results are views
