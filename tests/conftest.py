@@ -40,7 +40,7 @@ def pytest_terminal_summary(terminalreporter):
         return
     swapped = sum(s for s, _ in helpers.SWAPS.values())
     compared = sum(c for _, c in helpers.SWAPS.values())
-    cases = sorted(name for name, (s, _) in helpers.SWAPS.items() if s)
+    cases = sorted(f"{name} {s}/{c}" for name, (s, c) in helpers.SWAPS.items() if s)
     terminalreporter.write_line(
         f"near-tie swaps: {swapped} of {compared} kept indices in {len(helpers.SWAPS)} comparisons"
         + (f" (cases: {', '.join(cases)})" if cases else ""))
