@@ -259,83 +259,115 @@ def default_pool_blocks(w) -> int:
     return max(live, min(4 * live, (160 << 30) // pool_bytes_per_block(w)))
 
 
-def second_pool_leg(w2, args, dev, sc, sel, two_pass: bool):
-    """The same workload on a pool of another size (same sequences, same kernels, same algorithmic
-    bytes, other physical addresses): events around the whole step and its stages, restores outside
-    them."""
-    from triattention_amd import ops, synth
-    live = sum(w2.blocks_per_seq)
-    per_block = pool_bytes_per_block(w2)
-    tables = synth.make_block_tables(w2)
-    pool = synth.make_kv_pool(w2, tables, dev)
-    k_scales = v_scales = None
-    if w2.kv_dtype == "fp8":
-        caches, k_scales, v_scales = pool
-        kv = ops.PagedKV([c[0] for c in caches], [c[1] for c in caches], w2.rope_style, k_scales, v_scales)
-    else:
-        caches = pool
-        kv = ops.PagedKV.from_kv_caches(caches, w2.rope_style)
-    batch = ops.StepBatch(dev, w2.seq_lens, round_start=w2.seq_lens, budgets=w2.budget, block_tables=tables)
-    ws = ops.Workspace(kv, batch, sc)
-    rows = w2.num_seqs * w2.num_kv_heads
-    keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=dev)
-    fin_buf = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=dev)
-    raw_buf = None
-    if two_pass:
-        raw_buf = torch.empty(w2.num_seqs, w2.num_layers, batch.max_seq_len, w2.num_q_heads, dtype=torch.float32,
-                              device=dev)
-    nkeep_blocks = (w2.budget + w2.block_size - 1) // w2.block_size
-    ids = torch.tensor([b for tbl in tables for b in tbl[:nkeep_blocks]], device=dev, dtype=torch.long)
-    saved = [c[:, ids].clone() for c in caches]
-    saved_scales = None
-    if k_scales is not None:
-        slot = (ids.unsqueeze(1) * w2.block_size + torch.arange(w2.block_size, device=dev)).flatten()
-        saved_scales = [(ks[slot].clone(), vs[slot].clone()) for ks, vs in zip(k_scales, v_scales)]
+class StepRun:
+    """One workload resident on the device, and the step that is timed on it.
 
-    def restore():
-        for i, c in enumerate(caches):
-            c[:, ids] = saved[i]
-            if saved_scales is not None:
-                k_scales[i][slot] = saved_scales[i][0]
-                v_scales[i][slot] = saved_scales[i][1]
+    Stage boundaries (events): 0 | scores of every key -> selection scores | 1 | top-k | 2 |
+    compaction | 3.  Default path: ``select_paged`` (one resident kernel when the shape has one,
+    raw scores stay in LDS); ``two_pass``: ``score_paged`` writes the raw scores, ``select``
+    normalises and reduces.  Compaction is destructive, so the blocks it overwrites (the first
+    ceil(k / block_size) of every sequence) are saved once and restored between steps."""
 
-    def step(ev=None):
-        if ev is not None:
-            ev[0].record()
-        if two_pass:
-            raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
-            if ev is not None:
-                ev[1].record()
-            ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
+    def __init__(self, w, dev, sc, sel, force_two_pass: bool):
+        from triattention_amd import ops, synth
+        self.ops, self.w, self.sc, self.sel = ops, w, sc, sel
+        self.tables = synth.make_block_tables(w)
+        pool = synth.make_kv_pool(w, self.tables, dev)
+        self.k_scales = self.v_scales = None
+        if w.kv_dtype == "fp8":
+            self.caches, self.k_scales, self.v_scales = pool
+            self.kv = ops.PagedKV([c[0] for c in self.caches], [c[1] for c in self.caches], w.rope_style,
+                                  self.k_scales, self.v_scales)
         else:
-            ops.select_paged(kv, batch, sc, sel, ws, scores_out=fin_buf, want_keep=False)
-            if ev is not None:
-                ev[1].record()
-            ops.topk_batch(fin_buf, batch, w2.num_kv_heads, keep)
-        if ev is not None:
-            ev[2].record()
-        ops.compact(kv, batch, keep)
-        if ev is not None:
-            ev[3].record()
+            self.caches = pool
+            self.kv = ops.PagedKV.from_kv_caches(self.caches, w.rope_style)
+        self.batch = ops.StepBatch(dev, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=self.tables)
+        self.ws = ops.Workspace(self.kv, self.batch, sc)
+        rows = w.num_seqs * w.num_kv_heads
+        self.keep = torch.empty(rows, self.batch.max_budget, dtype=torch.int32, device=dev)
+        self.fin_buf = torch.empty(rows, self.batch.max_seq_len, dtype=torch.float32, device=dev)
+        self.path = "two_pass" if force_two_pass else ops.select_path(self.kv, self.batch, sc, sel)
+        self.two_pass = self.path == "two_pass"
+        self.raw_buf = None
+        if self.two_pass:
+            self.raw_buf = torch.empty(w.num_seqs, w.num_layers, self.batch.max_seq_len, w.num_q_heads,
+                                       dtype=torch.float32, device=dev)
+        nkeep_blocks = (w.budget + w.block_size - 1) // w.block_size
+        self.ids = torch.tensor([b for tbl in self.tables for b in tbl[:nkeep_blocks]], device=dev, dtype=torch.long)
+        self.saved = [c[:, self.ids].clone() for c in self.caches]
+        self.saved_scales = None
+        if self.k_scales is not None:
+            self.slot = (self.ids.unsqueeze(1) * w.block_size + torch.arange(w.block_size, device=dev)).flatten()
+            self.saved_scales = [(ks[self.slot].clone(), vs[self.slot].clone())
+                                 for ks, vs in zip(self.k_scales, self.v_scales)]
+        torch.cuda.synchronize()
 
-    for _ in range(args.warmup):
-        step()
-        restore()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
-    for i in range(args.steps):
-        step(evs[i])
-        restore()
-    torch.cuda.synchronize()
-    if not two_pass and ws.status() != 0:
+    def restore(self):
+        for i, c in enumerate(self.caches):
+            c[:, self.ids] = self.saved[i]
+            if self.saved_scales is not None:
+                self.k_scales[i][self.slot] = self.saved_scales[i][0]
+                self.v_scales[i][self.slot] = self.saved_scales[i][1]
+
+    def step(self, events=None):
+        ops = self.ops
+        if events is not None:
+            events[0].record()
+        if self.two_pass:
+            raw, _ = ops.score_paged(self.kv, self.batch, self.sc, self.ws, out=self.raw_buf)
+            if events is not None:
+                events[1].record()
+            ops.select(self.kv, self.batch, self.sc, self.sel, raw, self.ws, keep=self.keep)
+        else:
+            ops.select_paged(self.kv, self.batch, self.sc, self.sel, self.ws, scores_out=self.fin_buf, want_keep=False)
+            if events is not None:
+                events[1].record()
+            ops.topk_batch(self.fin_buf, self.batch, self.w.num_kv_heads, self.keep)
+        if events is not None:
+            events[2].record()
+        ops.compact(self.kv, self.batch, self.keep)
+        if events is not None:
+            events[3].record()
+
+    def timed(self, warmup: int, steps: int):
+        """``warmup`` untimed steps, then ``steps`` timed ones.  Everything is enqueued asynchronously
+        on one stream: restore(i-1), then the events and kernels of step i.  The host runs ahead while
+        the restore copies execute, so the event pairs bracket GPU time only and restores stay outside
+        every timed interval.  Returns (events per step, wall seconds of the timed region)."""
+        for _ in range(warmup):
+            self.step()
+            self.restore()
+        torch.cuda.synchronize()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+        wall0 = time.perf_counter()
+        for i in range(steps):
+            self.step(evs[i])
+            if i + 1 < steps:
+                self.restore()
+        torch.cuda.synchronize()
+        return evs, time.perf_counter() - wall0
+
+    def status_raised(self) -> bool:
+        return not self.two_pass and self.ws.status() != 0
+
+
+def second_pool_leg(w2, args, dev, sc, sel, force_two_pass: bool):
+    """The same workload on a pool of another size (same sequences, same kernels, same algorithmic
+    bytes, other physical addresses)."""
+    run = StepRun(w2, dev, sc, sel, force_two_pass)
+    evs, _ = run.timed(args.warmup, args.steps)
+    if run.status_raised():
         return {"error": "status word raised"}
     mean = lambda xs: sum(xs) / len(xs)
     ms = mean([e[0].elapsed_time(e[3]) for e in evs])
     algo = w2.algorithmic_bytes()
     gbs = algo["total"] / (ms * 1e-3) / 1e9
-    return {"pool_blocks_per_layer": w2.pool_blocks, "pool_occupancy": round(live / w2.pool_blocks, 4),
-            "pool_gib": round(w2.pool_blocks * per_block / 2**30, 1), "steps": args.steps, "ms_per_step": ms,
+    return {"pool_blocks_per_layer": w2.pool_blocks,
+            "pool_occupancy": round(sum(w2.blocks_per_seq) / w2.pool_blocks, 4),
+            "pool_gib": round(w2.pool_blocks * pool_bytes_per_block(w2) / 2**30, 1), "steps": args.steps,
+            "ms_per_step": ms,
             "stage_ms": {"score": mean([e[0].elapsed_time(e[1]) for e in evs]),
-                         "select" if two_pass else "topk": mean([e[1].elapsed_time(e[2]) for e in evs]),
+                         "select" if run.two_pass else "topk": mean([e[1].elapsed_time(e[2]) for e in evs]),
                          "compact": mean([e[2].elapsed_time(e[3]) for e in evs])},
             "value": sum(w2.seq_lens) / (ms * 1e-3), "achieved_gbs": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
 
@@ -382,88 +414,17 @@ def main() -> int:
             w_exact = w
             w = w.scaled(pool_occupancy=live / blocks)
     t_setup = time.perf_counter()
-    tables = synth.make_block_tables(w)
-    pool = synth.make_kv_pool(w, tables, dev)
-    if w.kv_dtype == "fp8":
-        caches, k_scales, v_scales = pool
-        kv = ops.PagedKV([c[0] for c in caches], [c[1] for c in caches], w.rope_style, k_scales, v_scales)
-    else:
-        caches = pool
-        kv = ops.PagedKV.from_kv_caches(caches, w.rope_style)
     qc, qa = synth.make_stats(w, dev)
     fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2, device=dev)
     sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev),
                          args.aggregation)
     sel = ops.SelectConfig(window_size=w.window_size)
-    batch = ops.StepBatch(dev, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=tables)
-    ws = ops.Workspace(kv, batch, sc)
-    keep = torch.empty(w.num_seqs * w.num_kv_heads, batch.max_budget, dtype=torch.int32, device=dev)
-
-    # Blocks that compaction overwrites (the first ceil(k/bs) of every sequence), saved for restore.
-    nkeep_blocks = (w.budget + w.block_size - 1) // w.block_size
-    ids = torch.tensor([b for tbl in tables for b in tbl[:nkeep_blocks]], device=dev, dtype=torch.long)
-    saved = [c[:, ids].clone() for c in caches]
-    saved_scales = None
-    if w.kv_dtype == "fp8":
-        slot = (ids.unsqueeze(1) * w.block_size + torch.arange(w.block_size, device=dev)).flatten()
-        saved_scales = [(ks[slot].clone(), vs[slot].clone()) for ks, vs in zip(k_scales, v_scales)]
-    torch.cuda.synchronize()
+    run = StepRun(w, dev, sc, sel, args.two_pass)
     setup_s = time.perf_counter() - t_setup
+    tables, caches, kv, batch, ws, keep, fin_buf = run.tables, run.caches, run.kv, run.batch, run.ws, run.keep, run.fin_buf
+    path, two_pass, restore, step = run.path, run.two_pass, run.restore, run.step
 
-    def restore():
-        for i, c in enumerate(caches):
-            c[:, ids] = saved[i]
-            if saved_scales is not None:
-                k_scales[i][slot] = saved_scales[i][0]
-                v_scales[i][slot] = saved_scales[i][1]
-
-    # Stage boundaries (events): 0 | scores of every key -> selection scores | 1 | top-k | 2 | compaction | 3.
-    # Default: select_paged (one resident kernel when the shape has one, raw scores stay in
-    # LDS).  --two-pass: score_paged writes the raw scores, select normalises and reduces.
-    rows = w.num_seqs * w.num_kv_heads
-    fin_buf = torch.empty(rows, batch.max_seq_len, dtype=torch.float32, device=dev)
-    path = "two_pass" if args.two_pass else ops.select_path(kv, batch, sc, sel)
-    two_pass = path == "two_pass"
-    raw_buf = None
-    if two_pass:
-        raw_buf = torch.empty(w.num_seqs, w.num_layers, batch.max_seq_len, w.num_q_heads, dtype=torch.float32,
-                              device=dev)
-
-    def step(events=None):
-        if events is not None:
-            events[0].record()
-        if two_pass:
-            raw, _ = ops.score_paged(kv, batch, sc, ws, out=raw_buf)
-            if events is not None:
-                events[1].record()
-            ops.select(kv, batch, sc, sel, raw, ws, keep=keep)
-        else:
-            ops.select_paged(kv, batch, sc, sel, ws, scores_out=fin_buf, want_keep=False)
-            if events is not None:
-                events[1].record()
-            ops.topk_batch(fin_buf, batch, w.num_kv_heads, keep)
-        if events is not None:
-            events[2].record()
-        ops.compact(kv, batch, keep)
-        if events is not None:
-            events[3].record()
-
-    for _ in range(args.warmup):
-        step()
-        restore()
-    torch.cuda.synchronize()
-
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
-    wall0 = time.perf_counter()
-    # Everything is enqueued asynchronously on one stream: restore(i-1), then the events
-    # and kernels of step i.  The host runs ahead while the restore copies execute, so the
-    # event pairs bracket GPU time only and restores stay outside every timed interval.
-    for i in range(args.steps):
-        step(evs[i])
-        if i + 1 < args.steps:
-            restore()
-    torch.cuda.synchronize()
-    wall_s = time.perf_counter() - wall0
+    evs, wall_s = run.timed(args.warmup, args.steps)
 
     ms = lambda a, b: a.elapsed_time(b)
     step_ms = [ms(e[0], e[3]) for e in evs]
@@ -616,10 +577,10 @@ def main() -> int:
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
         out["hook_batch_call"] = hook_latency(w, dev, calls=20, requests=len(w.seq_lens))
-    del saved, caches, pool, kv, restore, step
+    del run, tables, caches, kv, batch, ws, keep, fin_buf, restore, step
     torch.cuda.empty_cache()
     if w_exact is not None and not args.no_exact_pool:
-        out["exact_pool"] = second_pool_leg(w_exact, args, dev, sc, sel, two_pass)
+        out["exact_pool"] = second_pool_leg(w_exact, args, dev, sc, sel, args.two_pass)
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"], oracle_keep = cpu_baseline(w, args.cpu_layers, seq0)
