@@ -430,7 +430,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   f16x2 mag_seen = {(_Float16)0.f, (_Float16)0.f};
   // Scores of the 16 tokens of a step: MFMAs over keys and magnitudes, split columns added
   // by row rotations; lane (j, kb) ends up with the score of token 4*kb + j/4, query head j%4.
-  auto compute_step = [&](const StepData<DT, HD>& raw, int l, int t) __attribute__((always_inline)) {
+  auto compute_step = [&](const StepData<DT, HD>& raw, int l, int t, int which) __attribute__((always_inline)) {
     // The four bf16 A operands of the step as dwords (two elements each): the loaded
     // registers for bf16 keys, one conversion per dword (exact) for fp8 keys.
     uint32_t w[NS][4];
@@ -522,7 +522,8 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
         const f32x2 x = {r[2 * i], r[2 * i + 1]};
         (&lo.x)[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
       }
-      if constexpr (!FP8) mag_seen = __builtin_elementwise_max(mag_seen, __builtin_bit_cast(f16x2, hi.x));
+      if constexpr (!FP8)   // `which` is the step buffer's number: a constant after unrolling
+        mag_seen = __builtin_elementwise_max(mag_seen, __builtin_bit_cast(f16x2, (&hi.x)[which & 3]));
       constexpr int MT = TRI_KV_FP16;                // operand type of the magnitude MFMAs
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
@@ -685,8 +686,8 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   const int nsteps = (ntok + 15) >> 4;
   const int rotations = (nsteps + NB - 1) / NB;
   const int rot_before_consume = min(SL / (16 * NB), rotations);
-  auto score = [&](const StepData<DT, HD>& d, int l, int slot) __attribute__((always_inline)) {
-    if (slot < nsteps) compute_step(d, l, slot * 16);
+  auto score = [&](const StepData<DT, HD>& d, int l, int slot, int which) __attribute__((always_inline)) {
+    if (slot < nsteps) compute_step(d, l, slot * 16, which);
   };
   StepData<DT, HD> buf[NB];
   LayerBase base_cur = layer_base(l_begin), base_next = base_cur;
@@ -697,7 +698,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       const int s0 = wrap ? 0 : (r + 1) * NB;
 #pragma unroll
       for (int i = 0; i < NB; ++i) {
-        score(buf[i], l, r * NB + i);
+        score(buf[i], l, r * NB + i, i);
         load_step(buf[i], lb, min(s0 + i, nsteps - 1) * 16);
       }
     }
@@ -725,7 +726,8 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       // Against keys of ordinary size that is nothing (scaled by 2^-10, magnitudes around 2^-9, the
       // selection scores are as close to the fp64 ones as unscaled); keys that are all tiny (scaled by
       // 2^-14: errors of 2e-4 of the largest score) are left to the other kernels: no lane of the
-      // wave has seen a magnitude of 2^-9 in this layer (one pair in eight is looked at).
+      // wave has seen a magnitude of 2^-9 in this layer (of every step one pair in four is looked at,
+      // another one in each of the step buffers, so every frequency pair is among them).
       const bool seen = (float)mag_seen[0] >= 0x1p-9f || (float)mag_seen[1] >= 0x1p-9f;
       mag_seen = f16x2{(_Float16)0.f, (_Float16)0.f};
       if ((__any(bad) || !__any(seen)) && lane == 0) atomicExch(a.status, 2u);
