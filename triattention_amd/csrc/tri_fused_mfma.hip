@@ -290,7 +290,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
   const int seq_tiles = ceil_div(T, a.tile_tokens);
   const int heads_here = min(8, a.Hkv - chunk * 8);
 
-  float* ring = lds + wave * (RING * RQ);                      // [RING][query heads of the KV head]
+  float* ring = lds + wave * (RING * RQ);                      // [QG][RING][4 query heads]
   float* part = lds + W * (RING * RQ);                         // [waves][64][QG][2]
   float* stats = part + W * 128 * QG;                          // [2][32*QG score heads][2]
   uint32_t* ctl = reinterpret_cast<uint32_t*>(stats + 128 * QG);  // arrive count, claimed, ready
@@ -421,7 +421,11 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
     }
   };
 
-  const uint32_t lane_ring = (uint32_t)(4 * kb + rsel) * RQ + q;
+  // Ring of this wave: [group of four query heads][RING tokens][4], so that the 64 lanes of a store
+  // (16 tokens x 4 heads of one group) cover 64 consecutive words and the 16-byte reads of
+  // consecutive tokens are 16 bytes apart, whatever the number of groups (with [RING][8] the stores of
+  // one group fell on half the banks; it does not show in the kernel's time).
+  const uint32_t lane_ring = (uint32_t)(4 * kb + rsel) * 4 + q;
   float s1[QG], s2[QG];
 #pragma unroll
   for (int g = 0; g < QG; ++g) { s1[g] = 0.f; s2[g] = 0.f; }
@@ -547,7 +551,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       }
       if (FP8) v *= raw.scale;
       if (4 * g + q < a.G && tl < ntok) {
-        ring[slot0 * RQ + lane_ring + 4 * g] = v;
+        ring[(uint32_t)g * (RING * 4) + slot0 * 4 + lane_ring] = v;
         s1[g] += v;
         s2[g] = fmaf(v, v, s2[g]);
       }
@@ -653,7 +657,7 @@ void fused_mfma_kernel(FusedArgs a, const uint4* bmat) {
       float xs[RQ];
 #pragma unroll
       for (int g = 0; g < QG; ++g) {
-        const float4 x = *reinterpret_cast<const float4*>(&ring[((uint32_t)(l * TW + tl) % RING) * RQ + 4 * g]);
+        const float4 x = *reinterpret_cast<const float4*>(&ring[(uint32_t)g * (RING * 4) + ((uint32_t)(l * TW + tl) % RING) * 4]);
         xs[4 * g] = x.x; xs[4 * g + 1] = x.y; xs[4 * g + 2] = x.z; xs[4 * g + 3] = x.w;
       }
       float v;
