@@ -382,6 +382,8 @@ def main() -> int:
         print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
         return 2
 
+    from triattention_amd import build as tri_build
+    tri_build.ensure_built()          # loads what is built; builds only when there is no library at all
     from triattention_amd import ops, synth
 
     dev = torch.device("cuda:0")

@@ -18,6 +18,12 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """Tests load the library that is built; only when there is none do they build it."""
+    from triattention_amd import build as tri_build
+    tri_build.ensure_built()
+
+
 def pytest_collection_modifyitems(config, items):
     if torch.cuda.is_available():
         return

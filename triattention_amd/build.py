@@ -57,6 +57,15 @@ def build(verbose: bool = True, jobs: int | None = None) -> Path:
     return LIB_PATH
 
 
+def ensure_built(verbose: bool = False) -> Path:
+    """For tests, the smoke run and the benchmark: build the library when there is none, otherwise
+    leave what is built alone.  The product itself never calls this: ``_lib.load()`` raises when
+    the library is missing."""
+    if not LIB_PATH.exists():
+        build(verbose=verbose)
+    return LIB_PATH
+
+
 def _drain(procs, verbose):
     while procs:
         src, p = procs.pop(0)
