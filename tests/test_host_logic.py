@@ -715,3 +715,17 @@ int main(void) {
     assert lines[2] == "bytes 0"
     assert lines[3].startswith("rc -") and "bad layer/head count" in lines[3]
     assert lines[4].startswith("rc -") and "kv layout is NULL" in lines[4]
+
+
+def test_product_raises_when_the_library_is_missing(tmp_path, monkeypatch):
+    """No CPU, PyTorch or oracle fallback: with no shared library the loader raises and names the
+    build command (the tests, the smoke run and the benchmark build it beforehand; the product
+    never does, and never takes another path)."""
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libtriattention_hip.so")
+    with pytest.raises(RuntimeError, match="is missing"):
+        _lib.load()
+    import triattention_amd
+    pkg = Path(triattention_amd.__file__).parent
+    offenders = [str(p) for p in pkg.rglob("*.py") if re.search(r"^\s*(from|import)\s+oracle\b", p.read_text(), re.M)]
+    assert offenders == [], "the package must not import the oracle"
