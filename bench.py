@@ -528,7 +528,9 @@ def main() -> int:
                    "q_heads": w.num_q_heads, "head_dim": w.head_dim, "block_size": w.block_size,
                    "kv_dtype": w.kv_dtype, "pool_blocks_per_layer": w.pool_blocks,
                    "pool_occupancy": round(sum(w.blocks_per_seq) / w.pool_blocks, 4),
-                   "pool_gib": round(w.pool_blocks * pool_bytes_per_block(w) / 2**30, 1)},
+                   "pool_gib": round(w.pool_blocks * pool_bytes_per_block(w) / 2**30, 1),
+                   "pool_note": ("block tables are a random permutation of a shared pool of pool_blocks_per_layer blocks; "
+                                 "exact_pool (when present) is the same step on a pool of exactly the live blocks")},
         "achieved_gbs": step_gbs,
         "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
         "algorithmic_bytes": algo,
