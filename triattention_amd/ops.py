@@ -243,24 +243,31 @@ class StepBatch:
         if not self._table_in_flat:
             raise ValueError("this batch was not built from host lists with block tables")
         pitch = int(self.block_table.shape[1])
-        rows = []
-        for r in block_tables:
-            if len(r) > pitch:
-                raise ValueError(f"a block table of {len(r)} entries does not fit the batch's pitch of {pitch}")
-            rows.extend(int(x) for x in r)
-            rows.extend([0] * (pitch - len(r)))
-        pf = [int(x) for x in prefill_lens] if prefill_lens is not None else [0] * n
-        parts = [self.seq_lens_host, [int(x) for x in round_start], pf if self.prefill_lens is not None else [],
-                 self.budgets_host or [], rows]
-        if [len(p) for p in parts] != self._sizes or len(block_tables) != n:
+        if len(block_tables) != n or len(round_start) != n or (prefill_lens is not None and len(prefill_lens) != n):
             raise ValueError("refill needs the shapes the batch was built with")
         staging = getattr(self, "_staging", None)
         if staging is None:
+            # Pinned mirror of the device array; the lengths and budgets in it never change.
             staging = self._staging = torch.empty(self._flat.numel(), dtype=torch.int32, pin_memory=True)
+            self._host = staging.numpy()
+            self._host[:n] = self.seq_lens_host
+            o = 2 * n + self._sizes[2]
+            self._host[o:o + self._sizes[3]] = self.budgets_host or []
             self._staged = torch.cuda.Event()
         else:
             self._staged.synchronize()          # the previous copy out of the staging buffer has finished
-        staging.copy_(torch.tensor([x for part in parts for x in part], dtype=torch.int32))
+        host = self._host
+        host[n:2 * n] = round_start
+        if self.prefill_lens is not None:
+            host[2 * n:3 * n] = prefill_lens if prefill_lens is not None else 0
+        o = 2 * n + self._sizes[2] + self._sizes[3]
+        for r in block_tables:
+            m = len(r)
+            if m > pitch:
+                raise ValueError(f"a block table of {m} entries does not fit the batch's pitch of {pitch}")
+            host[o:o + m] = r
+            host[o + m:o + pitch] = 0
+            o += pitch
         self._flat.copy_(staging, non_blocking=True)
         self._staged.record()
 

@@ -288,7 +288,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         ``layer_kv``: [(layer_idx, kv_cache)] of the group; ``requests``: one dict per request
         with ``block_ids, total_tokens, prefill_len, protect_prefill, round_start, budget_total``
         and ``total_tokens > budget_total > 0``.  Returns the selector result dictionaries in
-        request order; the caches then hold the kept rows in slots ``0..k-1``.  Raises
+        request order (``indices``: int32, valid until this selector's next step); the caches then hold
+        the kept rows in slots ``0..k-1``.  Raises
         ``ResidentLaunchFailed`` with the caches of this group untouched when a wait inside the
         resident kernel expired; the caller repeats the call with ``allow_resident=False``, which
         takes the kernels that do not wait for each other."""
@@ -365,7 +366,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         if resident and _resident_failed(ws.status()):
             raise ResidentLaunchFailed("a wait inside the resident kernel expired; the caches were left untouched")
         h = kv.num_kv_heads
-        keep = keep.to(torch.long)           # one conversion; the per-request results are views
+        # The per-request indices are int32 views of a buffer this selector writes again at its next
+        # step (the hook reads their shape only; a caller that keeps them copies them).
         return [{"mode": "per_head", "indices": keep[b * h:(b + 1) * h, :k],
                  "semantic": "hf_aligned_global_per_head", "group_agg_mode": agg,
                  "debug_group_layer_indices": list(layer_ids), "debug_recent_count": _recent_count(t)}
