@@ -538,6 +538,8 @@ def main() -> int:
                      "compact": mean(compact_ms)},
         "stage_gbs": {"score": score_gbs, "compact": compact_gbs},
         "key_vectors_per_s": total_keys * w.num_layers * w.num_kv_heads / (ms_per_step * 1e-3),
+        "compact_ms_p50": sorted(compact_ms)[len(compact_ms) // 2],
+        "compact_ms_p99": sorted(compact_ms)[min(len(compact_ms) - 1, int(0.99 * len(compact_ms)))],
         "step_ms_p50": sorted(step_ms)[len(step_ms) // 2],
         "step_ms_p99": sorted(step_ms)[min(len(step_ms) - 1, int(0.99 * len(step_ms)))],
         "timed_region_wall_s": wall_s,
