@@ -356,7 +356,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                     ws = ops.Workspace(kv, batch, sc)
                     keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
                     graph = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(graph):
+                    # (thread-local error mode: another thread of the engine may use the GPU meanwhile)
+                    with torch.cuda.graph(graph, capture_error_mode="thread_local"):
                         ops.compress_step(kv, batch, sc, sel, ws, keep)
                     entry.update(graph=graph, batch=batch, ws=ws, keep=keep, resident=resident, kv=kv, sc=sc)
                     graph.replay()
