@@ -52,12 +52,17 @@ def parse_args():
     ap.add_argument("--seq-len", type=int, default=0,
                     help="override every sequence's cached length (e.g. budget + 128 for the steady-state step)")
     ap.add_argument("--sequences", type=int, default=0, help="override the number of sequences (with --seq-len)")
-    ap.add_argument("--no-exact-pool", "--no-scattered-pool", dest="no_exact_pool", action="store_true",
-                    help="skip the second leg: the same step on a pool that holds exactly the live blocks")
+    ap.add_argument("--no-scattered-pool", "--no-exact-pool", dest="no_scattered_pool", action="store_true",
+                    help="skip the second leg: the same step with the live blocks scattered over a pool four times "
+                         "their number (at most 160 GiB)")
     ap.add_argument("--pool-occupancy", type=float, default=0.0,
                     help="live blocks / blocks of the shared pool.  Default: the workload's own where it names one "
-                         "(config 3: 0.8), otherwise a pool four times the live blocks (at most 160 GiB): a serving "
-                         "engine's cache spans most of the HBM and a batch's blocks lie scattered over it")
+                         "(config 3: 0.8), otherwise 1 (a pool of exactly the live blocks)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the brief legs over the other benchmark configurations (default invocation only)")
+    ap.add_argument("--other-steps", type=int, default=10, help="timed steps of each of the other configurations")
+    ap.add_argument("--graph-steps", type=int, default=20,
+                    help="replays of the step captured into a HIP graph (resident path; 0: skip)")
     ap.add_argument("--kv-dtype", choices=["bf16", "fp16"], default="",
                     help="key/value dtype of the synthetic cache (default: the workload's own)")
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers")
@@ -125,17 +130,19 @@ def cpu_baseline(w, layers: int, seq0=None):
     return out, (keep, fin) if seq0 is not None else None
 
 
-def keep_differences(got: torch.Tensor, want: torch.Tensor, fin: torch.Tensor, ks, heads: int, tie: float = 1e-5):
+def keep_differences(got: torch.Tensor, want: torch.Tensor, fin: torch.Tensor, ks, heads: int, tie: float = 1e-5,
+                     lens=None):
     """Kept indices of ``got`` that ``want`` does not hold (rows = sequences x heads, CPU tensors), and
     how many of them are near-ties: selection score within ``tie`` x the largest finite score of the
-    row's sequence of the row's threshold (the k-th largest of ``fin``)."""
+    row's sequence of the row's threshold (the k-th largest of ``fin``).  ``lens``: the sequences' own
+    lengths (rows of a ragged batch hold nothing meaningful beyond them)."""
     diff = near = 0
     for r in range(got.shape[0]):
         k = ks[r // heads]
         a, b = set(got[r, :k].tolist()), set(want[r, :k].tolist())
         if a == b:
             continue
-        row = fin[r]
+        row = fin[r] if lens is None else fin[r, :lens[r // heads]]
         finite = row[torch.isfinite(row)]
         scale = float(finite.abs().max()) if finite.numel() else 1.0
         thr = float(torch.sort(row, descending=True).values[k - 1])
@@ -310,66 +317,199 @@ class StepRun:
                 self.v_scales[i][self.slot] = self.saved_scales[i][1]
 
     def step(self, events=None):
+        """The step as a serving engine issues it: ONE call of the C ABI's ``tri_compress_step`` (score +
+        select + compact, one launch sequence); ``events``: a pair recorded around the call."""
+        if self.two_pass:
+            return self.staged_step(events if events is None else [events[0], None, None, events[1]])
+        if events is not None:
+            events[0].record()
+        self.ops.compress_step(self.kv, self.batch, self.sc, self.sel, self.ws, self.keep)
+        if events is not None:
+            events[1].record()
+
+    def staged_step(self, events=None):
+        """The same kernels issued stage by stage (three calls of the C ABI), with an event at every stage
+        boundary: where the step's time goes.  The event records and the separate calls cost some 20 us a
+        step, which is why the step itself is timed by ``step``."""
         ops = self.ops
+        record = lambda i: events is not None and events[i] is not None and events[i].record()
         if events is not None:
             events[0].record()
         if self.two_pass:
             raw, _ = ops.score_paged(self.kv, self.batch, self.sc, self.ws, out=self.raw_buf)
-            if events is not None:
-                events[1].record()
+            record(1)
             ops.select(self.kv, self.batch, self.sc, self.sel, raw, self.ws, keep=self.keep)
         else:
             ops.select_paged(self.kv, self.batch, self.sc, self.sel, self.ws, scores_out=self.fin_buf, want_keep=False)
-            if events is not None:
-                events[1].record()
+            record(1)
             ops.topk_batch(self.fin_buf, self.batch, self.w.num_kv_heads, self.keep)
-        if events is not None:
-            events[2].record()
+        record(2)
         ops.compact(self.kv, self.batch, self.keep)
-        if events is not None:
-            events[3].record()
+        record(3)
 
-    def timed(self, warmup: int, steps: int):
+    def timed(self, warmup: int, steps: int, staged: bool = False):
         """``warmup`` untimed steps, then ``steps`` timed ones.  Everything is enqueued asynchronously
         on one stream: restore(i-1), then the events and kernels of step i.  The host runs ahead while
         the restore copies execute, so the event pairs bracket GPU time only and restores stay outside
-        every timed interval.  Returns (events per step, wall seconds of the timed region)."""
+        every timed interval.  Returns (events per step, wall seconds of the timed region): two events
+        per step, or four with ``staged`` (stage boundaries)."""
+        fn = self.staged_step if staged else self.step
         for _ in range(warmup):
-            self.step()
+            fn()
             self.restore()
         torch.cuda.synchronize()
-        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4 if staged else 2)] for _ in range(steps)]
         wall0 = time.perf_counter()
         for i in range(steps):
-            self.step(evs[i])
+            fn(evs[i])
             if i + 1 < steps:
                 self.restore()
         torch.cuda.synchronize()
         return evs, time.perf_counter() - wall0
 
+    def graph_timed(self, warmup: int, steps: int):
+        """The same one-call step captured once into a HIP graph and replayed (how the runtime's selector
+        issues a step whose shape it has seen before).  Returns the mean milliseconds per replay."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.step()
+        torch.cuda.current_stream().wait_stream(side)
+        self.restore()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, capture_error_mode="thread_local"):
+            self.step()
+        self.restore()
+        for _ in range(warmup):
+            graph.replay()
+            self.restore()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in evs:
+            a.record()
+            graph.replay()
+            b.record()
+            self.restore()
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs) / steps
+
     def status_raised(self) -> bool:
         return not self.two_pass and self.ws.status() != 0
 
 
-def second_pool_leg(w2, args, dev, sc, sel, force_two_pass: bool):
-    """The same workload on a pool of another size (same sequences, same kernels, same algorithmic
-    bytes, other physical addresses)."""
-    run = StepRun(w2, dev, sc, sel, force_two_pass)
-    evs, _ = run.timed(args.warmup, args.steps)
-    if run.status_raised():
-        return {"error": "status word raised"}
+def percentile(xs, q: float):
+    xs = sorted(xs)
+    return xs[min(len(xs) - 1, int(q * len(xs)))]
+
+
+def measure(run: "StepRun", warmup: int, steps: int) -> dict:
+    """Times ``steps`` one-call steps (two events each) and then ``steps`` staged ones (an event at every
+    stage boundary) on a resident workload.  ``ms_per_step`` and everything derived from it come from
+    the one-call steps; ``stage_ms`` from the staged ones."""
+    w = run.w
     mean = lambda xs: sum(xs) / len(xs)
-    ms = mean([e[0].elapsed_time(e[3]) for e in evs])
-    algo = w2.algorithmic_bytes()
+    evs, wall_s = run.timed(warmup, steps)
+    step_ms = [e[0].elapsed_time(e[1]) for e in evs]
+    if run.status_raised():
+        return {"error": "status word raised during the timed steps"}
+    run.restore()
+    sev, _ = run.timed(1, steps, staged=True)
+    if run.status_raised():
+        return {"error": "status word raised during the staged steps"}
+    run.restore()
+    score_ms = [e[0].elapsed_time(e[1]) for e in sev]
+    select_ms = [e[1].elapsed_time(e[2]) for e in sev]
+    compact_ms = [e[2].elapsed_time(e[3]) for e in sev]
+    ms = mean(step_ms)
+    algo = w.algorithmic_bytes()
     gbs = algo["total"] / (ms * 1e-3) / 1e9
-    return {"pool_blocks_per_layer": w2.pool_blocks,
-            "pool_occupancy": round(sum(w2.blocks_per_seq) / w2.pool_blocks, 4),
-            "pool_gib": round(w2.pool_blocks * pool_bytes_per_block(w2) / 2**30, 1), "steps": args.steps,
-            "ms_per_step": ms,
-            "stage_ms": {"score": mean([e[0].elapsed_time(e[1]) for e in evs]),
-                         "select" if run.two_pass else "topk": mean([e[1].elapsed_time(e[2]) for e in evs]),
-                         "compact": mean([e[2].elapsed_time(e[3]) for e in evs])},
-            "value": sum(w2.seq_lens) / (ms * 1e-3), "achieved_gbs": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+    return {
+        "steps": steps, "ms_per_step": ms, "value": sum(w.seq_lens) / (ms * 1e-3), "achieved_gbs": gbs,
+        "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "path": run.path,
+        "stage_ms": {"score": mean(score_ms), "select" if run.two_pass else "topk": mean(select_ms),
+                     "compact": mean(compact_ms)},
+        "staged_ms_per_step": mean([e[0].elapsed_time(e[3]) for e in sev]),
+        "stage_gbs": {"score": algo["score"] / (mean(score_ms) * 1e-3) / 1e9,
+                      "compact": algo["compact"] / (mean(compact_ms) * 1e-3) / 1e9},
+        "step_ms_p50": percentile(step_ms, 0.5), "step_ms_p99": percentile(step_ms, 0.99),
+        "compact_ms_p50": percentile(compact_ms, 0.5), "compact_ms_p99": percentile(compact_ms, 0.99),
+        "timed_region_wall_s": wall_s,
+    }
+
+
+def pool_description(w) -> dict:
+    return {"pool_blocks_per_layer": w.pool_blocks, "pool_occupancy": round(sum(w.blocks_per_seq) / w.pool_blocks, 4),
+            "pool_gib": round(w.pool_blocks * pool_bytes_per_block(w) / 2**30, 1)}
+
+
+def score_config(w, dev, aggregation: str = "mean"):
+    from triattention_amd import ops, synth
+    qc, qa = synth.make_stats(w, dev)
+    fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2, device=dev)
+    sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev),
+                         aggregation)
+    return sc, qc, qa
+
+
+def gpu_parity(run: "StepRun", keep_timed: torch.Tensor) -> dict:
+    """On the pristine cache: the timed path's keep rows again (must reproduce what the timed steps left)
+    and against the two-pass kernels' rows, with the near-tie count."""
+    ops, w = run.ops, run.w
+    heads = w.num_kv_heads
+    ks = [min(w.budget, t) for t in w.seq_lens]
+    two = ops.SelectConfig(window_size=w.window_size, allow_resident=False)
+    ops.select_paged(run.kv, run.batch, run.sc, two if run.two_pass else run.sel, run.ws, scores_out=run.fin_buf,
+                     want_keep=False)
+    keep_again = ops.topk_batch(run.fin_buf, run.batch, heads)
+    keep_tp, fin_tp, _ = ops.select_paged(run.kv, run.batch, run.sc, two, run.ws, want_scores=True)
+    torch.cuda.synchronize()
+    same = all(torch.equal(keep_again[b * heads:(b + 1) * heads, :k], keep_timed[b * heads:(b + 1) * heads, :k])
+               for b, k in enumerate(ks))
+    diff, near = keep_differences(keep_again.cpu(), keep_tp.cpu(), fin_tp.cpu(), ks, heads, lens=list(w.seq_lens))
+    return {"timed_path": run.path, "kept_indices_compared": sum(ks) * heads, "timed_keep_reproduced": same,
+            "vs_two_pass_diff": diff, "vs_two_pass_near_tie_swaps": near, "near_tie_bound": "1e-5 of the largest score",
+            "_rows0": keep_again[:heads, :ks[0]].cpu()}
+
+
+def oracle_seq0(run: "StepRun", qc, qa, rows0: torch.Tensor) -> dict:
+    """Sequence 0 of a resident workload through the CPU oracle (its own blocks copied to the host), and
+    the GPU's keep rows of that sequence against the oracle's."""
+    w = run.w
+    blocks0 = torch.tensor(run.tables[0], device=run.caches[0].device, dtype=torch.long)
+    seq0 = {"caches": [c[:, blocks0].cpu() for c in run.caches], "qc": qc.cpu(), "qa": qa.cpu()}
+    base, (okeep, ofin) = cpu_baseline(w, w.num_layers, seq0)
+    diff, near = keep_differences(rows0, okeep, ofin, [int(okeep.shape[1])], w.num_kv_heads)
+    return base, {"vs_oracle_seq0_diff": diff, "vs_oracle_seq0_near_tie_swaps": near,
+                  "vs_oracle_seq0_compared": int(okeep.numel())}
+
+
+def other_config(name: str, w, dev, steps: int, oracle: bool) -> dict:
+    """One of the other benchmark configurations, briefly: the same measurement as the headline leg, the
+    status word checked, the timed path's rows against the two-pass kernels' and (small ones) sequence 0
+    against the CPU oracle."""
+    t0 = time.perf_counter()
+    from triattention_amd import ops
+    sc, qc, qa = score_config(w, dev)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    run = StepRun(w, dev, sc, sel, False)
+    out = {"workload": w.name, "layers": w.num_layers, "sequences": w.num_seqs, "tokens_per_sequence": max(w.seq_lens),
+           "budget": w.budget, "kv_dtype": w.kv_dtype, **pool_description(w)}
+    out.update(measure(run, 2, steps))
+    if "error" not in out:
+        keep_timed = run.keep.clone()
+        run.restore()
+        par = gpu_parity(run, keep_timed)
+        rows0 = par.pop("_rows0")
+        if oracle and w.kv_dtype != "fp8":
+            _, vs = oracle_seq0(run, qc, qa, rows0)
+            par.update(vs)
+        out["parity_check"] = par
+    out["algorithmic_bytes"] = w.algorithmic_bytes()
+    out["wall_s"] = round(time.perf_counter() - t0, 2)
+    del run
+    torch.cuda.empty_cache()
+    return out
 
 
 def main() -> int:
@@ -389,6 +529,8 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = synth.config(args.config)
+    plain = args.config == 1 and not (args.seq_len or args.layers or args.q_heads or args.kv_heads or args.head_dim
+                                      or args.kv_dtype or args.two_pass or args.aggregation != "mean")
     if args.seq_len > 0:
         nseq = args.sequences if args.sequences > 0 else w.num_seqs
         w = w.scaled(name=f"{w.name}_b{nseq}_len{args.seq_len}", seq_lens=(args.seq_len,) * nseq)
@@ -401,10 +543,12 @@ def main() -> int:
         if "fp8" in (args.kv_dtype, w.kv_dtype):
             raise SystemExit("--kv-dtype switches between bf16 and fp16; the fp8 workload is --config 4")
         w = w.scaled(name=f"{w.name}_{args.kv_dtype}", kv_dtype=args.kv_dtype)
-    # The shared pool.  A workload that names its own occupancy keeps it; otherwise the live blocks are
-    # scattered over a pool four times their number, and a second leg (below) runs the same step on a
-    # pool that holds exactly the live blocks.
-    w_exact = None
+    # The shared pool.  A workload that names its own occupancy keeps it.  Otherwise the first leg, whose
+    # figures are the line's top-level ones, runs on a pool of exactly the live blocks (every block of
+    # the pool belongs to a sequence of the batch), and a second leg runs the same step with the live
+    # blocks scattered over a pool four times their number (a serving engine's cache spans most of
+    # the HBM and a batch's blocks lie scattered over it).
+    w_scattered = None
     if args.pool_occupancy > 0:
         if not 0.0 < args.pool_occupancy <= 1.0:
             raise SystemExit("--pool-occupancy is a fraction in (0, 1]")
@@ -413,40 +557,33 @@ def main() -> int:
         live = sum(w.blocks_per_seq)
         blocks = default_pool_blocks(w)
         if blocks > live:
-            w_exact = w
-            w = w.scaled(pool_occupancy=live / blocks)
+            w_scattered = w.scaled(pool_occupancy=live / blocks)
     t_setup = time.perf_counter()
-    qc, qa = synth.make_stats(w, dev)
-    fs = torch.ones(w.num_layers, w.num_q_heads, w.head_dim // 2, device=dev)
-    sc = ops.ScoreConfig(ops.fold_stats(qc, qa, fs), synth.rope_inv_freq(w, dev), synth.geometric_offsets(device=dev),
-                         args.aggregation)
+    sc, qc, qa = score_config(w, dev, args.aggregation)
     sel = ops.SelectConfig(window_size=w.window_size)
     run = StepRun(w, dev, sc, sel, args.two_pass)
     setup_s = time.perf_counter() - t_setup
-    tables, caches, kv, batch, ws, keep, fin_buf = run.tables, run.caches, run.kv, run.batch, run.ws, run.keep, run.fin_buf
-    path, two_pass, restore, step = run.path, run.two_pass, run.restore, run.step
+    path, two_pass = run.path, run.two_pass
 
-    evs, wall_s = run.timed(args.warmup, args.steps)
-
-    ms = lambda a, b: a.elapsed_time(b)
-    step_ms = [ms(e[0], e[3]) for e in evs]
-    score_ms = [ms(e[0], e[1]) for e in evs]
-    select_ms = [ms(e[1], e[2]) for e in evs]
-    compact_ms = [ms(e[2], e[3]) for e in evs]
-    mean = lambda xs: sum(xs) / len(xs)
-    ms_per_step = mean(step_ms)
+    m = measure(run, args.warmup, args.steps)
+    if "error" in m:
+        print("bench.py: the resident kernel raised its status word; the step did not do its work and the "
+              "timing is void", file=sys.stderr)
+        return 3
+    ms_per_step = m["ms_per_step"]
     total_keys = sum(w.seq_lens)
     algo = w.algorithmic_bytes()
-    keys_per_s = total_keys / (ms_per_step * 1e-3)
-    step_gbs = algo["total"] / (ms_per_step * 1e-3) / 1e9
-    score_gbs = algo["score"] / (mean(score_ms) * 1e-3) / 1e9
-    compact_gbs = algo["compact"] / (mean(compact_ms) * 1e-3) / 1e9
+    run.step()
+    torch.cuda.synchronize()
+    keep_timed = run.keep.clone()
+    run.restore()
 
-    if not two_pass and ws.status() != 0:
-        print("bench.py: the resident kernel raised its status word during the timed steps; the step did not "
-              "do its work and the timing is void", file=sys.stderr)
-        return 3
-    keep_timed = keep.clone()
+    graph_ms = None
+    if not two_pass and args.graph_steps > 0:
+        graph_ms = run.graph_timed(2, args.graph_steps)
+        if run.status_raised():
+            print("bench.py: status word raised during the graph replays", file=sys.stderr)
+            return 3
 
     # Sustained figure: the same step back to back (with the restore copies between, which keep the
     # memory system just as busy) for a few seconds, so the GPU sits at the clocks it holds under
@@ -456,20 +593,16 @@ def main() -> int:
         n = args.sustained_steps
         tail = max(1, min(100, n // 4))
         sev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(tail)]
-        restore()
+        run.restore()
         torch.cuda.synchronize()
         s0 = time.perf_counter()
         for i in range(n):
             j = i - (n - tail)
-            if j >= 0:
-                sev[j][0].record()
-            step()
-            if j >= 0:
-                sev[j][1].record()
-            restore()
+            run.step(sev[j] if j >= 0 else None)
+            run.restore()
         torch.cuda.synchronize()
         s_wall = time.perf_counter() - s0
-        if not two_pass and ws.status() != 0:
+        if run.status_raised():
             print("bench.py: status word raised during the sustained steps", file=sys.stderr)
             return 3
         tail_ms = sorted(a.elapsed_time(b) for a, b in sev)
@@ -480,28 +613,18 @@ def main() -> int:
                      "frac_of_hbm_peak": algo["total"] / (s_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
     # Parity of what was timed, outside every timed region: on the pristine cache the timed path's
-    # keep rows against the two-pass kernels' (and further down against the CPU oracle on sequence 0).
+    # keep rows against the two-pass kernels' and against the CPU oracle on sequence 0.
     parity = None
-    seq0 = None
+    cpu = None
     if not args.no_parity_check and args.aggregation == "mean":
-        restore()
-        heads = w.num_kv_heads
-        ks = [min(w.budget, t) for t in w.seq_lens]
-        two = ops.SelectConfig(window_size=w.window_size, allow_resident=False)
-        ops.select_paged(kv, batch, sc, two if two_pass else sel, ws, scores_out=fin_buf, want_keep=False)
-        keep_again = ops.topk_batch(fin_buf, batch, heads)
-        keep_tp, fin_tp, _ = ops.select_paged(kv, batch, sc, two, ws, want_scores=True)
-        torch.cuda.synchronize()
-        same_as_timed = all(torch.equal(keep_again[b * heads:(b + 1) * heads, :k], keep_timed[b * heads:(b + 1) * heads, :k])
-                            for b, k in enumerate(ks))
-        diff, near = keep_differences(keep_again.cpu(), keep_tp.cpu(), fin_tp.cpu(), ks, heads)
-        parity = {"timed_path": path, "kept_indices_compared": sum(ks) * heads, "timed_keep_reproduced": same_as_timed,
-                  "vs_two_pass_diff": diff, "vs_two_pass_near_tie_swaps": near, "near_tie_bound": "1e-5 of the largest score"}
-        gpu_rows0 = keep_again[:heads, :ks[0]].cpu()
-        del keep_tp, fin_tp
+        run.restore()
+        parity = gpu_parity(run, keep_timed)
+        rows0 = parity.pop("_rows0")
         if not args.no_cpu_baseline and w.kv_dtype != "fp8" and args.cpu_layers >= w.num_layers:
-            blocks0 = torch.tensor(tables[0], device=dev, dtype=torch.long)
-            seq0 = {"caches": [c[:, blocks0].cpu() for c in caches], "qc": qc.cpu(), "qa": qa.cpu(), "gpu_rows": gpu_rows0}
+            cpu, vs = oracle_seq0(run, qc, qa, rows0)
+            parity.update(vs)
+    if cpu is None and not args.no_cpu_baseline:
+        cpu, _ = cpu_baseline(w, args.cpu_layers)
 
     if args.aggregation == "mean":
         two_pass_kernel = "score_mean_kernel"
@@ -510,9 +633,10 @@ def main() -> int:
     else:
         two_pass_kernel = "score_max_kernel"
     traffic = MEASURED_TRAFFIC_BYTES.get((w.name, path)) if args.aggregation == "mean" else None
+    score_gbs = m["stage_gbs"]["score"]
     out = {
         "metric": "keys scored+compacted/sec & achieved HBM GB/s (% peak), Qwen3-8B 16k ctx",
-        "value": keys_per_s,
+        "value": m["value"],
         "unit": "keys/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -522,27 +646,27 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
+        "dtype_note": f"arithmetic in fp32 (accumulation, statistics, selection scores); keys and values stored as {w.kv_dtype}",
         "data": "synthetic",
         "config": {"workload": w.name, "layers": w.num_layers, "sequences": w.num_seqs,
                    "tokens_per_sequence": max(w.seq_lens), "budget": w.budget, "kv_heads": w.num_kv_heads,
                    "q_heads": w.num_q_heads, "head_dim": w.head_dim, "block_size": w.block_size,
-                   "kv_dtype": w.kv_dtype, "pool_blocks_per_layer": w.pool_blocks,
-                   "pool_occupancy": round(sum(w.blocks_per_seq) / w.pool_blocks, 4),
-                   "pool_gib": round(w.pool_blocks * pool_bytes_per_block(w) / 2**30, 1),
+                   "kv_dtype": w.kv_dtype, **pool_description(w),
                    "pool_note": ("block tables are a random permutation of a shared pool of pool_blocks_per_layer blocks; "
-                                 "exact_pool (when present) is the same step on a pool of exactly the live blocks")},
-        "achieved_gbs": step_gbs,
-        "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
+                                 "scattered_pool (when present) is the same step with the live blocks scattered over a "
+                                 "pool four times their number"),
+                   "step": "one call of tri_compress_step (score + select + compact), HIP events around the call"},
+        "achieved_gbs": m["achieved_gbs"],
+        "frac_of_hbm_peak": m["frac_of_hbm_peak"],
         "algorithmic_bytes": algo,
-        "stage_ms": {"score": mean(score_ms), "select" if two_pass else "topk": mean(select_ms),
-                     "compact": mean(compact_ms)},
-        "stage_gbs": {"score": score_gbs, "compact": compact_gbs},
+        "stage_ms": m["stage_ms"],
+        "staged_ms_per_step": m["staged_ms_per_step"],
+        "stage_note": "stage_ms: a second pass of the same steps issued stage by stage with an event at every boundary",
+        "stage_gbs": m["stage_gbs"],
         "key_vectors_per_s": total_keys * w.num_layers * w.num_kv_heads / (ms_per_step * 1e-3),
-        "compact_ms_p50": sorted(compact_ms)[len(compact_ms) // 2],
-        "compact_ms_p99": sorted(compact_ms)[min(len(compact_ms) - 1, int(0.99 * len(compact_ms)))],
-        "step_ms_p50": sorted(step_ms)[len(step_ms) // 2],
-        "step_ms_p99": sorted(step_ms)[min(len(step_ms) - 1, int(0.99 * len(step_ms)))],
-        "timed_region_wall_s": wall_s,
+        "compact_ms_p50": m["compact_ms_p50"], "compact_ms_p99": m["compact_ms_p99"],
+        "step_ms_p50": m["step_ms_p50"], "step_ms_p99": m["step_ms_p99"],
+        "timed_region_wall_s": m["timed_region_wall_s"],
         "setup_s": setup_s,
         "path": path,
         "roofline": {"kernel": {"two_pass": two_pass_kernel, "resident_valu": "fused_select_kernel",
@@ -552,6 +676,10 @@ def main() -> int:
                      "traffic_source": (traffic[1] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by "
                                         "the same counters on a 1 GiB copy; not measured by this run)") if traffic else None},
     }
+    if graph_ms is not None:
+        out["graph_replay"] = {"steps": args.graph_steps, "ms_per_step": graph_ms,
+                               "frac_of_hbm_peak": algo["total"] / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                               "what": "the same one-call step captured once into a HIP graph and replayed"}
     if sustained is not None:
         out["sustained"] = sustained
     if parity is not None:
@@ -568,7 +696,7 @@ def main() -> int:
     c1.record()
     torch.cuda.synchronize()
     out["device_copy_gbs"] = 5 * 2 * (1 << 30) / (c0.elapsed_time(c1) * 1e-3) / 1e9
-    out["frac_of_device_copy"] = step_gbs / out["device_copy_gbs"]
+    out["frac_of_device_copy"] = m["achieved_gbs"] / out["device_copy_gbs"]
     del src, dst
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -583,19 +711,31 @@ def main() -> int:
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
         out["hook_batch_call"] = hook_latency(w, dev, calls=20, requests=len(w.seq_lens))
-    del run, tables, caches, kv, batch, ws, keep, fin_buf, restore, step
+    del run
     torch.cuda.empty_cache()
-    if w_exact is not None and not args.no_exact_pool:
-        out["exact_pool"] = second_pool_leg(w_exact, args, dev, sc, sel, args.two_pass)
+    if w_scattered is not None and not args.no_scattered_pool:
+        run2 = StepRun(w_scattered, dev, sc, sel, args.two_pass)
+        leg = {**pool_description(w_scattered), **measure(run2, args.warmup, args.steps)}
+        del run2
         torch.cuda.empty_cache()
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"], oracle_keep = cpu_baseline(w, args.cpu_layers, seq0)
-        if oracle_keep is not None:
-            okeep, ofin = oracle_keep
-            heads = w.num_kv_heads
-            diff, near = keep_differences(seq0["gpu_rows"], okeep, ofin, [int(okeep.shape[1])], heads)
-            out["parity_check"].update({"vs_oracle_seq0_diff": diff, "vs_oracle_seq0_near_tie_swaps": near,
-                                        "vs_oracle_seq0_compared": int(okeep.numel())})
+        out["scattered_pool"] = leg
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    # The other benchmark configurations, briefly (the default invocation only).
+    if plain and not args.no_other_configs:
+        others = {}
+        steady = synth.config(1)
+        steady = steady.scaled(name=f"{steady.name}_len{steady.budget + 128}",
+                               seq_lens=(steady.budget + 128,) * steady.num_seqs)
+        for name, wo, oracle in (("c0", synth.config(0), True), ("steady_2176", steady, True),
+                                 ("c4", synth.config(4), False), ("c2", synth.config(2), False),
+                                 ("c3", synth.config(3), False)):
+            try:
+                others[name] = other_config(name, wo, dev, args.other_steps, oracle)
+            except Exception as exc:      # a leg that fails must not take the headline with it
+                others[name] = {"error": f"{type(exc).__name__}: {exc}"}
+                torch.cuda.empty_cache()
+        out["other_configs"] = others
     print(json.dumps(out))
     return 0
 
