@@ -524,7 +524,7 @@ def main() -> int:
 
     from triattention_amd import build as tri_build
     tri_build.ensure_built()          # loads what is built; builds only when there is no library at all
-    from triattention_amd import ops, synth
+    from triattention_amd import _lib, ops, synth
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -628,7 +628,7 @@ def main() -> int:
 
     if args.aggregation == "mean":
         two_pass_kernel = "score_mean_kernel"
-    elif w.kv_dtype == "bf16" and w.head_dim == 128 and os.environ.get("TRIATTN_MAX_KERNEL") != "valu":
+    elif w.kv_dtype == "bf16" and w.head_dim == 128 and _lib.get_tuning(_lib.TUNE_MAX_KERNEL) != 1:
         two_pass_kernel = "score_max_mfma_kernel"
     else:
         two_pass_kernel = "score_max_kernel"

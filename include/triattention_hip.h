@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 4
+#define TRI_ABI_VERSION 5
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -119,6 +119,48 @@ typedef struct tri_select_params {
 
 int tri_abi_version(void);
 const char* tri_last_error(void);
+/* SHA-256 (hex) of the sources and compiler flags this library was built from ("unknown" for a
+ * build outside the package's build script); the build script compares it with the sources next to
+ * the library and rebuilds a library that does not belong to them.  No counterpart in the reference. */
+const char* tri_source_digest(void);
+
+/* Process-wide settings of the library (no counterpart in the reference, whose Triton kernels have
+ * none of these choices).  The library itself reads no environment variable for them; the Python
+ * layer applies TRIATTN_RESIDENT_KERNEL / _WORKGROUPS / _LAYER_SPLIT / _SPIN_TICKS and
+ * TRIATTN_MAX_KERNEL once, when it loads the library.  tri_set_tuning returns TRI_OK or
+ * TRI_ERR_INVALID_ARGUMENT; tri_get_tuning returns the value in force (INT64_MIN for an unknown key).
+ * Settings are read when a call plans its launches; changing one while another thread is inside a
+ * call affects that call or the next. */
+typedef enum tri_tuning {
+  TRI_TUNE_RESIDENT_KERNEL = 0,     /* 0 (default): the library chooses by shape and batch; 1: the matrix-core
+                                       resident kernel whenever the shape has one, however small the launch;
+                                       2: the vector-unit resident kernel; 3: never a resident kernel */
+  TRI_TUNE_RESIDENT_WORKGROUPS = 1, /* 0 (default): the device's own capacity; n > 0: plan as if the device held
+                                       n resident workgroups (never more than it does): small inputs then need
+                                       several launches (tests) */
+  TRI_TUNE_LAYER_SPLIT = 2,         /* -1 (default): small batches are cut by layers unless the kernel was forced
+                                       with TRI_TUNE_RESIDENT_KERNEL = 1; 0: never; 1: always allowed */
+  TRI_TUNE_MAX_KERNEL = 3,          /* 0 (default): max aggregation on the matrix cores where a kernel exists;
+                                       1: always the vector-unit kernel (comparison runs) */
+  TRI_TUNE_RESIDENT_WAIT_US = 4     /* how long a resident workgroup waits for the other workgroups of its launch
+                                       before it raises status word 1, in microseconds: default 2,000,000; a serving
+                                       engine that shares the GPU may lower it (a starved launch costs this much
+                                       once, after which the selector stays on the other kernels); negative: every
+                                       wait gives up at once (exercises the failure path from the host) */
+} tri_tuning;
+int tri_set_tuning(int32_t key, int64_t value);
+int64_t tri_get_tuning(int32_t key);
+
+/* Resident launches of one process are chained on the device with an event (two of them running at
+ * the same time would each hold part of the CUs and wait for the other's workgroups).  The library
+ * does that itself for every launch it issues outside graph capture.  A launch sequence captured
+ * into a HIP graph contains no such wait or record (event nodes of a replay would refer to the
+ * capture-time record), so a caller that replays a captured tri_compress_step / tri_select_paged
+ * whose path is a resident kernel brackets the replay with these two calls on the stream it
+ * replays on: enter makes `stream` wait (on the device) for the previous resident launch of the
+ * process, leave records the replay as the latest one.  No counterpart in the reference. */
+int tri_resident_gate_enter(void* stream);
+int tri_resident_gate_leave(void* stream);
 
 /* Replaces the per-call stat preparation of core/scoring.py:259-271,346-351:
  * folded[l][a][0][f] = s*q_r, [1] = s*q_i, [2] = s*(q_abs - sqrt(q_r^2+q_i^2+1e-8))
@@ -237,7 +279,10 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
  * previous call's contents (nothing in it needs to start at zero except the status word, which
  * the call clears): calls that overlap in time on one GPU, from any streams or threads, race.
  * Results are those of tri_compress_step with no_resident = 1.  status_out (may be NULL)
- * receives the device address of the status word for callers that want to read it. */
+ * receives the device address of the status word for callers that want to read it.
+ * The first call on a device also looks up the array's address (hipGetSymbolAddress) and asks the
+ * occupancy calculator once; a caller that records the call into a graph makes one call on that
+ * device outside capture first. */
 #define TRI_STATIC_WORKSPACE_BYTES (64u << 20)
 int tri_compress_step_static(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                              const tri_select_params* sel, int32_t* keep, const uint32_t** status_out,

@@ -118,3 +118,35 @@ def assert_keep_matches(keep: torch.Tensor, want: torch.Tensor, fin: torch.Tenso
             assert abs(float(fin[h, idx]) - float(thr)) <= tie_tol, (h, idx, float(fin[h, idx]), float(thr))
             swapped += 1
     return swapped
+
+
+_TUNE_ENV = {"TRIATTN_RESIDENT_KERNEL": "resident_kernel", "TRIATTN_RESIDENT_WORKGROUPS": "resident_workgroups",
+             "TRIATTN_RESIDENT_LAYER_SPLIT": "layer_split", "TRIATTN_MAX_KERNEL": "max_kernel"}
+
+
+def tune(**settings):
+    """Process-wide settings of the library for the rest of the test (``tri_set_tuning``; an autouse
+    fixture puts the defaults back after every test): ``resident_kernel`` ("auto" / "mfma" / "valu" /
+    "off"), ``resident_workgroups``, ``layer_split``, ``max_kernel`` ("auto" / "valu", "mfma" = auto),
+    ``resident_wait_us`` (None: the default of two seconds).  Keys may also be given by the names of the
+    environment variables the Python layer reads at load time."""
+    from triattention_amd import _lib
+    for name, value in settings.items():
+        name = _TUNE_ENV.get(name, name)
+        key = _lib.tuning._KEYS[name]
+        if name == "resident_kernel":
+            value = _lib.RESIDENT_KERNEL_CHOICES[value] if isinstance(value, str) else int(value)
+        elif name == "max_kernel":
+            value = {"auto": 0, "mfma": 0, "valu": 1}[value] if isinstance(value, str) else int(value)
+        elif name == "resident_wait_us" and value is None:
+            value = TUNING_DEFAULTS[key]
+        _lib.set_tuning(key, int(value))
+
+
+TUNING_DEFAULTS = {0: 0, 1: 0, 2: -1, 3: 0, 4: 2_000_000}
+
+
+def reset_tuning():
+    from triattention_amd import _lib
+    for key, value in TUNING_DEFAULTS.items():
+        _lib.set_tuning(key, value)

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from conftest import load_golden
-from helpers import (KEEP_TIE_TOL, SELECT_SCORE_TOL, assert_keep_matches, build_inputs, device_objects, oracle_raw,
+from helpers import (KEEP_TIE_TOL, tune, SELECT_SCORE_TOL, assert_keep_matches, build_inputs, device_objects, oracle_raw,
                      record_swaps, score_tolerance, selection_score_tol)
 from oracle import compaction as ocp
 from oracle import scoring as osc
@@ -115,7 +115,7 @@ def test_max_aggregation_on_matrix_cores_matches_the_vector_unit_kernel(name, mo
     print(f"case={name} workload={w}", flush=True)
     out = {}
     for kernel in ("mfma", "valu"):
-        monkeypatch.setenv("TRIATTN_MAX_KERNEL", kernel)
+        tune(max_kernel=kernel)
         caches, kv, batch, sc = device_objects(w, inp, DEV, aggregation="max")
         raw, ws = ops.score_paged(kv, batch, sc)
         sel = ops.SelectConfig(window_size=w.window_size)
@@ -275,7 +275,7 @@ def test_group_selection_matches_reference_golden(tag, kw, path, fixture, monkey
     """Keep sets written by the reference's own selector (paged group branch), through the
     two-pass path and through both resident kernels."""
     if path != "two_pass":
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", path.split("_")[1])
+        tune(resident_kernel=path.split("_")[1])
     gold = load_golden(fixture)
     layers, hkv, t, d = gold["keys"].shape
     hq = gold["q_mean_complex"].shape[1]
@@ -348,8 +348,8 @@ def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(
         caches.append(kvc.to(DEV))
     tables = [(ids + c * pool).tolist() for c in range(copies)]
     if path != "two_pass":
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", path.split("_")[1])
-        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", str(workgroups))
+        tune(resident_kernel=path.split("_")[1])
+        tune(resident_workgroups=workgroups)
     kv = ops.PagedKV.from_kv_caches(caches)
     budget = int(gold["budget"])
     batch = ops.StepBatch(DEV, [t] * copies, round_start=[int(gold["round_start"])] * copies, budgets=budget,
@@ -719,8 +719,7 @@ def test_steady_state_step_matches_oracle(case, monkeypatch):
                                         "TRIATTN_RESIDENT_WORKGROUPS": "40"}),
         "sixteen_requests": (4, 16, {}),
     }[case]
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    tune(**env)
     w = synth.Workload("steady", layers, 32, 8, 128, (2176,) * seqs, 2048, index=70 + layers)
     inp = build_inputs(w)
     caches, kv, batch, sc = device_objects(w, inp, DEV)
@@ -772,9 +771,9 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
         pytest.skip("the vector-unit kernel holds four query heads per KV head")
     if kernel == "valu" and w.head_dim != 128:      # (64 and 256 exist on the matrix cores only)
         pytest.skip("the vector-unit kernel is built for a head dimension of 128")
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)      # take that kernel however small the launch
+    tune(resident_kernel=kernel)      # take that kernel however small the launch
     if "workgroups" in case:
-        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", str(case["workgroups"]))
+        tune(resident_workgroups=case["workgroups"])
     inp = build_inputs(w, case.get("kv_axis", 0))
     print(f"case={name} kernel={kernel} workload={w}", flush=True)
     caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=case.get("prefill_lens"))
@@ -852,10 +851,10 @@ def test_matrix_core_scores_carry_every_piece(kv_dtype, head_dim, monkeypatch):
     inp = build_inputs(w)
     caches, kv, batch, sc = device_objects(w, inp, DEV)
     sel = ops.SelectConfig(window_size=w.window_size, normalize=False, layer_reduce="max")
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    tune(resident_kernel="mfma")
     assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
     _, fin_r, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    tune(resident_kernel="off")
     _, fin_t, _ = ops.select_paged(kv, batch, sc, sel, want_scores=True)
     torch.cuda.synchronize()
     assert ws.status() == 0
@@ -884,12 +883,12 @@ def test_resident_selection_on_dense_keys(kernel, monkeypatch):
     batch = ops.StepBatch(DEV, lens, round_start=[900, 400, 512], budgets=128)
     sel = ops.SelectConfig(window_size=16)
     print(f"dense keys kernel={kernel}", flush=True)
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+    tune(resident_kernel=kernel)
     assert ops.select_path(kv, batch, sc, sel) == "resident_" + kernel
     keep_r, fin_r, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
     torch.cuda.synchronize()
     assert ws.status() == 0
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    tune(resident_kernel="off")
     assert ops.select_path(kv, batch, sc, sel) == "two_pass"
     keep_t, fin_t, _ = ops.select_paged(kv, batch, sc, sel, want_scores=True)
     torch.cuda.synchronize()
@@ -985,15 +984,57 @@ def test_resident_launch_next_to_another_streams_kernels():
             assert torch.equal(c.view(torch.int16), x.view(torch.int16))
 
 
+def test_replayed_resident_graph_is_chained_with_eager_resident_launches():
+    """A captured step holds no wait on the process's previous resident launch and no record of its
+    own (streams under capture are left alone).  Whoever replays such a graph brackets the replay with
+    ops.resident_gate(); replays on one stream then interleave with eager resident launches on another
+    without either starving the other: clean status words, the results of running alone."""
+    sel = ops.SelectConfig(window_size=12)
+    w1, inp1, caches1, kv1, batch1, sc1 = _resident_batch(21)
+    w2, inp2, caches2, kv2, batch2, sc2 = _resident_batch(22)
+    for kv, batch, sc in ((kv1, batch1, sc1), (kv2, batch2, sc2)):
+        assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    keep_a, fin_a, ws_a = ops.select_paged(kv1, batch1, sc1, sel, want_scores=True)
+    keep_b, fin_b, ws_b = ops.select_paged(kv2, batch2, sc2, sel, want_scores=True)
+    assert ws_a.status() == 0 and ws_b.status() == 0
+    want_a, want_b = (keep_a.clone(), fin_a.clone()), (keep_b.clone(), fin_b.clone())
+    s_graph, s_eager = torch.cuda.Stream(), torch.cuda.Stream()
+    s_graph.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s_graph):
+        ops.select_paged(kv1, batch1, sc1, sel, ws_a, keep=keep_a, scores_out=fin_a)     # warm-up on the capture stream
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s_graph):
+        ops.select_paged(kv1, batch1, sc1, sel, ws_a, keep=keep_a, scores_out=fin_a)
+    print("replays next to eager resident launches", flush=True)
+    for rep in range(4):
+        keep_a.zero_(); fin_a.zero_(); keep_b.zero_(); fin_b.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s_eager):
+            ops.select_paged(kv2, batch2, sc2, sel, ws_b, keep=keep_b, scores_out=fin_b)
+        with torch.cuda.stream(s_graph):
+            with ops.resident_gate():
+                graph.replay()
+        with torch.cuda.stream(s_eager):
+            ops.select_paged(kv2, batch2, sc2, sel, ws_b, keep=keep_b, scores_out=fin_b)
+        with torch.cuda.stream(s_graph):
+            with ops.resident_gate():
+                graph.replay()
+        torch.cuda.synchronize()
+        assert ws_a.status() == 0 and ws_b.status() == 0, rep
+        assert torch.equal(keep_a, want_a[0]) and torch.equal(fin_a, want_a[1]), rep
+        assert torch.equal(keep_b, want_b[0]) and torch.equal(fin_b, want_b[1]), rep
+
+
 @pytest.mark.parametrize("case", ["fewer_launches_planned_than_needed", "device_length_beyond_max_seq_len"])
 def test_host_lengths_that_disagree_with_the_device_raise_the_status_word(case, monkeypatch):
     """A caller of the C ABI whose host copy of the lengths is stale: the planner sizes launches
     and rows from the host values, the kernels read the device values.  Sequences that would not
     be scored (or lie beyond the planned rows) raise the status word (3), every workgroup still
     runs to its end inside the planned bounds, and the step's compaction leaves the cache alone."""
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    tune(resident_kernel="mfma")
     if case == "fewer_launches_planned_than_needed":
-        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", "16")
+        tune(resident_workgroups=16)
         w = small(seq_lens=(3000,) * 8, num_q_heads=32, num_kv_heads=8, budget=128, index=51)
     else:
         w = small(seq_lens=(1000, 700), num_q_heads=32, num_kv_heads=8, budget=128, index=52)
@@ -1071,16 +1112,16 @@ def test_expired_wait_raises_the_status_word_and_the_step_leaves_the_cache_alone
     without the limit then gives the result of the chained calls."""
     w, inp, caches, kv, batch, sc = _resident_batch(21)
     sel = ops.SelectConfig(window_size=w.window_size)
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+    tune(resident_kernel=kernel)
     assert ops.select_path(kv, batch, sc, sel) == "resident_" + kernel
     before = [c.clone() for c in caches]
-    monkeypatch.setenv("TRIATTN_RESIDENT_SPIN_TICKS", "-1")
+    tune(resident_wait_us=-1)
     print(f"forced expiry, kernel={kernel}", flush=True)
     _, ws = ops.compress_step(kv, batch, sc, sel)
     assert ws.status() != 0
     for c, c0 in zip(caches, before):
         assert torch.equal(c.view(torch.int16), c0.view(torch.int16))
-    monkeypatch.delenv("TRIATTN_RESIDENT_SPIN_TICKS")
+    tune(resident_wait_us=None)
     keep, ws = ops.compress_step(kv, batch, sc, sel, ws=ws)
     assert ws.status() == 0
     caches2, kv2, batch2, sc2 = device_objects(w, inp, DEV)
@@ -1102,12 +1143,12 @@ def test_fp16_coefficients_beyond_half_range_raise_the_status_word(monkeypatch):
     inp["qa"] = inp["qa"] * 1e6
     caches, kv, batch, sc = device_objects(w, inp, DEV)
     sel = ops.SelectConfig(window_size=w.window_size)
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    tune(resident_kernel="mfma")
     assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
     print("fp16 coefficient overflow", flush=True)
     _, _, ws = ops.select_paged(kv, batch, sc, sel)
     assert ws.status() != 0
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+    tune(resident_kernel="valu")
     _, _, ws = ops.select_paged(kv, batch, sc, sel)
     assert ws.status() == 0
 
@@ -1129,7 +1170,7 @@ def test_magnitudes_beyond_half_range_raise_the_status_word(monkeypatch, what):
         inp["qa"] = inp["qa"] * 1e6
     caches, kv, batch, sc = device_objects(w, inp, DEV)
     sel = ops.SelectConfig(window_size=w.window_size)
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")
+    tune(resident_kernel="mfma")
     assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
     print(f"magnitude overflow: {what}", flush=True)
     before = [c.clone() for c in caches]
@@ -1138,7 +1179,7 @@ def test_magnitudes_beyond_half_range_raise_the_status_word(monkeypatch, what):
     for c, c0 in zip(caches, before):
         assert torch.equal(c.view(torch.int16), c0.view(torch.int16))
     for kernel in ("valu", "off"):
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+        tune(resident_kernel=kernel)
         keep, fin, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
         assert ws.status() == 0 and bool(torch.isfinite(fin[0, :50]).all())
     keep = keep.cpu().long()
@@ -1153,7 +1194,7 @@ def test_magnitudes_beyond_half_range_raise_the_status_word(monkeypatch, what):
 
 
 def test_resident_path_falls_back_when_shape_has_no_kernel(monkeypatch):
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "mfma")        # even when asked for explicitly
+    tune(resident_kernel="mfma")        # even when asked for explicitly
     for kw, selkw in ((dict(num_q_heads=32, num_kv_heads=2), {}), (dict(head_dim=256, kv_dtype="fp8"), {}), (dict(head_dim=64, kv_dtype="fp8"), {}),
                       (dict(block_size=24), {}), ({}, dict(shared=True)), ({}, dict(layer_reduce=None))):
         w = small(**kw)
@@ -1295,7 +1336,7 @@ def test_fp8_cache_without_row_scales(monkeypatch):
     assert kv_b.struct.v_scale_layers is None or not kv_b.struct.v_scale_layers
     sel = ops.SelectConfig(window_size=w.window_size)
     for kernel in ("off", "mfma"):
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", kernel)
+        tune(resident_kernel=kernel)
         print(f"unscaled fp8, resident kernel setting {kernel}", flush=True)
         keep_a, fin_a, _ = ops.select_paged(kv_a, batch, sc, sel, want_scores=True)
         keep_b, fin_b, _ = ops.select_paged(kv_b, batch, sc, sel, want_scores=True)

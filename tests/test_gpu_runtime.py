@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from conftest import load_golden
-from helpers import assert_keep_matches, score_tolerance
+from helpers import assert_keep_matches, score_tolerance, tune
 from oracle import compaction as ocp
 from oracle import scoring as osc
 from oracle import selection as osel
@@ -258,7 +258,7 @@ def test_batch_hook_equals_the_hook_called_request_by_request(tmp_path, monkeypa
     One request is under budget and one asks for the prefill guard."""
     from helpers import build_inputs
     from triattention_amd import synth
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    tune(resident_kernel="off")
     w = synth.Workload(name="t", num_layers=3, num_q_heads=8, num_kv_heads=2, head_dim=128,
                        seq_lens=(300, 1000, 97, 513, 60), budget=96, block_size=16, window_size=12, rope_theta=1e6,
                        index=31)
@@ -324,10 +324,10 @@ def test_batch_hook_on_the_resident_kernel(tmp_path, monkeypatch):
 
     # forced failure of the resident launch: the hook repeats the step request by request
     runner_f, reqs_f, caches_f, sched_f, signals_f = _fake_runner(w, inp, tmp_path)
-    monkeypatch.setenv("TRIATTN_RESIDENT_SPIN_TICKS", "-1")
+    tune(resident_wait_us=-1)
     failed = RunnerHookCompressionExecutor(runner_f).execute_batch(signals_f, sched_f)
-    monkeypatch.delenv("TRIATTN_RESIDENT_SPIN_TICKS")
-    monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+    tune(resident_wait_us=None)
+    tune(resident_kernel="off")
     runner_s, reqs_s, caches_s, sched_s, signals_s = _fake_runner(w, inp, tmp_path)
     single = {rid: RunnerHookCompressionExecutor(runner_s).execute(rid, sig, sched_s) for rid, sig in signals_s.items()}
     torch.cuda.synchronize()
@@ -347,7 +347,7 @@ def test_repeated_shape_replays_a_graph_with_the_same_results(tmp_path, monkeypa
     from triattention_amd import synth
     from triattention_amd.runtime import selector as selector_mod
     if not resident:
-        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "off")
+        tune(resident_kernel="off")
     w = synth.Workload(name="t", num_layers=3, num_q_heads=8, num_kv_heads=2, head_dim=128,
                        seq_lens=(1184,) * (16 if resident else 1), budget=160, block_size=16, window_size=12,
                        rope_theta=1e6, index=41)

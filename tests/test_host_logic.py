@@ -11,6 +11,7 @@ import torch
 
 from conftest import GOLDEN, ROOT, load_golden
 from triattention_amd import _lib, rope
+from triattention_amd import build as tri_build
 from triattention_amd.core import stats as stats_mod
 from triattention_amd.core.compressor import CompressionState, gather_kv_by_indices, normalize_scores, \
     protect_window_tokens
@@ -33,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.tri_abi_version() == 4
+    assert lib.tri_abi_version() == _lib.ABI_VERSION == 5
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
@@ -729,3 +730,73 @@ def test_product_raises_when_the_library_is_missing(tmp_path, monkeypatch):
     pkg = Path(triattention_amd.__file__).parent
     offenders = [str(p) for p in pkg.rglob("*.py") if re.search(r"^\s*(from|import)\s+oracle\b", p.read_text(), re.M)]
     assert offenders == [], "the package must not import the oracle"
+
+
+def test_tuning_settings_round_trip_and_reject_bad_values():
+    """The process-wide settings replace environment variables inside the library: values come back
+    as set, out-of-range values and unknown keys are refused with a message, and the defaults are the
+    documented ones (tri_set_tuning / tri_get_tuning)."""
+    lib = _lib.load()
+    defaults = {_lib.TUNE_RESIDENT_KERNEL: 0, _lib.TUNE_RESIDENT_WORKGROUPS: 0, _lib.TUNE_LAYER_SPLIT: -1,
+                _lib.TUNE_MAX_KERNEL: 0, _lib.TUNE_RESIDENT_WAIT_US: 2_000_000}
+    for key, value in defaults.items():
+        assert _lib.get_tuning(key) == value
+    with _lib.tuning(resident_kernel="off", resident_workgroups=12, layer_split=1, max_kernel="valu", resident_wait_us=-1):
+        assert [_lib.get_tuning(k) for k in range(5)] == [3, 12, 1, 1, -1]
+    assert [_lib.get_tuning(k) for k in range(5)] == [defaults[k] for k in range(5)]
+    for key, bad in ((_lib.TUNE_RESIDENT_KERNEL, 4), (_lib.TUNE_RESIDENT_KERNEL, -1), (_lib.TUNE_LAYER_SPLIT, 2),
+                     (_lib.TUNE_MAX_KERNEL, 2), (_lib.TUNE_RESIDENT_WORKGROUPS, -3), (_lib.TUNE_RESIDENT_WAIT_US, 10**13),
+                     (17, 0)):
+        assert lib.tri_set_tuning(key, bad) == _lib.TRI_ERR_INVALID_ARGUMENT
+        assert lib.tri_last_error()
+    assert lib.tri_get_tuning(17) == -2**63
+    assert [_lib.get_tuning(k) for k in range(5)] == [defaults[k] for k in range(5)]
+
+
+def test_environment_is_applied_once_at_load(monkeypatch):
+    """The documented TRIATTN_* switches are read by the Python layer when it loads the library, not
+    by the library on every call."""
+    lib = _lib.load()
+    try:
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "valu")
+        monkeypatch.setenv("TRIATTN_RESIDENT_WORKGROUPS", "24")
+        monkeypatch.setenv("TRIATTN_RESIDENT_LAYER_SPLIT", "0")
+        monkeypatch.setenv("TRIATTN_RESIDENT_SPIN_TICKS", "-1")
+        monkeypatch.setenv("TRIATTN_MAX_KERNEL", "valu")
+        assert _lib.get_tuning(_lib.TUNE_RESIDENT_KERNEL) == 0        # nothing happens by itself
+        _lib._apply_environment(lib)
+        assert [_lib.get_tuning(k) for k in range(5)] == [2, 24, 0, 1, -1]
+        monkeypatch.setenv("TRIATTN_RESIDENT_KERNEL", "sideways")
+        with pytest.raises(ValueError, match="TRIATTN_RESIDENT_KERNEL"):
+            _lib._apply_environment(lib)
+    finally:
+        for key, value in {0: 0, 1: 0, 2: -1, 3: 0, 4: 2_000_000}.items():
+            _lib.set_tuning(key, value)
+
+
+def test_a_library_built_from_other_sources_is_rebuilt(tmp_path, monkeypatch):
+    """ensure_built compares the digest compiled into the library with the sources next to it: the
+    library of this checkout belongs to its sources; after one source file changes it does not, and
+    ensure_built builds (the build itself is replaced by a recorder here) and says why."""
+    import shutil
+    assert tri_build.stale() is None
+    assert tri_build.built_digest() == tri_build.source_digest() == _lib.load().tri_source_digest().decode()
+    csrc = tmp_path / "csrc"
+    shutil.copytree(tri_build.CSRC, csrc)
+    monkeypatch.setattr(tri_build, "CSRC", csrc)
+    assert tri_build.stale() is None                      # same content elsewhere: still the same library
+    calls = []
+    monkeypatch.setattr(tri_build, "build", lambda verbose=False, jobs=None: calls.append("build"))
+    tri_build.ensure_built()
+    assert calls == []
+    src = csrc / "tri_compact.hip"
+    src.write_text(src.read_text() + "\n// edited\n")
+    why = tri_build.stale()
+    assert why is not None and "built from other sources" in why
+    tri_build.ensure_built()
+    assert calls == ["build"]
+    # a file that is missing altogether
+    monkeypatch.setattr(tri_build, "LIB_PATH", tmp_path / "libtriattention_hip.so")
+    assert "is missing" in tri_build.stale()
+    tri_build.ensure_built()
+    assert calls == ["build", "build"]

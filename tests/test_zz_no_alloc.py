@@ -86,3 +86,61 @@ def test_static_scratch_rejects_steps_beyond_its_array():
     rc = lib.tri_compress_step_static(C.byref(kv.struct), C.byref(huge.struct), C.byref(sp), C.byref(ss),
                                       keep.data_ptr(), None, None)
     assert rc == _lib.TRI_ERR_WORKSPACE and b"static array" in lib.tri_last_error()
+
+
+def _free_device_bytes() -> int:
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return int(free.value)
+
+
+def test_static_scratch_step_allocates_nothing_and_runs_under_graph_capture():
+    """What the entry point is for.  After one warm-up call on the device (the first call looks up the
+    array's address and asks the occupancy calculator once), a call leaves the device's free memory
+    and torch's allocator exactly as they were, and the same call recorded into a HIP graph (where
+    an allocation would abort the capture) replays with the eager call's results."""
+    w = synth.Workload("static_graph", 3, 16, 4, 128, (1100, 640), 192, index=36)
+    inp = build_inputs(w)
+    sel = ops.SelectConfig(window_size=w.window_size)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    pristine = [c.clone() for c in caches]
+    keep = torch.empty(w.num_seqs * w.num_kv_heads, batch.max_budget, dtype=torch.int32, device=DEV)
+    status_at = ops.compress_step_static(kv, batch, sc, sel, keep)            # warm-up, and the eager result
+    assert _read_device_word(status_at) == 0
+    want_keep, want_caches = keep.clone(), [c.clone() for c in caches]
+
+    def restore():
+        for c, p in zip(caches, pristine):
+            c.copy_(p)
+
+    restore()
+    torch.cuda.synchronize()
+    before = (_free_device_bytes(), torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    ops.compress_step_static(kv, batch, sc, sel, keep)
+    torch.cuda.synchronize()
+    after = (_free_device_bytes(), torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert before == after
+    assert torch.equal(keep, want_keep)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        restore()
+        ops.compress_step_static(kv, batch, sc, sel, keep)                    # once on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    restore()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.compress_step_static(kv, batch, sc, sel, keep)
+    for rep in range(3):
+        restore()
+        keep.fill_(-3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _read_device_word(status_at) == 0
+        assert torch.equal(keep, want_keep), rep
+        for c, x in zip(caches, want_caches):
+            assert torch.equal(c.view(torch.int16), x.view(torch.int16)), rep

@@ -13,7 +13,7 @@ import os
 # TRIATTN_HIP_LIBRARY points at another build of the same ABI (e.g. an instrumented one).
 LIB_PATH = Path(os.environ.get("TRIATTN_HIP_LIBRARY") or Path(__file__).resolve().parent / "libtriattention_hip.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 STATIC_WORKSPACE_BYTES = 64 << 20
 TRI_OK = 0
 TRI_ERR_INVALID_ARGUMENT = -1
@@ -25,8 +25,13 @@ KV_BF16, KV_FP16, KV_FP8_E4M3 = 0, 1, 2
 ROPE_HALF, ROPE_INTERLEAVED = 0, 1
 REDUCE_MEAN, REDUCE_MAX, REDUCE_NONE = 0, 1, -1
 
+# tri_tuning keys
+TUNE_RESIDENT_KERNEL, TUNE_RESIDENT_WORKGROUPS, TUNE_LAYER_SPLIT, TUNE_MAX_KERNEL, TUNE_RESIDENT_WAIT_US = range(5)
+RESIDENT_KERNEL_CHOICES = {"auto": 0, "mfma": 1, "valu": 2, "off": 3}
+
 EXPORTS = (
-    "tri_abi_version", "tri_last_error", "tri_fold_stats", "tri_workspace_bytes", "tri_workspace_status_offset",
+    "tri_abi_version", "tri_last_error", "tri_source_digest", "tri_set_tuning", "tri_get_tuning", "tri_resident_gate_enter",
+    "tri_resident_gate_leave", "tri_fold_stats", "tri_workspace_bytes", "tri_workspace_status_offset",
     "tri_score_paged",
     "tri_select", "tri_select_paged", "tri_select_path", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
     "tri_compact_paged_full", "tri_compress_step", "tri_compress_step_static", "tri_qstats_workspace_bytes", "tri_qstats",
@@ -89,6 +94,12 @@ def load() -> C.CDLL:
     P, I32, I64, U64 = C.c_void_p, C.c_int32, C.c_int64, C.c_uint64
     lib.tri_abi_version.restype = C.c_int
     lib.tri_last_error.restype = C.c_char_p
+    lib.tri_source_digest.restype = C.c_char_p
+    lib.tri_set_tuning.argtypes = [I32, I64]
+    lib.tri_get_tuning.argtypes = [I32]
+    lib.tri_get_tuning.restype = I64
+    lib.tri_resident_gate_enter.argtypes = [P]
+    lib.tri_resident_gate_leave.argtypes = [P]
     lib.tri_fold_stats.argtypes = [P, P, P, P, I32, I32, I32, I32, I32, P, P]
     lib.tri_workspace_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams)]
     lib.tri_workspace_bytes.restype = U64
@@ -121,7 +132,73 @@ def load() -> C.CDLL:
     if lib.tri_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH}: ABI version {lib.tri_abi_version()} != {ABI_VERSION}; rebuild the library")
     _lib = lib
+    _apply_environment(lib)
     return lib
+
+
+def _apply_environment(lib) -> None:
+    """The library reads no environment variable; the ones documented for comparison runs are
+    applied here, once, when the library is loaded (later changes of the environment have no
+    effect: use ``set_tuning``)."""
+    env = os.environ
+    v = env.get("TRIATTN_RESIDENT_KERNEL", "").strip().lower()
+    if v:
+        if v not in RESIDENT_KERNEL_CHOICES:
+            raise ValueError(f"TRIATTN_RESIDENT_KERNEL={v!r}: one of {sorted(RESIDENT_KERNEL_CHOICES)}")
+        lib.tri_set_tuning(TUNE_RESIDENT_KERNEL, RESIDENT_KERNEL_CHOICES[v])
+    for name, key in (("TRIATTN_RESIDENT_WORKGROUPS", TUNE_RESIDENT_WORKGROUPS),
+                      ("TRIATTN_RESIDENT_LAYER_SPLIT", TUNE_LAYER_SPLIT)):
+        v = env.get(name, "").strip()
+        if v:
+            lib.tri_set_tuning(key, int(v))
+    v = env.get("TRIATTN_RESIDENT_SPIN_TICKS", "").strip()      # ticks of the 100 MHz wall clock
+    if v:
+        lib.tri_set_tuning(TUNE_RESIDENT_WAIT_US, -1 if int(v) < 0 else max(1, int(v) // 100))
+    if env.get("TRIATTN_MAX_KERNEL", "").strip().lower() == "valu":
+        lib.tri_set_tuning(TUNE_MAX_KERNEL, 1)
+
+
+def set_tuning(key: int, value: int) -> int:
+    """Set one process-wide setting of the library (``tri_set_tuning``); returns the previous value."""
+    lib = load()
+    old = int(lib.tri_get_tuning(key))
+    check(lib.tri_set_tuning(key, int(value)))
+    return old
+
+
+def get_tuning(key: int) -> int:
+    return int(load().tri_get_tuning(key))
+
+
+class tuning:
+    """Context manager: settings of the library for the duration of a block (tests, comparison runs).
+
+        with tuning(resident_kernel="mfma", resident_workgroups=16): ...
+    """
+
+    _KEYS = {"resident_kernel": TUNE_RESIDENT_KERNEL, "resident_workgroups": TUNE_RESIDENT_WORKGROUPS,
+             "layer_split": TUNE_LAYER_SPLIT, "max_kernel": TUNE_MAX_KERNEL, "resident_wait_us": TUNE_RESIDENT_WAIT_US}
+
+    def __init__(self, **settings):
+        self.settings, self.saved = {}, {}
+        for name, value in settings.items():
+            if name not in self._KEYS:
+                raise KeyError(name)
+            if name == "resident_kernel" and isinstance(value, str):
+                value = RESIDENT_KERNEL_CHOICES[value]
+            if name == "max_kernel" and isinstance(value, str):
+                value = {"auto": 0, "valu": 1}[value]
+            self.settings[self._KEYS[name]] = int(value)
+
+    def __enter__(self):
+        for key, value in self.settings.items():
+            self.saved[key] = set_tuning(key, value)
+        return self
+
+    def __exit__(self, *exc):
+        for key, value in self.saved.items():
+            set_tuning(key, value)
+        return False
 
 
 def check(code: int) -> None:

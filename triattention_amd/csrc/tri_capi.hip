@@ -4,6 +4,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
+#include <climits>
 #include <mutex>
 
 #include "tri_common.h"
@@ -95,14 +97,14 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
 }
 
 tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
-  // Resident kernels: bf16 and fp8 keys go to the matrix-core kernel, fp16 to the vector-unit
-  // one, and only launches that fill most of the chip take them.  TRIATTN_RESIDENT_KERNEL
-  // overrides the choice: "mfma" / "valu" take that kernel whenever the shape has it (however
-  // small the launch), "off" never takes a resident kernel.
-  const char* force = getenv("TRIATTN_RESIDENT_KERNEL");
-  const bool f_valu = force && strcmp(force, "valu") == 0;
-  const bool f_mfma = force && strcmp(force, "mfma") == 0;
-  const bool f_off = force && strcmp(force, "off") == 0;
+  // Resident kernels: two-byte and fp8 keys go to the matrix-core kernel where the shape has one,
+  // and only launches that fill most of the chip take them.  TRI_TUNE_RESIDENT_KERNEL overrides
+  // the choice: 1 / 2 take the matrix-core / vector-unit kernel whenever the shape has it (however
+  // small the launch), 3 never takes a resident kernel.
+  const int64_t force = tri::tuning(TRI_TUNE_RESIDENT_KERNEL);
+  const bool f_valu = force == 2;
+  const bool f_mfma = force == 1;
+  const bool f_off = force == 3;
   // The matrix-core kernel addresses the 16 rows of a step with 32-bit offsets from a scalar base.
   const bool want_mfma = (kv->kv_dtype == TRI_KV_BF16 || kv->kv_dtype == TRI_KV_FP16 || kv->kv_dtype == TRI_KV_FP8_E4M3) &&
                          !f_valu &&
@@ -111,10 +113,10 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   const bool paged = b->block_table != nullptr;
   const int resident = f_off ? 0 : tri::fused_resident_workgroups();
   tri::FusedPlan fused{};
-  // Small batches are cut by layers as well (TRIATTN_RESIDENT_LAYER_SPLIT=0 switches that off, =1
-  // switches it on where the kernel was forced, which otherwise keeps whole-model workgroups).
-  const char* split_env = getenv("TRIATTN_RESIDENT_LAYER_SPLIT");
-  const bool split = split_env ? strcmp(split_env, "0") != 0 : !f_mfma;
+  // Small batches are cut by layers as well (TRI_TUNE_LAYER_SPLIT = 0 switches that off, 1 switches
+  // it on where the kernel was forced, which otherwise keeps whole-model workgroups).
+  const int64_t split_set = tri::tuning(TRI_TUNE_LAYER_SPLIT);
+  const bool split = split_set >= 0 ? split_set != 0 : !f_mfma;
   if (want_mfma)
     fused = tri::plan_fused_mfma(b->num_seqs, kv->num_kv_heads, kv->head_dim, G, kv->block_size, paged,
                                  sp->aggregation, b->max_seq_len, resident, f_mfma, kv->kv_dtype, b->seq_lens_host,
@@ -143,6 +145,31 @@ ResidentGate& resident_gate() {
   static ResidentGate gate;
   return gate;
 }
+
+// Both with the gate's mutex held.  A stream under capture is left alone.
+bool gate_applies(hipStream_t s, int& dev) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < ResidentGate::kMaxDevices &&
+         hipStreamIsCapturing(s, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone;
+}
+int gate_enter(ResidentGate& gate, hipStream_t s) {
+  int dev = 0;
+  if (!gate_applies(s, dev) || !gate.event[dev]) return TRI_OK;
+  return launch_status(hipStreamWaitEvent(s, gate.event[dev], 0), "resident chain wait");
+}
+int gate_leave(ResidentGate& gate, hipStream_t s) {
+  int dev = 0;
+  if (!gate_applies(s, dev)) return TRI_OK;
+  if (!gate.event[dev]) {
+    const hipError_t e = hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming);
+    if (e != hipSuccess) return launch_status(e, "resident chain event");
+  }
+  return launch_status(hipEventRecord(gate.event[dev], s), "resident chain record");
+}
+
+// Process-wide settings (tri_set_tuning).
+constexpr int kTunings = 5;
+std::atomic<int64_t> g_tuning[kTunings] = {{0}, {0}, {-1}, {0}, {2000000}};
 
 // Device address of `scratch` on the current device, looked up once per device.
 struct StaticScratch {
@@ -290,27 +317,16 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
     // Two resident launches that run at the same time on one device would each hold part of
     // the CUs and wait for the other's workgroups until their waits expire.  Launches of this
     // process are therefore chained: each waits (on the device, not on the host) for the
-    // previous one on whatever stream that was.  Streams under graph capture are left alone.
+    // previous one on whatever stream that was.  Streams under graph capture are left alone
+    // (whoever replays the graph brackets the replay with tri_resident_gate_enter / _leave).
     ResidentGate& gate = resident_gate();
     std::lock_guard<std::mutex> lock(gate.mutex);
-    int dev = 0;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    const bool chain = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < ResidentGate::kMaxDevices &&
-                       hipStreamIsCapturing(s, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone;
-    if (chain && gate.event[dev]) {
-      e = hipStreamWaitEvent(s, gate.event[dev], 0);
-      if (e != hipSuccess) return launch_status(e, "resident chain wait");
-    }
+    int rc = gate_enter(gate, s);
+    if (rc) return rc;
     e = w.fused.eligible == 2 ? tri::launch_fused_mfma(a, s) : tri::launch_fused_select(a, s);
     if (e != hipSuccess) return launch_status(e, "fused_select");
-    if (chain) {
-      if (!gate.event[dev]) {
-        e = hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming);
-        if (e != hipSuccess) return launch_status(e, "resident chain event");
-      }
-      e = hipEventRecord(gate.event[dev], s);
-      if (e != hipSuccess) return launch_status(e, "resident chain record");
-    }
+    rc = gate_leave(gate, s);
+    if (rc) return rc;
   }
   if (!keep) return TRI_OK;   // selection scores only
   if (a.skip_layer_reduce)
@@ -347,11 +363,65 @@ int fill_compact(const tri_kv_layout* kv, const tri_batch* batch, const int32_t*
 
 }  // namespace
 
+namespace tri {
+int64_t tuning(int key) { return key >= 0 && key < kTunings ? g_tuning[key].load(std::memory_order_relaxed) : 0; }
+}  // namespace tri
+
 extern "C" {
 
 int tri_abi_version(void) { return TRI_ABI_VERSION; }
 
 const char* tri_last_error(void) { return g_err; }
+
+#ifndef TRI_SOURCE_DIGEST
+#define TRI_SOURCE_DIGEST "unknown"
+#endif
+const char* tri_source_digest(void) {
+  static const char digest[] = "TRI_SOURCE_DIGEST=" TRI_SOURCE_DIGEST;
+  return digest + sizeof("TRI_SOURCE_DIGEST=") - 1;
+}
+
+int tri_set_tuning(int32_t key, int64_t value) {
+  switch (key) {
+    case TRI_TUNE_RESIDENT_KERNEL:
+      if (value < 0 || value > 3) return fail(TRI_ERR_INVALID_ARGUMENT, "TRI_TUNE_RESIDENT_KERNEL takes 0..3, got %lld", (long long)value);
+      break;
+    case TRI_TUNE_RESIDENT_WORKGROUPS:
+      if (value < 0 || value > INT_MAX) return fail(TRI_ERR_INVALID_ARGUMENT, "TRI_TUNE_RESIDENT_WORKGROUPS %lld", (long long)value);
+      break;
+    case TRI_TUNE_LAYER_SPLIT:
+      if (value < -1 || value > 1) return fail(TRI_ERR_INVALID_ARGUMENT, "TRI_TUNE_LAYER_SPLIT takes -1, 0 or 1, got %lld", (long long)value);
+      break;
+    case TRI_TUNE_MAX_KERNEL:
+      if (value < 0 || value > 1) return fail(TRI_ERR_INVALID_ARGUMENT, "TRI_TUNE_MAX_KERNEL takes 0 or 1, got %lld", (long long)value);
+      break;
+    case TRI_TUNE_RESIDENT_WAIT_US:
+      // (the kernels count ticks of a 100 MHz clock in 64 bits)
+      if (value > (int64_t)3600 * 1000000) return fail(TRI_ERR_INVALID_ARGUMENT, "TRI_TUNE_RESIDENT_WAIT_US beyond one hour");
+      break;
+    default:
+      return fail(TRI_ERR_INVALID_ARGUMENT, "unknown tuning key %d", key);
+  }
+  g_tuning[key].store(value, std::memory_order_relaxed);
+  return TRI_OK;
+}
+
+int64_t tri_get_tuning(int32_t key) {
+  if (key < 0 || key >= kTunings) return INT64_MIN;
+  return g_tuning[key].load(std::memory_order_relaxed);
+}
+
+int tri_resident_gate_enter(void* stream) {
+  ResidentGate& gate = resident_gate();
+  std::lock_guard<std::mutex> lock(gate.mutex);
+  return gate_enter(gate, (hipStream_t)stream);
+}
+
+int tri_resident_gate_leave(void* stream) {
+  ResidentGate& gate = resident_gate();
+  std::lock_guard<std::mutex> lock(gate.mutex);
+  return gate_leave(gate, (hipStream_t)stream);
+}
 
 int tri_fold_stats(const float* q_mean_real, const float* q_mean_imag, const float* q_abs_mean,
                    const float* freq_scale_sq, int32_t num_layers, int32_t num_score_heads,

@@ -163,8 +163,10 @@ struct FusedLaunch {
   int skip_layer_reduce;         // 1: leave the groups' partial rows in fin_part (the top-k adds them while loading)
   FusedPlan plan;
 };
+// Process-wide settings (tri_set_tuning); defined in tri_capi.hip.
+int64_t tuning(int key);
 // Limit of the resident kernels' waits on other workgroups, in ticks of the 100 MHz wall
-// clock: 2 s, or TRIATTN_RESIDENT_SPIN_TICKS (tests: a negative value makes every wait give
+// clock, from TRI_TUNE_RESIDENT_WAIT_US (default 2 s; a negative value makes every wait give
 // up at once, which raises the status word while every workgroup still runs to its end).
 long long resident_spin_ticks();
 hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s);

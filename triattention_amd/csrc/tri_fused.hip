@@ -428,10 +428,8 @@ int fused_resident_workgroups() {
   }
   int n = cached[dev] > 0 ? cached[dev] : 0;
   // Tests: pretend the device is smaller, so that small inputs need several launches.
-  if (const char* v = std::getenv("TRIATTN_RESIDENT_WORKGROUPS")) {
-    const int want = std::atoi(v);
-    if (want > 0 && want < n) n = want;
-  }
+  const int64_t want = tuning(TRI_TUNE_RESIDENT_WORKGROUPS);
+  if (want > 0 && want < n) n = (int)want;
   return n;
 }
 
@@ -471,9 +469,8 @@ FusedPlan plan_fused(int B, int Hkv, int D, int G, int block_size, bool paged, i
 }
 
 long long resident_spin_ticks() {
-  const char* v = std::getenv("TRIATTN_RESIDENT_SPIN_TICKS");
-  if (v && *v) return std::atoll(v);
-  return 200000000LL;
+  const int64_t us = tuning(TRI_TUNE_RESIDENT_WAIT_US);
+  return us < 0 ? -1LL : (long long)us * 100LL;     // the wall clock ticks at 100 MHz
 }
 
 hipError_t launch_fused_select(const FusedLaunch& a, hipStream_t s) {

@@ -935,11 +935,8 @@ hipError_t launch_prepare(const float* folded, const float* omega, const float* 
   return hipGetLastError();
 }
 
-// TRIATTN_MAX_KERNEL=valu keeps max aggregation on the vector-unit kernel (comparison runs).
-static bool max_on_vector_unit() {
-  const char* v = std::getenv("TRIATTN_MAX_KERNEL");
-  return v && std::strcmp(v, "valu") == 0;
-}
+// TRI_TUNE_MAX_KERNEL = 1 keeps max aggregation on the vector-unit kernel (comparison runs).
+static bool max_on_vector_unit() { return tuning(TRI_TUNE_MAX_KERNEL) == 1; }
 
 hipError_t launch_score(const ScoreLaunch& a, hipStream_t s) {
   ScoreArgs k{};

@@ -588,6 +588,21 @@ def compress_step(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectCon
     return keep, ws
 
 
+class resident_gate:
+    """Brackets the replay of a captured launch sequence that contains a resident kernel: on entry the
+    current stream waits (on the device) for the process's previous resident launch, on exit the replay
+    is recorded as the latest one (``tri_resident_gate_enter`` / ``_leave``).  Launches the library issues
+    outside graph capture chain themselves; a graph holds no such wait or record."""
+
+    def __enter__(self):
+        _lib.check(_lib.load().tri_resident_gate_enter(_stream()))
+        return self
+
+    def __exit__(self, *exc):
+        _lib.check(_lib.load().tri_resident_gate_leave(_stream()))
+        return False
+
+
 def compress_step_static(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig, keep: torch.Tensor):
     """``compress_step`` on the library's own static scratch: the call allocates nothing (``keep``
     is the caller's, int32 [rows, max_budget]), always takes the score-then-select kernels, and

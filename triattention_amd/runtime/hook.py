@@ -603,6 +603,8 @@ def make_runner_compression_hook(base_runner: Any, config: TriAttentionRuntimeCo
                         reclaim[r.req_id].append(group)
         out = {}
         for r in batch:
+            # (what the one-by-one path leaves on the runner while it works on a request, hook_impl.py:60)
+            setattr(base_runner, "_triattention_active_req_id", r.req_id)
             if cache_len[r.req_id] is None:
                 out[r.req_id] = {"applied": False, "reason": "no_compactable_groups"}
                 continue

@@ -78,9 +78,15 @@ class _DeviceStats:
 # Steady-state steps (a shape seen before) replay their launch sequence from a HIP graph.
 GRAPH_REPLAY = True
 # ... for steps whose scratch stays below this many bytes: every captured shape keeps scratch and keep
-# rows of its own (up to eight shapes a selector), and the steps that repeat are the small ones
-# (budget + divide_length tokens a request).
+# rows of its own, and the steps that repeat are the small ones (budget + divide_length tokens a
+# request).  A selector keeps at most GRAPH_MAX_SHAPES captured shapes and at most
+# GRAPH_MAX_TOTAL_BYTES of their scratch, the least recently replayed one goes first; shapes seen once
+# are only remembered by their key (GRAPH_MAX_SEEN of them), so one-off batches never push a captured
+# shape out.
 GRAPH_MAX_SCRATCH_BYTES = 64 << 20
+GRAPH_MAX_SHAPES = 8
+GRAPH_MAX_TOTAL_BYTES = 256 << 20
+GRAPH_MAX_SEEN = 64
 GRAPH_COUNTS = {"captured": 0, "replayed": 0}     # process-wide, for tests and diagnostics
 
 
@@ -323,12 +329,21 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         # e.g. the first compression after a long prompt, never come back.)
         key = (id(kv), layer_ids, tuple(totals), tuple(ks), tuple(len(t) for t in tables), any(g > 0 for g in guards),
                agg, use_resident)
-        entry = holder.setdefault("graphs", {}).get(key) if GRAPH_REPLAY else None
+        graphs = holder.setdefault("graphs", {})       # captured shapes, least recently used first
+        seen = holder.setdefault("seen", {})           # keys of shapes that ran once, oldest first
+        entry = graphs.get(key) if GRAPH_REPLAY else None
         try:
-            if entry is not None and entry.get("graph") is not None:
+            if entry is not None:
+                graphs[key] = graphs.pop(key)          # most recently used
                 batch, ws, keep, resident = entry["batch"], entry["ws"], entry["keep"], entry["resident"]
                 batch.refill(rounds, tables, guards)
-                entry["graph"].replay()
+                if resident:
+                    # A graph holds neither the wait on the process's previous resident launch nor the
+                    # record of this one; the library's own gate is put around the replay.
+                    with ops.resident_gate():
+                        entry["graph"].replay()
+                else:
+                    entry["graph"].replay()
                 GRAPH_COUNTS["replayed"] += 1
             else:
                 batch = ops.StepBatch(kv.device, totals, round_start=rounds, budgets=ks, block_tables=tables,
@@ -337,7 +352,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                                        protect_prefill=any(g > 0 for g in guards), group_reduce="max", layer_reduce=agg,
                                        allow_resident=use_resident)
                 resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
-                if entry is None:
+                if not (GRAPH_REPLAY and key in seen):
                     # Scratch and keep rows of the previous step are reused when they fit; the results
                     # handed out below are fresh tensors.
                     keep_buf = holder.get("keep")
@@ -348,19 +363,27 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                                                  keep_buf[:rows * batch.max_budget].view(rows, batch.max_budget))
                     holder["ws"] = ws
                     if GRAPH_REPLAY and ws.bytes <= GRAPH_MAX_SCRATCH_BYTES:
-                        if len(holder["graphs"]) >= 8:
-                            holder["graphs"].pop(next(iter(holder["graphs"])))
-                        holder["graphs"][key] = {"graph": None}
+                        if len(seen) >= GRAPH_MAX_SEEN:
+                            seen.pop(next(iter(seen)))
+                        seen[key] = True
                 else:
                     # Second visit: buffers of the entry's own, capture (nothing runs), then replay.
+                    seen.pop(key, None)
                     ws = ops.Workspace(kv, batch, sc)
+                    while graphs and (len(graphs) >= GRAPH_MAX_SHAPES or
+                                      sum(e["ws"].bytes for e in graphs.values()) + ws.bytes > GRAPH_MAX_TOTAL_BYTES):
+                        graphs.pop(next(iter(graphs)))
                     keep = torch.empty(rows, batch.max_budget, dtype=torch.int32, device=kv.device)
                     graph = torch.cuda.CUDAGraph()
                     # (thread-local error mode: another thread of the engine may use the GPU meanwhile)
                     with torch.cuda.graph(graph, capture_error_mode="thread_local"):
                         ops.compress_step(kv, batch, sc, sel, ws, keep)
-                    entry.update(graph=graph, batch=batch, ws=ws, keep=keep, resident=resident, kv=kv, sc=sc)
-                    graph.replay()
+                    graphs[key] = dict(graph=graph, batch=batch, ws=ws, keep=keep, resident=resident, kv=kv, sc=sc)
+                    if resident:
+                        with ops.resident_gate():
+                            graph.replay()
+                    else:
+                        graph.replay()
                     GRAPH_COUNTS["captured"] += 1
         except Exception as exc:
             raise RuntimeError(f"{MARK}:score_failed:{type(exc).__name__}") from exc
