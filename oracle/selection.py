@@ -33,11 +33,15 @@ def score_chunk_tokens(block_size: int, total_tokens: int, score_chunk_max_token
     return upper
 
 
-def znorm_stats_streaming(raw: torch.Tensor, chunk_tokens: int, eps: float = 1e-8):
+def znorm_stats_streaming(raw: torch.Tensor, chunk_tokens: int, eps: float = 1e-8, exact: bool = False):
     """Per-row mean and safe std from chunked sums (selector_hf.py:884-913).
 
     mean = sum/N; var = (sumsq - N*mean^2)/(N-1) clamped at 0; std < eps -> 1.
+    ``exact``: the same formula with every sum and operation in double precision (what the
+    reference's fp32 arithmetic approximates; used to bound how far two correct fp32 evaluations
+    may disagree).
     """
+    ft = torch.float64 if exact else torch.float32
     total = raw.shape[-1]
     sum_vec = None
     sumsq_vec = None
@@ -45,7 +49,7 @@ def znorm_stats_streaming(raw: torch.Tensor, chunk_tokens: int, eps: float = 1e-
     start = 0
     while start < total:
         cur = min(chunk_tokens, total - start)
-        chunk = raw[..., start:start + cur].to(torch.float32)
+        chunk = raw[..., start:start + cur].to(ft)
         cs = chunk.sum(dim=-1)
         cq = (chunk * chunk).sum(dim=-1)
         sum_vec = cs if sum_vec is None else sum_vec + cs
@@ -63,10 +67,10 @@ def znorm_stats_streaming(raw: torch.Tensor, chunk_tokens: int, eps: float = 1e-
     return mean, std_safe
 
 
-def guard_mask(total_tokens: int, window_size: int, prefill_len: int, protect_prefill: bool):
+def guard_mask(total_tokens: int, window_size: int, prefill_len: int, protect_prefill: bool, device="cpu"):
     """Bool [T]: True where a token is always kept (selector_hf.py:417-441,121-130)."""
-    pos = torch.arange(total_tokens)
-    mask = torch.zeros(total_tokens, dtype=torch.bool)
+    pos = torch.arange(total_tokens, device=device)
+    mask = torch.zeros(total_tokens, dtype=torch.bool, device=device)
     if window_size > 0 and total_tokens > 0:
         recent = min(window_size, total_tokens)
         mask |= pos >= max(0, total_tokens - recent)
@@ -98,22 +102,25 @@ def group_final_scores(
     protect_prefill: bool = False,
     chunk_tokens: int | None = None,
     layer_agg: str = "mean",
+    exact: bool = False,
 ) -> torch.Tensor:
     """Fin[Hkv, T]: z-norm -> guards(+inf) -> GQA max -> mean (or max) over layers.
 
     selector_hf.py:916-989.  The reference walks chunks in the outer loop and
     layers in the inner loop; per element that is the same sequence of fp32
     operations as below (subtract, divide, fill, max, running add in layer
-    order, one division by the layer count).
+    order, one division by the layer count).  ``exact``: the same formula on the
+    same fp32 raw scores with every operation in double precision (returns fp64).
     """
+    ft = torch.float64 if exact else torch.float32
     total = raw_by_layer[0].shape[-1]
     chunk = total if chunk_tokens is None else chunk_tokens
-    guard = guard_mask(total, window_size, prefill_len, protect_prefill)
+    guard = guard_mask(total, window_size, prefill_len, protect_prefill, raw_by_layer[0].device)
     agg = None
     for raw in raw_by_layer:
-        x = raw.to(torch.float32)
+        x = raw.to(ft)
         if normalize:
-            mean, std_safe = znorm_stats_streaming(x, chunk)
+            mean, std_safe = znorm_stats_streaming(x, chunk, exact=exact)
             x = (x - mean.view(-1, 1)) / std_safe.view(-1, 1)
         if bool(guard.any()):
             x = x.masked_fill(guard.view(1, -1), float("inf"))

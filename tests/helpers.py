@@ -120,6 +120,54 @@ def assert_keep_matches(keep: torch.Tensor, want: torch.Tensor, fin: torch.Tenso
     return swapped
 
 
+def exact_gate(raw_by_layer, num_kv_heads: int, **kw):
+    """The kept-set gate of one fixture, derived from the fixture itself.  ``raw_by_layer``: the fp32
+    raw scores the selection starts from; ``kw``: the selection settings (as for
+    ``oracle.selection.group_final_scores``).  Returns (fin64, bound): the selection scores of the
+    same formula evaluated in double precision, and the largest distance of the reference's own fp32
+    selection scores (the oracle restates its arithmetic operation for operation) from them -- how far
+    the reference itself sits from exact arithmetic on this fixture (its streaming variance
+    sum(x^2) - n * mean^2 cancels leading digits, runtime/selector_hf.py:902-909)."""
+    fin32 = osel.group_final_scores(raw_by_layer, num_kv_heads, **kw)
+    fin64 = osel.group_final_scores(raw_by_layer, num_kv_heads, exact=True, **kw)
+    finite = torch.isfinite(fin32)
+    bound = float((fin32[finite].double() - fin64[finite]).abs().max()) if bool(finite.any()) else 0.0
+    return fin64, bound
+
+
+def device_exact_gate(raw: torch.Tensor, b: int, t: int, num_kv_heads: int, k: int, block_size: int = 16, **kw):
+    """The same gate for sizes the CPU oracle does not finish in seconds: the oracle's selection formula
+    run on the device on the raw scores the two-pass scorer wrote (``raw``: [B, L, Tmax, A] fp32 from
+    ``ops.score_paged``), for sequence ``b`` of ``t`` tokens.  Returns (want, fin64, bound) on the CPU:
+    the keep rows of the fp32 evaluation with the reference's chunked sums, the double-precision selection
+    scores, and the largest distance between the two evaluations."""
+    rows = [raw[b, l, :t].t() for l in range(raw.shape[1])]
+    kw.setdefault("chunk_tokens", osel.score_chunk_tokens(block_size, t))
+    fin32 = osel.group_final_scores(rows, num_kv_heads, **kw)
+    fin64 = osel.group_final_scores(rows, num_kv_heads, exact=True, **kw)
+    finite = torch.isfinite(fin32)
+    bound = float((fin32[finite].double() - fin64[finite]).abs().max()) if bool(finite.any()) else 0.0
+    return osel.topk_ascending(fin32, k).cpu(), fin64.cpu(), bound
+
+
+def assert_keep_within_exact_bound(keep: torch.Tensor, want: torch.Tensor, fin64: torch.Tensor, k: int, bound: float):
+    """Kept sets equal to the reference's, except indices whose exact (double precision) selection score
+    lies no further from the exact threshold score (the k-th largest) than ``bound``, the reference's own
+    distance from exact arithmetic on this fixture: there the reference's fp32 rounding, not the formula,
+    decides which side of the threshold an index falls on.  Returns the number of such indices."""
+    swapped = 0
+    for h in range(want.shape[0]):
+        a, b = set(keep[h].tolist()), set(want[h].tolist())
+        if a == b:
+            continue
+        thr = float(torch.sort(fin64[h], descending=True).values[k - 1])
+        for idx in a ^ b:
+            gap = abs(float(fin64[h, idx]) - thr)
+            assert gap <= bound, (h, idx, float(fin64[h, idx]), thr, gap, bound)
+            swapped += 1
+    return swapped
+
+
 _TUNE_ENV = {"TRIATTN_RESIDENT_KERNEL": "resident_kernel", "TRIATTN_RESIDENT_WORKGROUPS": "resident_workgroups",
              "TRIATTN_RESIDENT_LAYER_SPLIT": "layer_split", "TRIATTN_MAX_KERNEL": "max_kernel"}
 

@@ -177,3 +177,36 @@ def test_chunk_size_rule():
     assert osel.score_chunk_tokens(16, 300, 4096) == 300
     assert osel.score_chunk_tokens(16, 5000, 4096) == 4096
     assert osel.score_chunk_tokens(16, 8, 4096) == 16
+
+
+def test_exact_mode_is_the_textbook_z_score_in_double():
+    """The double-precision mode of the selection scores (what the kept-set gate measures distances
+    against) is pinned by an independent evaluation: numpy float64, two-pass mean and unbiased
+    variance (not the streaming formula), max over each group of query heads, mean over layers,
+    guards as +inf.  The fp32 mode stays within a few eps * kappa of it, kappa = mean(x^2) / var(x)
+    being what the streaming variance cancels (here ~100, mean 10 against std 1)."""
+    import numpy as np
+    g = torch.Generator().manual_seed(5)
+    layers, hq, hkv, t = 3, 8, 2, 700
+    raw = [torch.randn(hq, t, generator=g) + 10.0 for _ in range(layers)]
+    kw = dict(window_size=16, prefill_len=5, protect_prefill=True, chunk_tokens=64)
+    fin64 = osel.group_final_scores(raw, hkv, exact=True, **kw)
+    assert fin64.dtype == torch.float64
+    acc = np.zeros((hkv, t))
+    for r in raw:
+        x = r.numpy().astype(np.float64)
+        z = (x - x.mean(-1, keepdims=True)) / x.std(-1, ddof=1, keepdims=True)
+        acc += z.reshape(hkv, hq // hkv, t).max(1)
+    want = acc / layers
+    guard = np.zeros(t, dtype=bool)
+    guard[:5] = True
+    guard[-16:] = True
+    got = fin64.numpy()
+    assert np.isinf(got[:, guard]).all() and (got[:, guard] > 0).all()
+    assert np.abs(got[:, ~guard] - want[:, ~guard]).max() < 1e-12
+    fin32 = osel.group_final_scores(raw, hkv, **kw)
+    dev = np.abs(fin32.numpy().astype(np.float64)[:, ~guard] - want[:, ~guard]).max()
+    assert 1e-7 < dev < 64 * 2.0 ** -24 * 101 * np.abs(want[:, ~guard]).max()
+    # the layer maximum and the unnormalised variant take the same route
+    mx = osel.group_final_scores(raw, hkv, exact=True, layer_agg="max", normalize=False, window_size=0)
+    assert torch.equal(mx, torch.stack([r.double().view(hkv, hq // hkv, t).max(1).values for r in raw]).max(0).values)
