@@ -319,14 +319,23 @@ def test_group_selection_matches_reference_golden(tag, kw, path, fixture, monkey
 
 
 @pytest.mark.parametrize("tag,protect", [("default", False), ("chunk64_prefill", True)])
-@pytest.mark.parametrize("path,copies,workgroups", [
-    ("two_pass", 1, None),
-    ("resident_mfma", 1, 5),        # five tiles of 1024 tokens on the eight-wave instance the benchmark times
-    ("resident_mfma", 3, 15),       # three requests in one launch, each must come out as the single one
-    ("resident_mfma", 3, 10),       # ... and in two launches (two sequences, then one)
-    ("resident_valu", 1, 5),
+@pytest.mark.parametrize("fixture,path,copies,workgroups", [
+    ("selector_c1_shape.pt", "two_pass", 1, None),
+    ("selector_c1_shape.pt", "resident_mfma", 1, 5),    # five tiles of 1024 tokens on the eight-wave instance the benchmark times
+    ("selector_c1_shape.pt", "resident_mfma", 3, 15),   # three requests in one launch, each must come out as the single one
+    ("selector_c1_shape.pt", "resident_mfma", 3, 10),   # ... and in two launches (two sequences, then one)
+    ("selector_c1_shape.pt", "resident_valu", 1, 5),
+    # eight query heads per KV head (Qwen3-32B attention), 37 % kept: tiles of 512 tokens on the instance the
+    # 8 x 32768-token configuration runs (two column groups, slack of 64)
+    ("selector_c2_shape.pt", "two_pass", 1, None),
+    ("selector_c2_shape.pt", "resident_mfma", 1, 10),
+    ("selector_c2_shape.pt", "resident_mfma", 2, 10),   # two requests, one launch each
+    # head dimension 64 with the statistics shipped for GPT-OSS-120B and its YaRN frequencies
+    ("selector_gpt_oss_shape.pt", "two_pass", 1, None),
+    ("selector_gpt_oss_shape.pt", "resident_mfma", 1, 10),
+    ("selector_gpt_oss_shape.pt", "resident_mfma", 2, 20),
 ])
-def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(tag, protect, path, copies,
+def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(tag, protect, fixture, path, copies,
                                                                                 workgroups, monkeypatch):
     """The reference's keep sets for a 5000-token request of 32 query / 8 KV heads of 128 (budget
     2048, window 128; written by tests/golden/make_c1_shape_golden.py): its variance streams over
@@ -337,7 +346,7 @@ def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(
     further from the double-precision threshold than the reference's own fp32 selection scores lie
     from the double-precision ones on this fixture (helpers.exact_gate)."""
     from golden.hashed_inputs import checksum, hashed_rows
-    gold = load_golden("selector_c1_shape.pt")
+    gold = load_golden(fixture)
     layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
     keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
     assert checksum(keys) == int(gold["key_checksum"]), "the hashed keys differ from the ones the golden was written for"
@@ -367,8 +376,11 @@ def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(
     keep, _, ws = ops.select_paged(kv, batch, sc, sel)
     assert ws.status() == 0
     want = gold[f"group_{tag}_keep"].long()
-    okeep, ofin, fin64, bound = _c1_shape_oracle(tag)
-    assert torch.equal(okeep, want)          # the oracle reproduces the reference's keep set exactly
+    okeep, ofin, fin64, bound = _head_shape_oracle(fixture, tag)
+    # The oracle reproduces the reference's keep set: exactly on the machine the golden was written on
+    # (tests/test_oracle_selection.py asserts that); torch's CPU reductions associate differently on other
+    # CPUs, so here the two may differ where the fp32 evaluation itself is undecided.
+    assert_keep_within_exact_bound(okeep, want, fin64, int(gold["budget"]), bound)
     scale = float(ofin[torch.isfinite(ofin)].abs().max())
     # (the reference's own distance from exact arithmetic: 8e-6 of the largest score with one 4096-token
     # chunk, 2e-5 with chunks of 64; the kernels, which sum the statistics in double, sit 6e-6 .. 7e-6 away)
@@ -379,18 +391,19 @@ def test_group_selection_at_the_benchmarked_head_shape_matches_reference_golden(
         # Identical to the reference's rows except where the reference's own fp32 rounding, not the
         # formula, decides on which side of the threshold an index falls.
         swapped += assert_keep_within_exact_bound(got[c], want, fin64, budget, bound)
-    record_swaps(f"reference_golden_c1_shape:{path}:{copies}x:{workgroups}:{tag}", swapped, copies * hkv * budget)
+    record_swaps(f"reference_golden_{fixture[9:-9]}_shape:{path}:{copies}x:{workgroups}:{tag}", swapped,
+                 copies * hkv * budget)
     assert swapped <= 2 * copies, swapped
 
 
-_C1_SHAPE_ORACLE: dict = {}
+_HEAD_SHAPE_ORACLE: dict = {}
 
 
-def _c1_shape_oracle(tag):
-    """Keep rows and selection scores of the CPU oracle for tests/golden/selector_c1_shape.pt."""
-    if tag not in _C1_SHAPE_ORACLE:
+def _head_shape_oracle(fixture, tag):
+    """Keep rows, fp32 and double-precision selection scores of the CPU oracle for a head-shape golden."""
+    if (fixture, tag) not in _HEAD_SHAPE_ORACLE:
         from golden.hashed_inputs import hashed_rows
-        gold = load_golden("selector_c1_shape.pt")
+        gold = load_golden(fixture)
         layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
         keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
         offs = osc.geometric_offsets(65536)
@@ -399,8 +412,8 @@ def _c1_shape_oracle(tag):
                for l in range(layers)]
         kw = dict(chunk_tokens=64, protect_prefill=True) if tag == "chunk64_prefill" else dict(chunk_tokens=4096)
         kw.update(window_size=int(gold["window"]), prefill_len=int(gold["prefill_len"]))
-        _C1_SHAPE_ORACLE[tag] = osel.group_keep_per_head(raw, hkv, int(gold["budget"]), **kw) + exact_gate(raw, hkv, **kw)
-    return _C1_SHAPE_ORACLE[tag]
+        _HEAD_SHAPE_ORACLE[(fixture, tag)] = osel.group_keep_per_head(raw, hkv, int(gold["budget"]), **kw) + exact_gate(raw, hkv, **kw)
+    return _HEAD_SHAPE_ORACLE[(fixture, tag)]
 
 
 @pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])

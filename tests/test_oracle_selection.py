@@ -72,14 +72,18 @@ def test_layer_selection_matches_reference(tag, fixture):
     assert torch.equal(keep, want)
 
 
+@pytest.mark.parametrize("fixture", ["selector_c1_shape.pt", "selector_c2_shape.pt", "selector_gpt_oss_shape.pt"])
 @pytest.mark.parametrize("tag,kw", [("default", dict(chunk_tokens=4096)),
                                     ("chunk64_prefill", dict(chunk_tokens=64, protect_prefill=True))])
-def test_group_selection_matches_reference_across_chunks_at_the_benchmarked_head_shape(tag, kw):
-    """32 query / 8 KV heads of 128, 5000 tokens, budget 2048: the reference's streaming variance
-    spans two 4096-token chunks (79 chunks of 64 in the second setting) and its chunked top-k
-    merges.  The keys are rebuilt from the fixture's seed and checked against its checksum."""
+def test_group_selection_matches_reference_across_chunks_at_the_benchmarked_head_shape(tag, kw, fixture):
+    """5000 tokens at the benchmarked head shapes -- 32 query / 8 KV heads of 128 at budget 2048, 64 / 8
+    heads of 128 at budget 1850 (eight query heads per KV head, 37 % kept), 64 / 8 heads of 64 with two
+    layers of the statistics the reference ships for GPT-OSS-120B and that model's YaRN frequencies: the
+    reference's streaming variance spans two 4096-token chunks (79 chunks of 64 in the second setting)
+    and its chunked top-k merges.  The keys are rebuilt from the fixture's seed and checked against its
+    checksum."""
     from golden.hashed_inputs import checksum, hashed_rows
-    gold = load_golden("selector_c1_shape.pt")
+    gold = load_golden(fixture)
     layers, hq, hkv, d, t, bs = (int(x) for x in gold["shape"])
     keys = hashed_rows(int(gold["key_seed"]), layers, hkv, t, d)
     assert checksum(keys) == int(gold["key_checksum"])
