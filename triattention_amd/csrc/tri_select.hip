@@ -399,9 +399,27 @@ __global__ __launch_bounds__(kTopkThreads) void topk_rows_reg_kernel(const float
   for (int shift = 24; shift >= 0; shift -= 8) {
     if (tid < 256) hist[tid] = 0;
     __syncthreads();
+    // Selection scores are sums of z-scores of similar size, so the leading digit (sign and the top
+    // exponent bits) takes three or four values in a whole row and the first pass would send all 64
+    // lanes of every atomic to the same few counters, one after the other.  The lanes of a wave that
+    // hold the same digit are counted with a ballot and added once (up to four distinct digits per
+    // round; what is left, and the later passes, whose digits are spread, take the plain atomics).
 #pragma unroll
-    for (int i = 0; i < VPT; ++i)
-      if (i < nvalid && (key[i] & mask) == prefix) atomicAdd(&hist[(key[i] >> shift) & 255u], 1u);
+    for (int i = 0; i < VPT; ++i) {
+      const bool part = i < nvalid && (key[i] & mask) == prefix;
+      const uint32_t digit = (key[i] >> shift) & 255u;
+      unsigned long long todo = __ballot(part);
+      if (shift == 24) {
+        for (int it = 0; it < 4 && todo; ++it) {
+          const int leader = __builtin_amdgcn_readfirstlane(__ffsll((long long)todo) - 1);
+          const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)digit, leader);
+          const unsigned long long same = __ballot(part && digit == dl) & todo;
+          if (lane == leader) atomicAdd(&hist[dl], (uint32_t)__popcll(same));
+          todo &= ~same;
+        }
+      }
+      if ((todo >> lane) & 1ull) atomicAdd(&hist[digit], 1u);
+    }
     __syncthreads();
     if (wave == 0) {
       // lane owns bins 4*lane .. 4*lane+3; ge[j] = candidates whose digit is >= that bin
