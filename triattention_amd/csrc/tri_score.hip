@@ -513,7 +513,6 @@ __global__ __launch_bounds__(kScoreThreads) void score_max_kernel(ScoreArgs a) {
 // rows and per-tile sums.
 typedef __bf16 mx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float mx_f32x4 __attribute__((ext_vector_type(4)));
-constexpr int kDppRowMirror = 0x140;   // row_mirror
 constexpr int kDppRor4 = 0x124;        // row_ror:4
 
 __device__ __forceinline__ mx_f32x4 mx_mfma(const uint4& a, const uint4& b, mx_f32x4 c) {
@@ -535,15 +534,76 @@ __device__ __forceinline__ float bf16_elem(const uint4& v, int e) {   // e: comp
   return (e & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
 }
 
+// max(keep, send of the lane `lane ^ 1` / `^ 2` / `^ 4` / `^ 8` of the row of 16): one instruction (two
+// for ^ 4, which no single lane pattern of this chip expresses).  Written out because the compiler puts a
+// quieting v_max in front of every operand of fmaxf and moves the other lane's value into a register
+// first; the idle cycles cover the distance this chip requires between a vector instruction's write and a
+// lane-crossing read of that register.
+__device__ __forceinline__ float max_xor1(float keep, float send) {
+  float r;
+  asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(send), "v"(keep));
+  return r;
+}
+__device__ __forceinline__ float max_xor2(float keep, float send) {
+  float r;
+  asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(send), "v"(keep));
+  return r;
+}
+__device__ __forceinline__ float max_xor4(float keep, float send) {
+  float r = keep;      // lanes 0..3 and 8..11 of a row take lane + 4, the others lane - 4
+  asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+      "v_max_f32_dpp %0, %1, %0 row_ror:4 row_mask:0xf bank_mask:0xa" : "+v"(r) : "v"(send));
+  return r;
+}
+__device__ __forceinline__ float max_xor8(float keep, float send) {
+  float r;
+  asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %2 row_ror:8 row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(send), "v"(keep));
+  return r;
+}
+__device__ __forceinline__ float max_plain(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+// m[i] = sqrt(x[i].lo^2 + x[i].hi^2) for four packed bf16 pairs (see magnitudes4 of the resident kernel:
+// the spacing this chip requires after a dot product's and a transcendental's write is provided here).
+__device__ __forceinline__ void pair_magnitudes4(const uint32_t (&x)[4], float* m) {
+  asm("v_dot2_f32_bf16 %0, %4, %4, 0\n\t"
+      "v_dot2_f32_bf16 %1, %5, %5, 0\n\t"
+      "v_dot2_f32_bf16 %2, %6, %6, 0\n\t"
+      "v_dot2_f32_bf16 %3, %7, %7, 0\n\t"
+      "v_sqrt_f32 %0, %0\n\t"
+      "v_sqrt_f32 %1, %1\n\t"
+      "v_sqrt_f32 %2, %2\n\t"
+      "v_sqrt_f32 %3, %3\n\t"
+      "s_nop 0"
+      : "=&v"(m[0]), "=&v"(m[1]), "=&v"(m[2]), "=&v"(m[3])
+      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]));
+}
+typedef __bf16 mx_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float mx_f32x2 __attribute__((ext_vector_type(2)));
+// Two fp32 values as packed bf16 and what is left of them as packed bf16 (16 bits of each value).
+__device__ __forceinline__ void split_pair_bf16(float x0, float x1, uint32_t& hi, uint32_t& lo) {
+  const mx_f32x2 x = {x0, x1};
+  hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, mx_bf16x2));
+  const mx_f32x2 r = {x0 - __uint_as_float(hi << 16), x1 - __uint_as_float(hi & 0xffff0000u)};
+  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(r, mx_bf16x2));
+}
+
 constexpr int kMaxMfmaHeads = 4;   // query heads of one KV head per workgroup
+constexpr int kMaxMfmaTilesPerGroup = 8;   // consecutive 512-token tiles per workgroup
+// Waves of a workgroup (they share the operand slabs in LDS; two workgroups fit a CU).  Eight waves, four
+// per SIMD in 128 registers, run no faster (6.84 against 6.85 ms on 16 x 16384 tokens x 36 layers).
+constexpr int kMaxMfmaWaves = 4;
+constexpr int kMaxMfmaThreads = kMaxMfmaWaves * 64;
 constexpr int kTrigPitch = 65;     // floats per offset in LDS (odd: 16 offsets read at once fall into 16 banks)
 __host__ __device__ constexpr size_t max_mfma_lds_bytes(int nx, int no) {
   return (size_t)(kMaxMfmaHeads + nx) * 12 * 64 * 16 + 2 * 64 * 16 + 3 * kMaxMfmaHeads * 64 * 4 +
-         (size_t)2 * no * kTrigPitch * 4 + (kScoreTileTokens + 2) * 4 + 4 * kMaxMfmaHeads * 2 * 4;
+         (size_t)2 * no * kTrigPitch * 4 + (kScoreTileTokens + 2) * 4 + kMaxMfmaWaves * kMaxMfmaHeads * 2 * 4;
 }
 
 template <int NX, bool IL>
-__global__ __launch_bounds__(kScoreThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(kMaxMfmaThreads) __attribute__((amdgpu_waves_per_eu(kMaxMfmaWaves / 2, kMaxMfmaWaves / 2)))
 void score_max_mfma_kernel(ScoreArgs a) {
   constexpr int F = 64;
   constexpr int NT = kMaxMfmaHeads + NX;
@@ -554,31 +614,25 @@ void score_max_mfma_kernel(ScoreArgs a) {
   float* tcos = cf + 3 * kMaxMfmaHeads * F;                    // [NO][kTrigPitch]
   float* tsin = tcos + a.NO * kTrigPitch;                      // [NO][kTrigPitch]
   int* lds_blk = reinterpret_cast<int*>(tsin + a.NO * kTrigPitch);   // [kScoreTileTokens + 2]
-  float* red = reinterpret_cast<float*>(lds_blk + kScoreTileTokens + 2);   // [4 waves][4 heads][2]
+  float* red = reinterpret_cast<float*>(lds_blk + kScoreTileTokens + 2);   // [waves][4 heads][2]
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int tile = blockIdx.x;
   const int head = blockIdx.y / a.QC, qc = blockIdx.y % a.QC;
+  const int tile_group = blockIdx.x;
   const int q0 = qc * kMaxMfmaHeads, nq = min(kMaxMfmaHeads, a.G - q0);
   const int b = blockIdx.z / a.L, l = blockIdx.z % a.L;
   const int seq_len = a.seq_lens[b];
-  const int n0 = tile * kScoreTileTokens;
-  if (n0 >= seq_len) return;
-  const int n1 = min(n0 + kScoreTileTokens, seq_len);
+  // The operand slabs depend on (sequence, layer, KV head, group of query heads) only: a workgroup
+  // builds them once (as many vector instructions as scoring 400 tokens) and then takes
+  // kMaxMfmaTilesPerGroup consecutive tiles of 512 tokens.
+  if (tile_group * kMaxMfmaTilesPerGroup * kScoreTileTokens >= seq_len) return;
 
-  int lb0 = 0;
-  if (a.block_table_pitch >= 0) {
-    lb0 = n0 / a.block_size;
-    const int lb1 = (n1 - 1) / a.block_size;
-    for (int i = threadIdx.x; i <= lb1 - lb0; i += kScoreThreads)
-      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
-  }
-  for (int i = threadIdx.x; i < 3 * kMaxMfmaHeads * F; i += kScoreThreads) {
+  for (int i = threadIdx.x; i < 3 * kMaxMfmaHeads * F; i += kMaxMfmaThreads) {
     const int which = i / (kMaxMfmaHeads * F), q = (i / F) % kMaxMfmaHeads, f = i % F;
     const int ah = head * a.G + q0 + min(q, nq - 1);
     cf[i] = q < nq ? a.coef[(((int64_t)(b * a.L + l) * a.A + ah) * 3 + which) * F + f] : 0.f;
   }
-  for (int i = threadIdx.x; i < a.NO * F; i += kScoreThreads) {
+  for (int i = threadIdx.x; i < a.NO * F; i += kMaxMfmaThreads) {
     const int j = i / F, f = i % F;
     tcos[j * kTrigPitch + f] = a.trig[((int64_t)(b * a.NO + j) * 2 + 0) * F + f];
     tsin[j * kTrigPitch + f] = a.trig[((int64_t)(b * a.NO + j) * 2 + 1) * F + f];
@@ -588,13 +642,15 @@ void score_max_mfma_kernel(ScoreArgs a) {
   // Operand slabs.  Lane (c16 = lane % 16, kb = lane / 16) of slab (t, s) holds one column
   // and key elements 32 s + 8 kb + 0..7; the column is (head t, offset c16) in the first
   // four tiles and (head c16 % 4, offset 16 + 4 (t - 4) + c16 / 4) in the others.
-  for (int i = threadIdx.x; i < NT * 4 * 64; i += kScoreThreads) {
+  for (int i = threadIdx.x; i < NT * 4 * 64; i += kMaxMfmaThreads) {
     const int ln = i & 63, sl = (i >> 6) & 3, t = i >> 8;
     const int c16 = ln & 15, kb = ln >> 4;
     const int q = t < kMaxMfmaHeads ? t : (c16 & 3);
     const int j = t < kMaxMfmaHeads ? c16 : 16 + 4 * (t - kMaxMfmaHeads) + (c16 >> 2);
-    const bool live = q < nq && j < a.NO;
-    const int jc = live ? j : 0;
+    // A column beyond the last offset repeats a live one of the same head (the first, or in the
+    // further tiles the last), so that the maxima below need no masks.
+    const bool live = q < nq;
+    const int jc = j < a.NO ? j : (t < kMaxMfmaHeads ? 0 : a.NO - 1);
     uint32_t w[3][4];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -618,7 +674,7 @@ void score_max_mfma_kernel(ScoreArgs a) {
   }
   // Magnitude slabs: column c16 = query head (c16 % 4), piece (c16 / 4) of E; element e of slab
   // m is the pair whose magnitude the same lane forms from its key registers below.
-  for (int i = threadIdx.x; i < 2 * 64; i += kScoreThreads) {
+  for (int i = threadIdx.x; i < 2 * 64; i += kMaxMfmaThreads) {
     const int ln = i & 63, m = i >> 6;
     const int c16 = ln & 15, kb = ln >> 4;
     const int q = c16 & 3, piece = c16 >> 2;
@@ -635,21 +691,35 @@ void score_max_mfma_kernel(ScoreArgs a) {
     }
     Bm[m * 64 + ln] = uint4{w[0], w[1], w[2], w[3]};
   }
-  __syncthreads();
 
   const int r16 = lane & 15, kb = lane >> 4;
-  const bool main_col = r16 < a.NO;             // this lane's column of the first four tiles is an offset
-  bool extra_col[NX > 0 ? NX : 1];              // ... and of the further tiles
-#pragma unroll
-  for (int x = 0; x < NX; ++x) extra_col[x] = 16 + 4 * x + (r16 >> 2) < a.NO;
+  const bool b0 = (r16 & 1) != 0, b1 = (r16 & 2) != 0, b2 = (r16 & 4) != 0, b3 = (r16 & 8) != 0;
+  // After the maxima lane r16 of a row group holds the score of query head r16 % 4 and of the group's
+  // token r16 / 4: every lane stores one score.
+  const int out_q = r16 & 3, out_i = r16 >> 2;
+  const bool far_spread = a.NO > 17;            // more than one offset beyond the first 16: they sit in different lanes
   const char* kbase = reinterpret_cast<const char*>(a.k_layers[l]);
   const int64_t lane_off = (int64_t)head * a.stride_head + 8 * kb;
-  constexpr int TW = kScoreTileTokens / 4;
+  constexpr int TW = kScoreTileTokens / kMaxMfmaWaves;
+  const bool out_lane = out_q < nq;
+  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer +
+                   (int64_t)(head * a.G + q0 + (out_lane ? out_q : 0)) * a.raw_stride_head;
+
+  for (int tile = tile_group * kMaxMfmaTilesPerGroup; tile < (tile_group + 1) * kMaxMfmaTilesPerGroup; ++tile) {
+  const int n0 = tile * kScoreTileTokens;
+  if (n0 >= seq_len) break;                     // (the same for every thread of the workgroup)
+  const int n1 = min(n0 + kScoreTileTokens, seq_len);
+  __syncthreads();                              // slabs built; the previous tile's block ids and sums read
+  int lb0 = 0;
+  if (a.block_table_pitch >= 0) {
+    lb0 = n0 / a.block_size;
+    const int lb1 = (n1 - 1) / a.block_size;
+    for (int i = threadIdx.x; i <= lb1 - lb0; i += kMaxMfmaThreads)
+      lds_blk[i] = a.block_table[(int64_t)b * a.block_table_pitch + lb0 + i];
+    __syncthreads();
+  }
   const int wstart = n0 + wave * TW;
   const int wend = min(wstart + TW, n1);
-  const bool out_lane = r16 < nq;
-  float* raw_row = a.raw + (int64_t)(b * a.L + l) * a.raw_stride_layer +
-                   (int64_t)(head * a.G + q0 + (out_lane ? r16 : 0)) * a.raw_stride_head;
   float s1 = 0.f, s2 = 0.f;
 
   // Row lane % 16 of the step that starts at token t0: four 16-byte pieces, one per key slab.
@@ -675,70 +745,96 @@ void score_max_mfma_kernel(ScoreArgs a) {
 
   // What follows the key products of one 16-token step: magnitude term, maxima, stores.
   auto finish = [&](const uint4 (&A)[4], mx_f32x4 (&acc)[NT], int t0) __attribute__((always_inline)) {
-    // Magnitudes of this lane's 16 pairs as two bf16 pieces each.
+    // Magnitudes of this lane's 16 pairs (dot product of the bf16 pair with itself, square root) as
+    // two bf16 pieces each.
     mx_f32x4 accm = mx_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
+      float mag[8];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint32_t x[4];
+        if (IL) {
+          const uint4& v = A[2 * m + h];
+          x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+        } else {
+          const uint32_t re[2] = {h ? A[m].z : A[m].x, h ? A[m].w : A[m].y};
+          const uint32_t im[2] = {h ? A[m + 2].z : A[m + 2].x, h ? A[m + 2].w : A[m + 2].y};
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            x[2 * i] = __builtin_amdgcn_perm(im[i], re[i], 0x05040100u);
+            x[2 * i + 1] = __builtin_amdgcn_perm(im[i], re[i], 0x07060302u);
+          }
+        }
+        pair_magnitudes4(x, &mag[4 * h]);
+      }
       uint32_t hi[4], lo[4];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float kr, ki;
-        if (IL) {
-          kr = bf16_elem(A[2 * m + (e >> 2)], 2 * (e & 3));
-          ki = bf16_elem(A[2 * m + (e >> 2)], 2 * (e & 3) + 1);
-        } else {
-          kr = bf16_elem(A[m], e);
-          ki = bf16_elem(A[m + 2], e);
-        }
-        const float mag = __builtin_amdgcn_sqrtf(fmaf(ki, ki, kr * kr));
-        const uint32_t h = bf16_bits(mag);
-        const uint32_t lw = bf16_bits(mag - __uint_as_float(h << 16));
-        if (e & 1) { hi[e >> 1] |= h << 16; lo[e >> 1] |= lw << 16; }
-        else { hi[e >> 1] = h; lo[e >> 1] = lw; }
-      }
+      for (int i = 0; i < 4; ++i) split_pair_bf16(mag[2 * i], mag[2 * i + 1], hi[i], lo[i]);
       const uint4 bm = Bm[m * 64 + lane];
       accm = mx_mfma(uint4{lo[0], lo[1], lo[2], lo[3]}, bm, accm);
       accm = mx_mfma(uint4{hi[0], hi[1], hi[2], hi[3]}, bm, accm);
     }
 
-    // Offsets from 16 on: the maximum over this lane's columns of the further tiles, then over
-    // the four lanes of the same query head (lane % 4).
-    float far[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    // Offsets 0..15 of head q are the 16 lanes of a row group in tile q: 16 values per lane (4 heads x 4
+    // tokens), each to be maximised over the 16 lanes.  A transposed butterfly: at every stage a lane
+    // keeps half of its values and hands the other half to the lane one bit away, so the 16 + 8 + 4 + 2
+    // values shrink to the one of (head r16 % 4, token r16 / 4) in 15 exchanges.
+    float u[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const float x = acc[2 * p][i], y = acc[2 * p + 1][i];
+        u[p][i] = max_xor1(b0 ? y : x, b0 ? x : y);
+      }
+    float v4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v4[i] = max_xor2(b1 ? u[1][i] : u[0][i], b1 ? u[0][i] : u[1][i]);
+    float w2[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) w2[p] = max_xor4(b2 ? v4[2 * p + 1] : v4[2 * p], b2 ? v4[2 * p] : v4[2 * p + 1]);
+    float best = max_xor8(b3 ? w2[1] : w2[0], b3 ? w2[0] : w2[1]);
+
+    // Offsets from 16 on: the further tiles hold them as column 4 (j - 16) + head, i.e. this lane's head
+    // already; the maximum over the tiles, then (more than one such offset) over the four lanes of the head.
     if constexpr (NX > 0) {
+      float f[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = -INFINITY;
+        float v = acc[kMaxMfmaHeads][i];
 #pragma unroll
-        for (int x = 0; x < NX; ++x) v = extra_col[x] ? fmaxf(v, acc[kMaxMfmaHeads + x][i]) : v;
-        v = fmaxf(v, dpp<kDppRor4>(v));
-        v = fmaxf(v, dpp<kDppRor8>(v));
-        far[i] = v;
+        for (int x = 1; x < NX; ++x) v = max_plain(v, acc[kMaxMfmaHeads + x][i]);
+        f[i] = v;
       }
-    }
-    // Offsets 0..15 of head q: the 16 lanes of the row group; lane q keeps the result.
-    float val[4] = {0.f, 0.f, 0.f, 0.f};
+      float v = b3 ? (b2 ? f[3] : f[2]) : (b2 ? f[1] : f[0]);
+      if (far_spread) {
+        // every lane of the head needs the maximum of token out_i over the head's four lanes, which
+        // hold different tokens' selections: reduce all four tokens, then select
 #pragma unroll
-    for (int q = 0; q < kMaxMfmaHeads; ++q) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v = main_col ? acc[q][i] : -INFINITY;
-        v = fmaxf(v, dpp<kDppXor1>(v));
-        v = fmaxf(v, dpp<kDppXor2>(v));
-        v = fmaxf(v, dpp<kDppHalfMirror>(v));
-        v = fmaxf(v, dpp<kDppRowMirror>(v));
-        if (r16 == q) val[i] = v;
+        for (int i = 0; i < 4; ++i) {
+          f[i] = max_xor4(f[i], f[i]);
+          f[i] = max_xor8(f[i], f[i]);
+        }
+        v = b3 ? (b2 ? f[3] : f[2]) : (b2 ? f[1] : f[0]);
       }
+      best = max_plain(best, v);
     }
+    // Magnitude term: the three pieces of E sit four lanes apart (column group 3 is zero).
+    float ex[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float ex = accm[i] + __shfl_down(accm[i], 4, 16) + __shfl_down(accm[i], 8, 16);
-      const int tk = t0 + 4 * kb + i;
-      if (out_lane && tk < wend) {
-        const float v = fmaxf(val[i], far[i]) + ex;
-        raw_row[(int64_t)tk * a.raw_stride_token] = v;
-        s1 += v;
-        s2 = fmaf(v, v, s2);
-      }
+      float x = accm[i];
+      x += dpp<kDppRor4>(x);
+      x += dpp<kDppRor8>(x);
+      ex[i] = x;
+    }
+    const float v = best + (b3 ? (b2 ? ex[3] : ex[2]) : (b2 ? ex[1] : ex[0]));
+    const int tk = t0 + 4 * kb + out_i;
+    if (out_lane && tk < wend) {
+      raw_row[(int64_t)tk * a.raw_stride_token] = v;
+      s1 += v;
+      s2 = fmaf(v, v, s2);
     }
   };
 
@@ -765,7 +861,8 @@ void score_max_mfma_kernel(ScoreArgs a) {
           acc1[t] = mx_mfma(A1[sl], bk, acc1[t]);
         }
       // One tile's operands at a time: left to itself the scheduler requests the slabs of all
-      // tiles up front and spills the keys to make room for them.
+      // tiles up front and spills the keys to make room for them.  (Requesting a tile's twelve slabs
+      // one tile ahead, into a second set of registers, changes nothing: 6.84 -> 6.86 ms.)
       __builtin_amdgcn_sched_barrier(0);
     }
     finish(A0, acc0, t0);
@@ -776,8 +873,9 @@ void score_max_mfma_kernel(ScoreArgs a) {
   }
 
   // Per-tile sums of every query head: over the four row groups of a wave, then the waves.
-  s1 += __shfl_xor(s1, 16); s1 += __shfl_xor(s1, 32);
-  s2 += __shfl_xor(s2, 16); s2 += __shfl_xor(s2, 32);
+  // (lane r16 of every row group holds the sums of head r16 % 4 over its token r16 / 4)
+  s1 += __shfl_xor(s1, 4); s1 += __shfl_xor(s1, 8); s1 += __shfl_xor(s1, 16); s1 += __shfl_xor(s1, 32);
+  s2 += __shfl_xor(s2, 4); s2 += __shfl_xor(s2, 8); s2 += __shfl_xor(s2, 16); s2 += __shfl_xor(s2, 32);
   if (lane < kMaxMfmaHeads) {
     red[(wave * kMaxMfmaHeads + lane) * 2 + 0] = s1;
     red[(wave * kMaxMfmaHeads + lane) * 2 + 1] = s2;
@@ -785,7 +883,7 @@ void score_max_mfma_kernel(ScoreArgs a) {
   __syncthreads();
   if ((int)threadIdx.x < nq) {
     float t1 = 0.f, t2 = 0.f;
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < kMaxMfmaWaves; ++w) {
       t1 += red[(w * kMaxMfmaHeads + threadIdx.x) * 2 + 0];
       t2 += red[(w * kMaxMfmaHeads + threadIdx.x) * 2 + 1];
     }
@@ -793,6 +891,7 @@ void score_max_mfma_kernel(ScoreArgs a) {
     out[0] = t1;
     out[1] = t2;
   }
+  }   // tiles of this workgroup
 }
 
 template <int NX>
@@ -801,15 +900,15 @@ hipError_t launch_max_mfma_nx(const ScoreArgs& k, dim3 grid, int il, size_t lds,
                       : reinterpret_cast<const void*>(&score_max_mfma_kernel<NX, false>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  if (il) hipLaunchKernelGGL((score_max_mfma_kernel<NX, true>), grid, dim3(kScoreThreads), lds, s, k);
-  else hipLaunchKernelGGL((score_max_mfma_kernel<NX, false>), grid, dim3(kScoreThreads), lds, s, k);
+  if (il) hipLaunchKernelGGL((score_max_mfma_kernel<NX, true>), grid, dim3(kMaxMfmaThreads), lds, s, k);
+  else hipLaunchKernelGGL((score_max_mfma_kernel<NX, false>), grid, dim3(kMaxMfmaThreads), lds, s, k);
   return hipGetLastError();
 }
 
 hipError_t launch_max_mfma(const ScoreArgs& k, int B, int il, hipStream_t s) {
   const int nx = k.NO > 16 ? ceil_div(k.NO - 16, 4) : 0;
   const size_t lds = max_mfma_lds_bytes(nx, k.NO);
-  dim3 grid(k.num_tiles, k.Hkv * k.QC, B * k.L);
+  dim3 grid(ceil_div(k.num_tiles, kMaxMfmaTilesPerGroup), k.Hkv * k.QC, B * k.L);
   switch (nx) {
     case 0: return launch_max_mfma_nx<0>(k, grid, il, lds, s);
     case 1: return launch_max_mfma_nx<1>(k, grid, il, lds, s);
