@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # the same counters read for the 1 GiB copies of --copy-calibration).  Keyed by
 # (workload, path); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_482_130 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
+    ("c1_qwen3_8b_36l_b16_16k", "resident_mfma"): (9_472_453 * 1024 * 2 + 12_800 * 1024,     # fused_mfma_kernel
                                                     "profiles/c1_step_hbm_counters.txt"),
 }
 
