@@ -1432,3 +1432,33 @@ def test_research_path_selection_matches_oracle(hq, hkv, decode_start, keep_coun
                                   tie_tol=KEEP_TIE_TOL * scale)
     record_swaps(f"research_path_vs_oracle:{hq}/{hkv}:{decode_start}", swapped, hkv * k)
     assert swapped == 0
+
+
+@pytest.mark.parametrize("case", ["half_d128", "interleaved_d64", "half_scaled"])
+def test_research_path_scores_match_the_references_own_helpers(case):
+    """``hf_selection.score_keys_for_round`` -- the kernels on the cache's rotated keys, nothing un-rotated,
+    no position table -- against the scores the reference's research path computes for the same keys
+    with its own helpers (fixture written by tests/golden/make_hf_score_golden.py: ``invert_rope`` ->
+    ``compute_frequency_statistics_from_means`` -> ``score_keys_for_round``, methods/pruning_utils.py), for
+    mean and max over the offsets, with and without the MLR term, half and interleaved pairing, key
+    positions that do not start at zero and an attention scale of 1.25.  Tolerance: 1e-3 of a head's
+    RMS (the two forms evaluate fp32 phases of up to 65536 rad differently; measured ~1e-4)."""
+    from triattention_amd import hf_selection
+    gold = load_golden("hf_score.pt")[case]
+    k_rot = gold["k_rot"].to(DEV).unsqueeze(0)                                  # [1, Hkv, T, D] bf16, as a cache holds them
+    qc = torch.stack([gold["q_mean_real"], gold["q_mean_imag"]], dim=-1)
+    worst = 0.0
+    for tag, mlr in (("", False), ("_nomlr", True)):
+        for agg in ("mean", "max"):
+            print(f"research path scores: {case} {agg}{tag}", flush=True)
+            got = hf_selection.score_keys_for_round(k_rot, qc, gold["q_abs_mean"], gold["inv_freq"], gold["offsets"],
+                                                    gold["freq_scale_sq"], int(gold["round_start"]), aggregation=agg,
+                                                    rope_style=gold["style"], attention_scale=float(gold["scale"]),
+                                                    disable_mlr=mlr).cpu()
+            want = gold[f"scores_{agg}{tag}"]
+            assert got.shape == want.shape and got.dtype == torch.float32
+            rms = want.pow(2).mean(dim=-1, keepdim=True).sqrt()
+            err = float(((got - want).abs() / rms).max())
+            worst = max(worst, err)
+            assert err < 1e-3, (case, agg, tag, err)
+    print(f"research path scores: {case} worst error {worst:.2e} of a head's RMS", flush=True)

@@ -185,3 +185,37 @@ def test_fp8_dequant_closed_form():
     codes = torch.tensor([[[0.5, -1.5, 448.0, 0.0]]]).to(torch.float8_e4m3fn)
     scales = torch.tensor([[0.25]])
     assert osc.dequant_fp8(codes, scales).flatten().tolist() == [0.125, -0.375, 112.0, 0.0]
+
+
+@pytest.mark.parametrize("case", ["half_d128", "interleaved_d64", "half_scaled"])
+def test_unrotated_form_matches_the_research_paths_own_scores(case):
+    """``oracle.scoring.raw_scores_unrotated`` (and ``oracle.calibration.invert_rope``, the same inverse
+    rotation) against outputs of the reference's own helpers on the keys of a Hugging Face cache
+    (fixture written by tests/golden/make_hf_score_golden.py from methods/pruning_utils.py:
+    ``invert_rope`` -> ``compute_frequency_statistics_from_means`` -> ``score_keys_for_round``): mean
+    and max over the offsets, with and without the MLR term.  Then the form the kernels evaluate --
+    rotated keys, no positions -- against the same reference scores: a rotated key carries its
+    position in its phase, and one factor of the attention scale."""
+    from oracle import calibration as ocal
+    gold = load_golden("hf_score.pt")[case]
+    style, scale = gold["style"], float(gold["scale"])
+    k_rot = gold["k_rot"]
+    hkv = k_rot.shape[0]
+    hq = gold["q_abs_mean"].shape[0]
+    k_un = ocal.invert_rope(k_rot.float(), gold["cos"], gold["sin"], scale, style)
+    assert torch.equal(k_un, gold["k_unrot"])
+    qc = torch.stack([gold["q_mean_real"], gold["q_mean_imag"]], dim=-1)
+    fs = gold["freq_scale_sq"].unsqueeze(0).expand(hq, -1)
+    rs = int(gold["round_start"])
+    for tag, mlr in (("", False), ("_nomlr", True)):
+        for agg in ("mean", "max"):
+            want = gold[f"scores_{agg}{tag}"]
+            got = osc.raw_scores_unrotated(k_un.repeat_interleave(hq // hkv, dim=0), gold["positions"], qc,
+                                           gold["q_abs_mean"], gold["inv_freq"], gold["offsets"], fs, rs, agg, style,
+                                           disable_mlr=mlr)
+            scale_of = float(want.abs().max())
+            assert float((got - want).abs().max()) <= 2e-6 * scale_of, (case, agg, tag)
+            rotated = osc.raw_scores(k_rot.float().repeat_interleave(hq // hkv, dim=0), qc, gold["q_abs_mean"],
+                                     gold["inv_freq"], gold["offsets"], fs, rs, agg, style, disable_mlr=mlr) / scale
+            # (fp32 phases of up to 65536 rad carry errors of 4e-3 rad, different ones in the two forms)
+            assert float((rotated - want).abs().max()) <= 5e-4 * scale_of, (case, agg, tag)

@@ -19,6 +19,47 @@ import torch
 from . import ops
 
 
+def score_keys_for_round(key_states: torch.Tensor, q_mean_complex: torch.Tensor, q_abs_mean: torch.Tensor,
+                         inv_freq: torch.Tensor, offsets: torch.Tensor, freq_scale_sq: torch.Tensor, round_start: int,
+                         aggregation: str = "mean", rope_style: str = "half", attention_scale: float = 1.0,
+                         disable_mlr: bool = False, disable_trig: bool = False) -> torch.Tensor:
+    """Raw scores ``[Hq, T]`` (fp32, on the device) of the cached keys of one layer for the round that
+    starts at ``round_start``: what the research path computes per sampled head by un-rotating the
+    keys, forming amplitude / phase / extra against the head's query statistics and summing
+    ``amp * cos((round_start - p + offset) * omega + phi) + extra`` over the frequency pairs
+    (triattention/methods/pruning_utils.py:51-82, 245-309, called from methods/triattention.py:627-660).
+
+    ``key_states``: the cache's POST-RoPE keys ``[1, Hkv, T, D]`` in bf16 / fp16, as they lie.  A rotated
+    key carries its position in its phase, ``k_rot = scale * k * exp(i p omega)``, so
+    ``q conj(k_rot) exp(i (round_start + offset) omega)`` is the reference's term at ``round_start - p + offset``
+    times ``scale``: nothing is un-rotated and no position table is needed (positions that have gaps after
+    earlier pruning included); the result is divided by ``attention_scale``.  ``q_mean_complex``
+    ``[Hq, F, 2]`` (or complex ``[Hq, F]``) and ``q_abs_mean`` ``[Hq, F]`` are the statistics of the layer's
+    query heads; one read of a KV head's keys serves its whole group of query heads."""
+    if key_states.ndim != 4 or key_states.shape[0] != 1:
+        raise ValueError(f"expected [1, Hkv, T, D] key states, got {tuple(key_states.shape)}")
+    if attention_scale == 0:
+        raise ValueError("attention scaling factor must be non-zero")
+    dev = key_states.device
+    if q_mean_complex.is_complex():
+        q_mean_complex = torch.view_as_real(q_mean_complex)
+    qc = q_mean_complex.to(device=dev, dtype=torch.float32)
+    qa = q_abs_mean.to(device=dev, dtype=torch.float32)
+    fs = freq_scale_sq.to(device=dev, dtype=torch.float32)
+    if fs.ndim == 1:
+        fs = fs.unsqueeze(0).expand(qa.shape[0], -1)
+    total = int(key_states.shape[2])
+    kv = ops.PagedKV([key_states.permute(0, 2, 1, 3)], None, rope_style)                   # [1, T, Hkv, D] view, no copy
+    batch = ops.StepBatch(dev, [total], round_start=[int(round_start)])
+    folded = ops.fold_stats(qc.unsqueeze(0), qa.unsqueeze(0), fs.contiguous().unsqueeze(0),
+                            disable_mlr=disable_mlr, disable_trig=disable_trig)
+    sc = ops.ScoreConfig(folded, inv_freq.to(device=dev, dtype=torch.float32).contiguous(),
+                         offsets.to(device=dev, dtype=torch.float32).contiguous(), aggregation)
+    raw, _ = ops.score_paged(kv, batch, sc, head_major=True)                               # [1, 1, Hq, T]
+    scores = raw[0, 0]
+    return scores if attention_scale == 1.0 else scores / float(attention_scale)
+
+
 def select_keep_indices_per_head(key_states_by_layer: Sequence[torch.Tensor], *, decode_start: int, keep_count: int,
                                  folded_stats: torch.Tensor, inv_freq: torch.Tensor, offsets: torch.Tensor,
                                  round_start: int, normalize: bool = True, rope_style: str = "half",
