@@ -257,8 +257,7 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
 int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
                     hipStream_t s) {
-  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident &&
-                     sel->normalize != 2;
+  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident;
   if (!fused) {
     // The status word belongs to the resident kernel; on this path it just reads "fine".
     const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
@@ -513,8 +512,7 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident &&
-          sel->normalize != 2)
+  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident)
              ? w.fused.eligible : 0;
 }
 

@@ -188,6 +188,18 @@ __global__ void fused_clear_kernel(unsigned long long* xchg, int64_t words, uint
   if (i == 0) *status = 0u;
 }
 
+// The research path's normalisation (methods/triattention.py:255-258; tri_select_params.normalize = 2):
+// population standard deviation clamped from below at 1e-6, from the double-precision sums, as the
+// two-pass path's finalize_stats_kernel evaluates it.  `mine` / `other`: this lane's total and its
+// neighbour's; `odd`: this lane holds the sum of squares.
+__device__ __forceinline__ void population_mean_std(double mine, double other, bool odd, int T, float& mean, float& sd) {
+  const double sum = odd ? other : mine, sumsq = odd ? mine : other;
+  const double m = sum / (double)T;
+  const double v = sumsq / (double)T - m * m;
+  mean = (float)m;
+  sd = fmaxf((float)sqrt(v > 0.0 ? v : 0.0), 1e-6f);
+}
+
 // Mean and safe standard deviation, over all tokens of sequence b, of layer l's raw scores
 // for `items / 2` consecutive score heads starting at head ah0: waits (bounded) until every
 // tile of the sequence has published its tagged sums, adds them in tile order in double,
@@ -230,17 +242,22 @@ __device__ __forceinline__ void gather_layer_stats(const FusedArgs& a, int b, in
         if (t0 + u < seq_tiles) acc += (double)__uint_as_float((uint32_t)w[u]);
     }
     // Lanes 2i / 2i+1 hold the sum and the sum of squares of head ah0 + base/2 + i.
-    const float mine = (float)acc;
-    const float other = __shfl_xor(mine, 1);
-    const float sum = (lane & 1) ? other : mine;
-    const float sumsq = (lane & 1) ? mine : other;
-    const float cnt = (float)T;
-    const float mean = __fdiv_rn(sum, cnt);
-    float var = 0.f;
-    if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(mean, mean))), (float)(T - 1));
-    var = fmaxf(var, 0.f);
-    float sd = __fsqrt_rn(var);
-    if (sd < 1e-8f) sd = 1.f;
+    float mean, sd;
+    if (a.normalize == 2) {
+      population_mean_std(acc, __shfl_xor(acc, 1), (lane & 1) != 0, T, mean, sd);
+    } else {
+      const float mine = (float)acc;
+      const float other = __shfl_xor(mine, 1);
+      const float sum = (lane & 1) ? other : mine;
+      const float sumsq = (lane & 1) ? mine : other;
+      const float cnt = (float)T;
+      mean = __fdiv_rn(sum, cnt);
+      float var = 0.f;
+      if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(mean, mean))), (float)(T - 1));
+      var = fmaxf(var, 0.f);
+      sd = __fsqrt_rn(var);
+      if (sd < 1e-8f) sd = 1.f;
+    }
     if (live) st[item] = (lane & 1) ? sd : mean;
   }
 }
@@ -303,13 +320,18 @@ __device__ __forceinline__ void gather_head_stats(const FusedArgs& a, int b, int
   const float cnt = (float)T;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float sum = __shfl(mine, 2 * i), sumsq = __shfl(mine, 2 * i + 1);
-    const float m = __fdiv_rn(sum, cnt);
-    float var = 0.f;
-    if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(m, m))), (float)(T - 1));
-    var = fmaxf(var, 0.f);
-    float s = __fsqrt_rn(var);
-    if (s < 1e-8f) s = 1.f;
+    float m, s;
+    if (a.normalize == 2) {
+      population_mean_std(__shfl(total, 2 * i), __shfl(total, 2 * i + 1), false, T, m, s);
+    } else {
+      const float sum = __shfl(mine, 2 * i), sumsq = __shfl(mine, 2 * i + 1);
+      m = __fdiv_rn(sum, cnt);
+      float var = 0.f;
+      if (T > 1) var = __fdiv_rn(__fsub_rn(sumsq, __fmul_rn(cnt, __fmul_rn(m, m))), (float)(T - 1));
+      var = fmaxf(var, 0.f);
+      s = __fsqrt_rn(var);
+      if (s < 1e-8f) s = 1.f;
+    }
     if (i < heads) { mean[i] = m; sd[i] = s; }
   }
 }
