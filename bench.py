@@ -76,6 +76,8 @@ def parse_args():
     ap.add_argument("--hook-latency", action="store_true",
                     help="also time the runner hook for one request and the batch hook for a batch of requests of "
                          "budget + 128 tokens, host side included")
+    ap.add_argument("--flat-pool", action="store_true",
+                    help="also time one request on a token-level pool (the SGLang backend's cache) through flat_pool")
     ap.add_argument("--query-stats", action="store_true",
                     help="also time the calibration statistics kernel on one layer's captured queries "
                          "(32 heads x 32768 tokens x 128, bf16)")
@@ -254,6 +256,59 @@ def query_stats_leg(dev, heads: int = 32, tokens: int = 32768, dim: int = 128, c
     med = times[len(times) // 2]
     return {"heads": heads, "tokens": tokens, "head_dim": dim, "dtype": "bf16", "ms_median": med,
             "query_bytes": nbytes, "gbs": nbytes / (med * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
+def flat_pool_leg(dev, layers: int = 36, heads: int = 8, q_heads: int = 32, dim: int = 128, tokens: int = 16384,
+                  budget: int = 2048, calls: int = 10):
+    """One request on a token-level pool (the SGLang backend's cache: per-layer [slots, H, D] buffers, a
+    req_to_token table with one slot per token): selection in the backend's order of operations, then
+    per-head compaction, through ``triattention_amd.flat_pool``.  One token per block, so the scorer is
+    the two-pass vector-unit kernel.  Bytes as for the paged step: every key row once, kept rows of K
+    and V read and written."""
+    from triattention_amd import flat_pool, ops
+    g = torch.Generator(device=dev).manual_seed(77)
+    slots = tokens + 64
+    k_buffers = [torch.randn(slots, heads, dim, generator=g, device=dev).to(torch.bfloat16) for _ in range(layers)]
+    v_buffers = [torch.randn(slots, heads, dim, generator=g, device=dev).to(torch.bfloat16) for _ in range(layers)]
+    perm = (torch.randperm(slots - 1, generator=g, device=dev) + 1)[:tokens].to(torch.int32)       # slot 0 is the dummy slot
+    req_to_token = torch.zeros(2, tokens + 8, dtype=torch.int32, device=dev)
+    req_to_token[1, :tokens] = perm
+    f = dim // 2
+    qc = torch.randn(layers, q_heads, f, 2, generator=g, device=dev)
+    qa = qc.pow(2).sum(-1).sqrt() + torch.randn(layers, q_heads, f, generator=g, device=dev).abs()
+    folded = ops.fold_stats(qc, qa, torch.ones(layers, q_heads, f, device=dev))
+    inv = 1e6 ** (-torch.arange(0, dim, 2, device=dev, dtype=torch.float32) / dim)
+    offsets = torch.tensor([float(2 ** j) for j in range(17)], device=dev)
+    score = ops.ScoreConfig(folded, inv, offsets)
+    saved_k = [b[perm[:budget].long()].clone() for b in k_buffers]
+    saved_v = [b[perm[:budget].long()].clone() for b in v_buffers]
+    sel_ms, cmp_ms = [], []
+    for i in range(calls + 2):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        ev[0].record()
+        keep = flat_pool.select_keep_indices_per_head(k_buffers, req_to_token, 1, tokens, score, budget=budget,
+                                                      round_start=tokens)
+        ev[1].record()
+        flat_pool.compact_request_kv_in_place_per_head(k_buffers, v_buffers, req_to_token, 1, keep, tokens)
+        ev[2].record()
+        torch.cuda.synchronize()
+        for b, sk, sv, vb in zip(k_buffers, saved_k, saved_v, v_buffers):              # put the overwritten prefix back
+            b[perm[:budget].long()] = sk
+            vb[perm[:budget].long()] = sv
+        if i >= 2:
+            sel_ms.append(ev[0].elapsed_time(ev[1]))
+            cmp_ms.append(ev[1].elapsed_time(ev[2]))
+    sel_ms.sort()
+    cmp_ms.sort()
+    row = heads * dim * 2
+    score_bytes = layers * tokens * row
+    compact_bytes = layers * budget * row * 4
+    sm, cm = sel_ms[len(sel_ms) // 2], cmp_ms[len(cmp_ms) // 2]
+    total = (score_bytes + compact_bytes) / ((sm + cm) * 1e-3) / 1e9
+    return {"layers": layers, "kv_heads": heads, "q_heads": q_heads, "head_dim": dim, "tokens": tokens, "budget": budget,
+            "calls": calls, "select_ms_median": sm, "compact_ms_median": cm, "host_included": True,
+            "algorithmic_bytes": {"score": score_bytes, "compact": compact_bytes},
+            "achieved_gbs": total, "frac_of_hbm_peak": total / HBM_PEAK_GBS}
 
 
 def pool_bytes_per_block(w) -> int:
@@ -708,6 +763,8 @@ def main() -> int:
         del src, dst
     if args.query_stats:
         out["query_stats"] = query_stats_leg(dev)
+    if args.flat_pool:
+        out["flat_pool"] = flat_pool_leg(dev)
     if args.hook_latency and w.kv_dtype != "fp8":
         out["hook_call"] = hook_latency(w, dev)
         out["hook_batch_call"] = hook_latency(w, dev, calls=20, requests=len(w.seq_lens))

@@ -249,6 +249,8 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
   a.raw = raw; a.raw_stride_layer = rs_layer; a.raw_stride_token = rs_token; a.raw_stride_head = rs_head;
   a.fin = fin ? fin : at<float>(ws, w.fin);
   a.keep = keep;
+  a.group_scratch = at<double>(ws, w.coef);
+  a.group_scratch_bytes = w.trig - w.coef;
   return launch_status(tri::launch_select(a, s), "select");
 }
 

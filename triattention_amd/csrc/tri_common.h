@@ -130,6 +130,10 @@ struct SelectLaunch {
   int64_t raw_stride_layer, raw_stride_token, raw_stride_head;
   float* fin;          // [rows][Tmax]
   int32_t* keep;       // [rows][max_budget]
+  // Scratch for the chunk sums of the reduce-first statistics (group_first): any part of the workspace
+  // that no later launch of the call reads (the scorer's coefficient tables: every score call rebuilds them).
+  double* group_scratch;
+  int64_t group_scratch_bytes;
 };
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s);
 hipError_t launch_clear_status(uint32_t* status, hipStream_t s);

@@ -104,6 +104,72 @@ __global__ __launch_bounds__(256) void group_stats_kernel(const float* raw, int6
   }
 }
 
+// The same statistics for the usual layout -- four query heads per KV head, raw scores head-contiguous
+// ([token][head], 16-byte aligned), a power-of-two number of KV heads -- in two launches that read whole
+// token rows: a workgroup takes a chunk of 2048 tokens of one (sequence, layer) with thread = (token,
+// KV head), so a wave reads 1 KB of consecutive memory per load where the kernel above reads 16 bytes
+// of every 128-byte row eight times over (one request of 16384 tokens x 36 layers: 117 -> 30 us), and
+// leaves the chunk's sums in double; the second launch adds the chunks in order.
+constexpr int kGroupStatsChunk = 2048;
+__global__ __launch_bounds__(256) void group_stats_partial_kernel(const float* raw, int64_t stride_layer,
+                                                                  int64_t stride_token, const int32_t* seq_lens, int L,
+                                                                  int Hkv, int chunks, int group_reduce,
+                                                                  double* partial) {
+  __shared__ double red[256][2];
+  const int c = blockIdx.x, bl = blockIdx.y, b = bl / L;
+  const int T = seq_lens[b];
+  const int h = threadIdx.x % Hkv, tn = threadIdx.x / Hkv, tstep = 256 / Hkv;
+  const int n_end = min(T, (c + 1) * kGroupStatsChunk);
+  const float* base = raw + (int64_t)bl * stride_layer + h * 4;
+  double s = 0.0, q = 0.0;
+  for (int n = c * kGroupStatsChunk + tn; n < n_end; n += tstep) {
+    const float4 x = *reinterpret_cast<const float4*>(base + (int64_t)n * stride_token);
+    float m;
+    if (group_reduce == TRI_REDUCE_MAX) m = fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w));
+    else m = __fdiv_rn(__fadd_rn(__fadd_rn(__fadd_rn(x.x, x.y), x.z), x.w), 4.f);
+    s += (double)m;
+    q += (double)m * (double)m;
+  }
+  red[threadIdx.x][0] = s;
+  red[threadIdx.x][1] = q;
+  __syncthreads();
+  for (int off = 128; off >= Hkv; off >>= 1) {       // threads `off` apart hold the same KV head
+    if ((int)threadIdx.x < off) {
+      red[threadIdx.x][0] += red[threadIdx.x + off][0];
+      red[threadIdx.x][1] += red[threadIdx.x + off][1];
+    }
+    __syncthreads();
+  }
+  if ((int)threadIdx.x < Hkv) {
+    double* out = partial + (((int64_t)bl * chunks + c) * Hkv + threadIdx.x) * 2;
+    out[0] = red[threadIdx.x][0];
+    out[1] = red[threadIdx.x][1];
+  }
+}
+
+__global__ void group_stats_finish_kernel(const double* partial, const int32_t* seq_lens, int BL, int L, int Hkv, int A,
+                                          int chunks, float* mustd) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= BL * Hkv) return;
+  const int h = idx % Hkv, bl = idx / Hkv, b = bl / L;
+  const int T = seq_lens[b];
+  const int nc = ceil_div(T, kGroupStatsChunk);
+  double s = 0.0, q = 0.0;
+  for (int c = 0; c < nc; ++c) {
+    const double* p = partial + (((int64_t)bl * chunks + c) * Hkv + h) * 2;
+    s += p[0];
+    q += p[1];
+  }
+  const double mean = s / (double)T;
+  double var = T > 1 ? (q - (double)T * mean * mean) / (double)(T - 1) : 0.0;
+  if (var < 0.0) var = 0.0;
+  float sd = (float)sqrt(var);
+  if (sd < 1e-8f) sd = 1.f;
+  float* out = mustd + ((int64_t)bl * A + h) * 2;
+  out[0] = (float)mean;
+  out[1] = sd;
+}
+
 struct CombineArgs {
   const float* raw;
   const float* mustd;
@@ -150,11 +216,18 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
       // Default shape: one KV head per thread, four query heads in one 16-byte load;
       // four layers in flight per thread.
       const float* raw0 = a.raw + (int64_t)b * a.L * a.raw_stride_layer + (int64_t)n * a.raw_stride_token + r * 4;
-      const float* ms0 = a.mustd + ((int64_t)b * a.L * a.A + r * 4) * 2;
+      // Reduce-first order (group_first): the statistics are those of the KV head's reduced score and
+      // sit in entry r of the layer's table; they arrive in m01.x / m01.y (m23 unused).
+      const float* ms0 = a.mustd + ((int64_t)b * a.L * a.A + (a.group_first ? r : r * 4)) * 2;
       auto layer_value = [&](const float4& x, const float4& m01, const float4& m23) {
         // mustd is [head][mean, std]: m01 = (mean0, std0, mean1, std1), m23 likewise.
         float v;
-        if (a.group_reduce == TRI_REDUCE_MAX) {
+        if (a.group_first) {
+          const float m = (a.group_reduce == TRI_REDUCE_MAX)
+                              ? fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))
+                              : __fdiv_rn(__fadd_rn(__fadd_rn(__fadd_rn(x.x, x.y), x.z), x.w), 4.f);
+          v = zscore(m, m01.x, m01.y);
+        } else if (a.group_reduce == TRI_REDUCE_MAX) {
           v = fmaxf(fmaxf(zscore(x.x, m01.x, m01.y), zscore(x.y, m01.z, m01.w)),
                     fmaxf(zscore(x.z, m23.x, m23.y), zscore(x.w, m23.z, m23.w)));
         } else {
@@ -171,8 +244,14 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
         for (int u = 0; u < 4; ++u) {
           x[u] = *reinterpret_cast<const float4*>(raw0 + (int64_t)(l + u) * a.raw_stride_layer);
           const float* ms = ms0 + (int64_t)(l + u) * a.A * 2;
-          m01[u] = *reinterpret_cast<const float4*>(ms);
-          m23[u] = *reinterpret_cast<const float4*>(ms + 4);
+          if (a.group_first) {
+            const float2 m = *reinterpret_cast<const float2*>(ms);
+            m01[u] = float4{m.x, m.y, 0.f, 0.f};
+            m23[u] = m01[u];
+          } else {
+            m01[u] = *reinterpret_cast<const float4*>(ms);
+            m23[u] = *reinterpret_cast<const float4*>(ms + 4);
+          }
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -184,7 +263,16 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
       for (; l < l_end; ++l) {
         const float4 x = *reinterpret_cast<const float4*>(raw0 + (int64_t)l * a.raw_stride_layer);
         const float* ms = ms0 + (int64_t)l * a.A * 2;
-        const float v = layer_value(x, *reinterpret_cast<const float4*>(ms), *reinterpret_cast<const float4*>(ms + 4));
+        float4 m01, m23;
+        if (a.group_first) {
+          const float2 m = *reinterpret_cast<const float2*>(ms);
+          m01 = float4{m.x, m.y, 0.f, 0.f};
+          m23 = m01;
+        } else {
+          m01 = *reinterpret_cast<const float4*>(ms);
+          m23 = *reinterpret_cast<const float4*>(ms + 4);
+        }
+        const float v = layer_value(x, m01, m23);
         if (l == l_begin) acc = v;
         else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
       }
@@ -550,7 +638,21 @@ hipError_t launch_clear_status(uint32_t* status, hipStream_t s) {
 
 hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const int n = a.B * a.L * a.A;
-  if (a.group_first)
+  // Whole token rows for the usual layout; the chunk sums ([B][L][chunks of 2048][Hkv][2] doubles) go
+  // into scratch the caller names.
+  const int chunks = ceil_div(a.Tmax, kGroupStatsChunk);
+  const bool rows = a.group_first && a.normalize && a.G == 4 && a.A == a.Hkv * 4 && a.raw_stride_head == 1 &&
+                    a.raw_stride_token % 4 == 0 && a.raw_stride_layer % 4 == 0 &&
+                    (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 && a.Hkv <= 128 && (a.Hkv & (a.Hkv - 1)) == 0 &&
+                    a.group_scratch != nullptr &&
+                    (int64_t)a.B * a.L * chunks * a.Hkv * 16 <= a.group_scratch_bytes;
+  if (rows) {
+    double* part = a.group_scratch;
+    hipLaunchKernelGGL(group_stats_partial_kernel, dim3(chunks, a.B * a.L), dim3(256), 0, s, a.raw, a.raw_stride_layer,
+                       a.raw_stride_token, a.seq_lens, a.L, a.Hkv, chunks, a.group_reduce, part);
+    hipLaunchKernelGGL(group_stats_finish_kernel, dim3(ceil_div(a.B * a.L * a.Hkv, 256)), dim3(256), 0, s, part,
+                       a.seq_lens, a.B * a.L, a.L, a.Hkv, a.A, chunks, a.mustd);
+  } else if (a.group_first)
     hipLaunchKernelGGL(group_stats_kernel, dim3(a.B * a.L * a.Hkv), dim3(256), 0, s, a.raw, a.raw_stride_layer,
                        a.raw_stride_token, a.raw_stride_head, a.seq_lens, a.L, a.Hkv, a.A, a.G, a.group_reduce,
                        a.normalize, a.mustd);
@@ -581,7 +683,7 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const bool per_layer = a.layer_reduce < 0;
   dim3 grid(ceil_div(a.Tmax, c.tokens_per_wg), per_layer ? a.L : 1, a.B);
   const size_t smem = (size_t)c.rows_per_seq * c.tokens_per_wg * sizeof(float);
-  const bool vec4 = !a.group_first && a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
+  const bool vec4 = a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
                     a.raw_stride_layer % 4 == 0 && (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(a.mustd) % 16) == 0;
   if (vec4)
