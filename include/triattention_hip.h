@@ -138,7 +138,8 @@ typedef enum tri_tuning {
   TRI_TUNE_RESIDENT_WORKGROUPS = 1, /* 0 (default): the device's own capacity; n > 0: plan as if the device held
                                        n resident workgroups (never more than it does): small inputs then need
                                        several launches (tests) */
-  TRI_TUNE_LAYER_SPLIT = 2,         /* -1 (default): small batches are cut by layers unless the kernel was forced
+  TRI_TUNE_LAYER_SPLIT = 2,         /* -1 (default): single-launch batches are cut by layers where that shortens the
+                                       longest workgroup, unless the kernel was forced
                                        with TRI_TUNE_RESIDENT_KERNEL = 1; 0: never; 1: always allowed */
   TRI_TUNE_MAX_KERNEL = 3,          /* 0 (default): max aggregation on the matrix cores where a kernel exists;
                                        1: always the vector-unit kernel (comparison runs) */

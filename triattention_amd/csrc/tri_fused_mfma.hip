@@ -1053,29 +1053,37 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   // workgroups: 0.40 ms against 0.48 ms on the two-pass kernels.)
   const int64_t need = waves == 4 ? 45 : 60;
   int layer_groups = 1, layers_per_group = L;
-  if (split_layers && L > 1 && (int64_t)B * tiles * HC <= resident &&
-      (int64_t)B * tiles * HC * 100 < (int64_t)resident * need) {
-    // A few requests (the reference's runner compresses one at a time,
-    // runtime/runner_compression_actions.py:24): whole-model workgroups would use a fraction of
-    // the chip, e.g. 17 of 256 CUs for one request of 2176 tokens.  The layers are independent
-    // until the reduction over them, so they are cut into groups and a workgroup runs one
-    // (sequence, group, tile); fewest layers per group first, with tiles as long as the chip then
-    // has room for (a workgroup pays its per-layer exchange once per layer, so one layer of a
-    // long tile beats several layers of a short one): one request of 2176 tokens x 36 layers
-    // becomes 36 groups x 7 tiles of 320 tokens = 252 workgroups.
+  if (split_layers && L > 1 && (int64_t)B * tiles * HC <= resident) {
+    // A batch that is one launch: the layers are independent until the reduction over them, so
+    // they can be cut into groups, a workgroup running one (sequence, group, tile).  A launch takes
+    // as long as its longest workgroup: layers x (tile tokens + the fixed work of a layer, worth
+    // ~32 tokens: the exchange of the statistics, the coefficient loads).  Whole-model workgroups
+    // of a few requests (the reference's runner compresses one at a time,
+    // runtime/runner_compression_actions.py:24) would use a fraction of the chip, 17 of 256 CUs
+    // for one request of 2176 tokens x 36 layers: that becomes 36 groups x 7 tiles of 320 tokens
+    // = 252 workgroups.  Mid-size batches gain as well: 16 requests of 2176 tokens are 16 x 12
+    // tiles of 192 tokens x 36 layers (75 % of the CUs) or, with four groups of nine layers,
+    // 16 x 4 x 4 tiles of 576 tokens on every CU, a quarter less per workgroup.  A cut must
+    // win 5 % to be taken: the groups' partial sums cost a pass of their own, and a launch that
+    // fills the chip already is bound by HBM as much as by its longest workgroup (16 x 8192 tokens
+    // as two groups of 1024-token tiles: 1 % slower than whole-model tiles of 512).
     const int granule = (kv_dtype == TRI_KV_FP8_E4M3 || (D == 64 && G <= 4)) ? 128 : 64;
     const int tw_max = tws[ntw - 1];                       // the longest tile any instance of this shape holds
     const bool one_instance = !(waves == kFusedWaves && D == 128);
-    for (int lpg = 1; lpg < L; ++lpg) {
+    constexpr int kLayerFixed = 32;
+    int64_t best = (int64_t)L * (tile + kLayerFixed) * 95 / 100;
+    for (int lpg = L - 1; lpg >= 1; --lpg) {
       const int groups = ceil_div(L, lpg);
       const int64_t units = (int64_t)B * groups * HC;
-      if (units > resident) continue;
+      if (units > resident) break;                         // fewer layers per group: more groups still
       const int tiles_max = (int)min((int64_t)64, resident / units);
       int t = ceil_div(ceil_div(Tmax, tiles_max), granule) * granule;
       t = min(tw_max, max(128, t));
       const int nt = ceil_div(Tmax, t);
       if (units * nt > resident) continue;
-      if (units * nt <= (int64_t)B * tiles * HC) break;      // no better than whole-model workgroups
+      const int64_t cost = (int64_t)lpg * (t + kLayerFixed) + groups;
+      if (cost >= best) continue;
+      best = cost;
       layer_groups = groups;
       layers_per_group = lpg;
       tile = t;
@@ -1083,7 +1091,6 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
       if (!one_instance)
         for (int i = 0; i < ntw; ++i)
           if (tws[i] >= t) { tw = tws[i]; break; }           // the instance with the smallest ring that holds the tile
-      break;
     }
   }
   if (!any_fill && (int64_t)B * layer_groups * tiles * HC * 100 < (int64_t)resident * need) return p;
