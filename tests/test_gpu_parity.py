@@ -930,22 +930,30 @@ def test_resident_selection_on_dense_keys(kernel, monkeypatch):
                             ft, 128, tie_tol=2e-3 * scale)
 
 
-def test_resident_path_is_taken_only_by_launches_that_fill_the_chip():
+def test_resident_path_is_taken_unless_multi_layer_workgroups_would_underfill_the_chip():
+    """Workgroups that run one layer make a short launch however few they are; workgroups that run
+    several layers must fill most of the chip, or the two-pass kernels take the batch."""
     sel = ops.SelectConfig(window_size=12)
-    cases = (((300,), "two_pass"), ((3072,) * 16, "resident_mfma"), ((2176,) * 16, "resident_mfma"),
-             ((16384,), "two_pass"),           # one sequence: at most 64 tiles, a quarter of the chip
-             ((2176,) * 4, "two_pass"),        # 4 x 17 tiles of 128
-             ((8192,) * 4, "resident_mfma"))   # 4 x 64 tiles of 128
-    for seq_lens, want in cases:
-        w = small(seq_lens=seq_lens, num_layers=1, num_q_heads=32, num_kv_heads=8)
+    cases = ((1, None, (300,), "resident_mfma"),             # 3 tiles of 128, one layer
+             (1, None, (16384,), "resident_mfma"),           # 64 tiles, a quarter of the chip, one layer
+             (1, None, (2176,) * 4, "resident_mfma"),
+             (4, None, (300,), "resident_mfma"),             # cut into 4 layer groups x 3 tiles
+             (4, 0, (300,), "two_pass"),                     # layer groups switched off: 3 workgroups x 4 layers
+             (4, 0, (2176,) * 4, "two_pass"),                # 4 x 17 tiles of 128 x 4 layers
+             (4, 0, (8192,) * 4, "resident_mfma"),           # 4 x 64 tiles of 128: the chip is full
+             (4, None, (128,) * 130, "two_pass"),            # 130 workgroups, two layer groups would not fit
+             (1, None, (3072,) * 16, "resident_mfma"), (1, None, (2176,) * 16, "resident_mfma"))
+    for layers, split, seq_lens, want in cases:
+        tune(layer_split=-1 if split is None else split)
+        w = small(seq_lens=seq_lens, num_layers=layers, num_q_heads=32, num_kv_heads=8)
         tables = synth.make_block_tables(w)
         cache = torch.zeros(2, w.pool_blocks, w.block_size, w.num_kv_heads, w.head_dim, dtype=torch.bfloat16, device=DEV)
-        kv = ops.PagedKV.from_kv_caches([cache])
+        kv = ops.PagedKV.from_kv_caches([cache] * layers)
         batch = ops.StepBatch(DEV, w.seq_lens, round_start=w.seq_lens, budgets=w.budget, block_tables=tables)
         qc, qa = synth.make_stats(w, DEV)
         sc = ops.ScoreConfig(ops.fold_stats(qc, qa, torch.ones_like(qa)), synth.rope_inv_freq(w, DEV),
                              synth.geometric_offsets(device=DEV))
-        assert ops.select_path(kv, batch, sc, sel) == want, seq_lens
+        assert ops.select_path(kv, batch, sc, sel) == want, (layers, split, seq_lens)
 
 
 def _resident_batch(seed_index):

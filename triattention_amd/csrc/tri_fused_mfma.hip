@@ -1093,7 +1093,13 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
           if (tws[i] >= t) { tw = tws[i]; break; }           // the instance with the smallest ring that holds the tile
     }
   }
-  if (!any_fill && (int64_t)B * layer_groups * tiles * HC * 100 < (int64_t)resident * need) return p;
+  // The rule above is about workgroups that run layer after layer on a chip they do not fill.  With
+  // one layer per workgroup the launch is short however few workgroups it has, and the two-pass
+  // kernels pay five launches before their first byte: one layer of 1 x 4096 tokens as 32 tiles of
+  // 128 takes 0.049 ms (score + select) against 0.079 ms.
+  if (!any_fill && layers_per_group > 1 &&
+      (int64_t)B * layer_groups * tiles * HC * 100 < (int64_t)resident * need)
+    return p;
   p.eligible = 2;
   p.tw = tw;
   p.HC = HC;
