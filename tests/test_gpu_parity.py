@@ -793,6 +793,8 @@ def test_resident_selection_matches_two_pass(name, kernel, monkeypatch):
     tune(resident_kernel=kernel)      # take that kernel however small the launch
     if "workgroups" in case:
         tune(resident_workgroups=case["workgroups"])
+    if "layer_split" in case:
+        tune(layer_split=case["layer_split"])
     inp = build_inputs(w, case.get("kv_axis", 0))
     print(f"case={name} kernel={kernel} workload={w}", flush=True)
     caches, kv, batch, sc = device_objects(w, inp, DEV, prefill_lens=case.get("prefill_lens"))
@@ -843,8 +845,13 @@ def _random_resident_case(seed: int):
     nseq = r.choice([1, 2, 3, 5, 9])
     seq_lens = tuple(r.choice([1, 15, 16, 17, 63, 64, 65, 127, 129, 300, 511, 513, 1023, 1025, 2049, 3000])
                      for _ in range(nseq))
+    layers = r.choice([1, 2, 3])
+    r2 = random.Random(10_000 + seed)           # (drawn apart, so that the other fields of a seed stay what they were)
+    split = r2.random() < 0.5                   # let the planner cut the layers into groups of workgroups
+    if split:
+        layers = r2.choice([2, 3, 4, 5, 6, 7])
     w = small(kv_dtype=kv_dtype, head_dim=head_dim, num_q_heads=hkv * g, num_kv_heads=hkv, seq_lens=seq_lens,
-              num_layers=r.choice([1, 2, 3]), budget=r.choice([1, 16, 96, 200]), block_size=r.choice([16, 16, 32, 128]),
+              num_layers=layers, budget=r.choice([1, 16, 96, 200]), block_size=r.choice([16, 16, 32, 128]),
               window_size=r.choice([0, 1, 12, 200]), rope_style=r.choice(["half", "interleaved"]), index=100 + seed)
     case = dict(w=w, sel=dict(normalize=r.random() < 0.8, group_reduce=r.choice(["max", "max", "mean"]),
                               layer_reduce=r.choice(["mean", "mean", "max"])))
@@ -853,6 +860,8 @@ def _random_resident_case(seed: int):
         case["prefill_lens"] = [r.randrange(0, t + 1) for t in seq_lens]
     if r.random() < 0.4:
         case["workgroups"] = r.choice([16, 24, 40])      # enough for the longest sequence at its smallest tile
+    if split:
+        case["layer_split"] = 1
     return case
 
 
