@@ -446,6 +446,43 @@ def test_layer_selection_matches_reference_golden(tag, kw, fixture):
     assert torch.equal(got, gold[f"layer1_{tag}_keep"])
 
 
+@pytest.mark.parametrize("fixture", ["selector_group.pt", "selector_group_d128.pt"])
+@pytest.mark.parametrize("tag,kw", [("default", dict()), ("nonorm", dict(normalize=False))])
+def test_one_layer_of_a_per_layer_selection_takes_the_resident_kernel(tag, kw, fixture):
+    """The reference's per-layer modes call the selector once per layer (runtime/selector_hf.py:473-747
+    from the layer loop): a keep set per layer of a one-layer call is the group selection of that layer,
+    so the call takes the resident kernel and still gives the reference's rows for layer 1."""
+    gold = load_golden(fixture)
+    layers, hkv, t, d = gold["keys"].shape
+    hq = gold["q_mean_complex"].shape[1]
+    bs, pool = int(gold["block_size"]), int(gold["pool_blocks"])
+    ids = gold["block_ids"].tolist()
+    kvc = torch.zeros(2, pool, bs, hkv, d, dtype=torch.bfloat16)
+    tok = torch.arange(t)
+    blk = torch.tensor(ids)[tok // bs]
+    kvc[0, blk, tok % bs] = gold["keys"][1].transpose(0, 1)
+    kv = ops.PagedKV.from_kv_caches([kvc.to(DEV)])
+    batch = ops.StepBatch(DEV, [t], round_start=[int(gold["round_start"])], budgets=int(gold["budget"]),
+                          block_tables=[ids], prefill_lens=[int(gold["prefill_len"])])
+    folded = ops.fold_stats(gold["q_mean_complex"][1:2].to(DEV), gold["q_abs_mean"][1:2].to(DEV),
+                            torch.ones(1, hq, d // 2, device=DEV))
+    sc = ops.ScoreConfig(folded, gold["omega"].to(DEV), synth.geometric_offsets(device=DEV))
+    sel = ops.SelectConfig(normalize=kw.get("normalize", True), window_size=int(gold["window"]), layer_reduce=None)
+    assert ops.select_path(kv, batch, sc, sel) == "resident_mfma"
+    keep, fin, ws = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    sel.allow_resident = False
+    assert ops.select_path(kv, batch, sc, sel) == "two_pass"
+    keep_t, fin_t, _ = ops.select_paged(kv, batch, sc, sel, want_scores=True)
+    torch.cuda.synchronize()
+    assert ws.status() == 0
+    assert torch.equal(keep.cpu().long().view(hkv, -1), gold[f"layer1_{tag}_keep"])
+    assert torch.equal(keep_t.cpu().long().view(hkv, -1), gold[f"layer1_{tag}_keep"])
+    a, b = fin.cpu().view(hkv, -1)[:, :t], fin_t.cpu().view(hkv, -1)[:, :t]
+    m = torch.isfinite(b)
+    assert torch.equal(torch.isfinite(a), m)
+    assert float((a[m] - b[m]).abs().max()) <= 1e-4 * float(b[m].abs().max())
+
+
 @pytest.mark.parametrize("width", [3000, 8192, 16384, 20001, 32768, 40000])
 def test_topk_rows_by_width(width):
     """Rows up to 8192 / 16384 / 32768 elements are selected from registers (three kernel

@@ -254,12 +254,23 @@ int do_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_p
   return launch_status(tri::launch_select(a, s), "select");
 }
 
+// A keep set per layer (layer_reduce -1) of a single layer is the mean over that one layer: same
+// rows, same scores (x / 1).  The reference's per-layer modes call their selector once per layer
+// (runtime/selector_hf.py:473-747 from the layer loop), so those calls may take a resident kernel.
+int layer_reduce_of(const tri_kv_layout* kv, const tri_select_params* sel) {
+  return (sel->layer_reduce < 0 && kv->num_layers == 1) ? TRI_REDUCE_MEAN : sel->layer_reduce;
+}
+
+bool takes_resident(const tri::Workspace& w, const tri_kv_layout* kv, const tri_select_params* sel) {
+  return w.fused.eligible && layer_reduce_of(kv, sel) >= 0 && !sel->shared && !sel->group_first && !sel->no_resident;
+}
+
 // Selection straight from the paged keys: the resident kernel when the shape has one,
 // else score into the workspace and select from there.
 int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel, float* fin, int32_t* keep, void* ws, const tri::Workspace& w,
                     hipStream_t s) {
-  const bool fused = w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident;
+  const bool fused = takes_resident(w, kv, sel);
   if (!fused) {
     // The status word belongs to the resident kernel; on this path it just reads "fine".
     const hipError_t ce = tri::launch_clear_status(at<uint32_t>(ws, w.status), s);
@@ -284,7 +295,7 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   a.block_size = kv->block_size; a.kv_dtype = kv->kv_dtype; a.rope_style = kv->rope_style;
   a.A = sp->num_score_heads; a.G = sp->num_score_heads / kv->num_kv_heads; a.Tmax = batch->max_seq_len;
   a.normalize = sel->normalize; a.window_size = sel->window_size; a.protect_prefill = sel->protect_prefill;
-  a.group_reduce = sel->group_reduce; a.layer_reduce = sel->layer_reduce;
+  a.group_reduce = sel->group_reduce; a.layer_reduce = layer_reduce_of(kv, sel);
   a.stride_block = kv->stride_block; a.stride_token = kv->stride_token; a.stride_head = kv->stride_head;
   a.k_layers = kv->k_layers; a.k_scale_layers = kv->k_scale_layers;
   a.block_table = batch->block_table; a.block_table_pitch = batch->block_table_pitch;
@@ -333,7 +344,7 @@ int do_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   if (a.skip_layer_reduce)
     return launch_status(tri::launch_topk_rows(a.fin_part, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, a.Tmax,
                                                keep, batch->max_budget, s, w.fused.layer_groups,
-                                               (int64_t)a.B * a.Hkv * a.Tmax, sel->layer_reduce == TRI_REDUCE_MAX),
+                                               (int64_t)a.B * a.Hkv * a.Tmax, a.layer_reduce == TRI_REDUCE_MAX),
                          "topk_rows");
   return launch_status(tri::launch_topk_rows(a.fin, a.Tmax, a.B * a.Hkv, a.seq_lens, batch->budgets, a.Hkv, a.Tmax, keep,
                                              batch->max_budget, s),
@@ -514,8 +525,7 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
                     const tri_select_params* sel) {
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
-  return (w.fused.eligible && sel->layer_reduce >= 0 && !sel->shared && !sel->group_first && !sel->no_resident)
-             ? w.fused.eligible : 0;
+  return takes_resident(w, kv, sel) ? w.fused.eligible : 0;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,

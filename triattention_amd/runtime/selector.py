@@ -195,7 +195,7 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
                                group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared,
                                allow_resident=holder.get("resident_ok", True))
         try:
-            resident = ops.select_path(kv, batch, sc, sel) != "two_pass"   # (a single request: only when forced)
+            resident = ops.select_path(kv, batch, sc, sel) != "two_pass"
             keep, _, ws = ops.select_paged(kv, batch, sc, sel)
             if resident and _resident_failed(ws.status()):
                 # The keep lists mean nothing.  Nothing has been moved yet; score again on the
