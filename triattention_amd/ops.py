@@ -153,7 +153,7 @@ class PagedKV:
                     raise ValueError("all layers must share shape, strides, dtype and device")
             hit = cls.from_kv_caches(kv_caches, rope_style, kv_axis)
             hit._keep = None
-            if len(cls._recent) >= 16:
+            if len(cls._recent) >= 256:         # (the per-layer modes come with one tensor at a time: 2 x layers keys)
                 cls._recent.pop(next(iter(cls._recent)))
             cls._recent[key] = hit
         return hit
@@ -233,6 +233,27 @@ class StepBatch:
             block_table_pitch=pitch, block_table=_ptr(self.block_table), seq_lens=_ptr(self.seq_lens),
             round_start=_ptr(self.round_start), prefill_lens=_ptr(self.prefill_lens),
             budgets=_ptr(self.budgets), seq_lens_host=C.cast(self._lens_host, C.c_void_p))
+
+    _recent: "dict[tuple, StepBatch]" = {}
+
+    @classmethod
+    def for_request(cls, device, total_tokens: int, block_ids, round_start: int | None = None,
+                    budget: int | None = None, prefill_len: int | None = None) -> "StepBatch":
+        """The batch of a single request, for callers that come back with the same request several
+        times in a row (the per-layer selection modes: one selection and one compaction per layer,
+        all with the same lengths and block ids): built once per set of values and reused.  The
+        device arrays of a batch are only ever read, so sharing one between launches is safe."""
+        ids = tuple(int(x) for x in block_ids)
+        key = (str(device), int(total_tokens), ids, round_start, budget, prefill_len)
+        hit = cls._recent.get(key)
+        if hit is None:
+            hit = cls(device, [int(total_tokens)], round_start=None if round_start is None else [int(round_start)],
+                      budgets=None if budget is None else [int(budget)], block_tables=[list(ids)],
+                      prefill_lens=None if prefill_len is None else [int(prefill_len)])
+            if len(cls._recent) >= 8:
+                cls._recent.pop(next(iter(cls._recent)))
+            cls._recent[key] = hit
+        return hit
 
     def refill(self, round_start, block_tables, prefill_lens=None) -> None:
         """New round starts, block tables and prefill lengths for the SAME sequence lengths and

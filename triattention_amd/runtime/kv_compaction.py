@@ -196,7 +196,7 @@ def _run_compaction(kv_caches, block_ids, block_size: int, keep_rows: torch.Tens
     if kv.block_size != block_size:
         raise ValueError(f"block_size={block_size} does not match the cache's {kv.block_size}")
     k = int(keep_rows.shape[1])
-    batch = ops.StepBatch(kv.device, [total_tokens], budgets=[k], block_tables=[_block_ids_list(block_ids)])
+    batch = ops.StepBatch.for_request(kv.device, total_tokens, _block_ids_list(block_ids), budget=k)
     ops.compact(kv, batch, keep_rows.to(device=kv.device, dtype=torch.int32).contiguous(),
                 shared=shared, full_permutation=full_permutation)
     if expected is not None:

@@ -186,10 +186,13 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         omega, offsets = st.vectors(kv.device)
         sc = ops.ScoreConfig(st.folded(layer_ids, score_heads, kv.device), omega, offsets,
                              config.sparse_score_aggregation)
-        tables = None if block_ids is None else [
-            block_ids.flatten().tolist() if isinstance(block_ids, torch.Tensor) else [int(x) for x in block_ids]]
-        batch = ops.StepBatch(kv.device, [total_tokens], round_start=[round_start], budgets=[k],
-                              block_tables=tables, prefill_lens=[prefill_len])
+        if block_ids is None:
+            batch = ops.StepBatch(kv.device, [total_tokens], round_start=[round_start], budgets=[k],
+                                  prefill_lens=[prefill_len])
+        else:
+            ids = block_ids.flatten().tolist() if isinstance(block_ids, torch.Tensor) else block_ids
+            batch = ops.StepBatch.for_request(kv.device, total_tokens, ids, round_start=int(round_start), budget=int(k),
+                                              prefill_len=int(prefill_len))
         sel = ops.SelectConfig(normalize=config.sparse_normalize_scores, window_size=config.window_size,
                                protect_prefill=bool(protect_prefill and prefill_len > 0),
                                group_reduce=group_reduce, layer_reduce=layer_reduce, shared=shared,
@@ -230,8 +233,8 @@ def build_triattention_selector(config: TriAttentionRuntimeConfig, base_runner: 
         score_heads, group_reduce = _head_layout(kv.num_kv_heads)
         per_head = mode in {"per_head", "per_layer_per_head"}
         # One call per layer and request: on the resident kernel every one of them would end in a read
-        # of the status word (one request of 2176 tokens x 36 layers: 13.2 ms through the hook against
-        # 11.5 ms on the two-pass kernels, whose launches queue up behind each other unwatched).
+        # of the status word, where the two-pass launches queue up behind each other unwatched (one
+        # request of 2176 tokens x 36 layers through the hook: 15 % slower on the resident kernel).
         keep = _score_and_select(kv, (int(layer_idx),), tables, total_tokens, prefill_len, protect_prefill,
                                  round_start, k, None, group_reduce, score_heads, shared=not per_head,
                                  allow_resident=False)
