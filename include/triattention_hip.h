@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 5
+#define TRI_ABI_VERSION 6
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -235,6 +235,28 @@ int tri_select_paged(const tri_kv_layout* kv, const tri_batch* batch, const tri_
  * Host-only.  No counterpart in the reference (it has a single path). */
 int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
                     const tri_select_params* sel);
+
+/* How tri_select_paged / tri_compress_step would cut these arguments into workgroups: the path
+ * as tri_select_path reports it and, for the resident kernels, the tile length, the tiles of the
+ * longest sequence, the groups the layers are cut into (1: every workgroup runs the whole model)
+ * and the number of launches (0: as many as the device-side packing of the ragged lengths needs,
+ * at most ceil(num_seqs / sequences per launch)).  assume_resident_workgroups > 0 answers for a
+ * device that holds that many resident workgroups at once (a dry run that touches no device:
+ * capacity planning, tests of the planner on a host without a GPU; 256 is an MI355X with 8-wave
+ * workgroups); 0 answers for the current device.  Host-only.  No counterpart in the reference. */
+typedef struct tri_plan_info {
+  int32_t path;                 /* 0 two-pass, 1 resident on the vector unit, 2 resident on the matrix cores */
+  int32_t tile_tokens;          /* tokens a workgroup scores per layer (0 on the two-pass path) */
+  int32_t tiles_per_seq;        /* by max_seq_len */
+  int32_t layer_groups;
+  int32_t layers_per_group;
+  int32_t launches;
+  int32_t waves_per_workgroup;
+  int32_t resident_workgroups;  /* capacity the plan was made for, in workgroups of eight waves (two of four waves take the place of one) */
+  int64_t workspace_bytes;      /* what tri_workspace_bytes returns for that plan */
+} tri_plan_info;
+int tri_describe_plan(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                      const tri_select_params* sel, int32_t assume_resident_workgroups, tri_plan_info* out);
 
 /* Top-k of arbitrary fp32 rows (core/compressor.py:388-409): keep[r][0..k_r) =
  * ascending indices of the k_r largest of scores[r][0..len_r). */

@@ -1000,6 +1000,13 @@ def test_resident_path_is_taken_unless_multi_layer_workgroups_would_underfill_th
         sc = ops.ScoreConfig(ops.fold_stats(qc, qa, torch.ones_like(qa)), synth.rope_inv_freq(w, DEV),
                              synth.geometric_offsets(device=DEV))
         assert ops.select_path(kv, batch, sc, sel) == want, (layers, split, seq_lens)
+        info = ops.describe_plan(kv, batch, sc, sel)
+        assert info["path"] == want
+        if want != "two_pass":
+            # the dry run for a device of this one's size gives this device's plan, and a launch fits the device
+            assert ops.describe_plan(kv, batch, sc, sel, assume_resident_workgroups=info["resident_workgroups"]) == info
+            assert info["launches"] == 1 and info["layer_groups"] * info["layers_per_group"] >= layers
+            assert len(seq_lens) * info["layer_groups"] * info["tiles_per_seq"] <= info["resident_workgroups"]
 
 
 def _resident_batch(seed_index):

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.tri_abi_version() == _lib.ABI_VERSION == 5
+    assert lib.tri_abi_version() == _lib.ABI_VERSION == 6
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
@@ -800,3 +800,59 @@ def test_a_library_built_from_other_sources_is_rebuilt(tmp_path, monkeypatch):
     assert "is missing" in tri_build.stale()
     tri_build.ensure_built()
     assert calls == ["build", "build"]
+
+
+# ---------------------------------------------------------------- the planner, on a pretended device
+def _describe(layers, q_heads, kv_heads, head_dim, lens, assume=256, kv_dtype=0, host_lens=True, **select):
+    import ctypes as C
+    lib = _lib.load()
+    kv = _lib.KvLayout(num_layers=layers, num_kv_heads=kv_heads, head_dim=head_dim, block_size=16, kv_dtype=kv_dtype,
+                       stride_block=16 * kv_heads * head_dim, stride_token=kv_heads * head_dim, stride_head=head_dim,
+                       k_layers=8, v_layers=8, k_scale_layers=8 if kv_dtype == 2 else None)
+    arr = (C.c_int32 * len(lens))(*lens)
+    batch = _lib.Batch(num_seqs=len(lens), max_seq_len=max(lens), max_budget=64, block_table_pitch=4096, block_table=8,
+                       seq_lens=8, round_start=8, budgets=8, seq_lens_host=C.cast(arr, C.c_void_p) if host_lens else None)
+    sp = _lib.ScoreParams(num_score_heads=q_heads, num_offsets=17, folded=16, omega=8, offsets=8)
+    kw = dict(normalize=1, window_size=128, group_reduce=1)
+    kw.update(select)
+    sel = _lib.SelectParams(**kw)
+    info = _lib.PlanInfo()
+    rc = lib.tri_describe_plan(C.byref(kv), C.byref(batch), C.byref(sp), C.byref(sel), assume, C.byref(info))
+    assert rc == 0, lib.tri_last_error()
+    assert info.workspace_bytes > 0
+    return (info.path, info.tile_tokens, info.tiles_per_seq, info.layer_groups, info.layers_per_group, info.launches)
+
+
+def test_planner_cuts_the_benchmarked_shapes_as_documented():
+    """``tri_describe_plan`` for a device that holds 256 resident workgroups (an MI355X), without one:
+    (path, tile tokens, tiles of the longest sequence, layer groups, layers per group, launches)."""
+    from triattention_amd import synth
+    q8b = (36, 32, 8, 128)
+    assert _describe(*q8b, [16384] * 16) == (2, 1024, 16, 1, 36, 1)          # C1: one workgroup per CU, whole model
+    assert _describe(*q8b, [8192] * 16) == (2, 512, 16, 1, 36, 1)            # a full chip is not cut by layers
+    assert _describe(*q8b, [2176] * 16) == (2, 576, 4, 4, 9, 1)              # steady state: 16 x 4 groups x 4 tiles
+    assert _describe(*q8b, [2176]) == (2, 320, 7, 36, 1, 1)                  # one request: a workgroup per layer and tile
+    assert _describe(*q8b, [2176] * 3) == (2, 320, 7, 12, 3, 1)
+    assert _describe(1, 32, 8, 128, [4096]) == (2, 128, 32, 1, 1, 1)         # C0: one layer, an eighth of the chip
+    assert _describe(*q8b, [128] * 130)[0] == 0                              # 130 whole-model workgroups, no room for two groups
+    assert _describe(64, 64, 8, 128, [32768] * 8) == (2, 512, 64, 1, 64, 2)  # C2: two launches of four sequences
+    assert _describe(64, 64, 8, 128, [32768] * 8, host_lens=False)[5] == 0   # lengths unknown to the host: packed on the device
+    assert _describe(32, 32, 8, 128, [16384] * 16, kv_dtype=2) == (2, 1024, 16, 1, 32, 1)          # C4
+    assert _describe(28, 28, 4, 128, [2176] * 16) == (2, 448, 5, 6, 5, 1)    # four-wave workgroups, two per CU
+    assert _describe(36, 64, 8, 64, [16384] * 16) == (2, 512, 32, 1, 36, 2)  # GPT-OSS head shape
+    c3 = synth.config(3)
+    path, tile, tiles, groups, _, launches = _describe(*q8b, list(c3.seq_lens))
+    assert (path, tile, groups, launches) == (2, 640, 1, 7)      # 1777 tiles of 640 tokens: seven launches, 98 % full
+    assert (launches - 1) * 256 < sum(-(-t // tile) for t in c3.seq_lens) <= launches * 256
+    # what keeps a call off the resident kernels
+    assert _describe(*q8b, [16384] * 16, layer_reduce=-1)[0] == 0            # a keep set per layer, several layers
+    assert _describe(1, 32, 8, 128, [4096], layer_reduce=-1)[0] == 2         # ... of one layer: the same thing as its mean
+    assert _describe(*q8b, [16384] * 16, shared=1)[0] == 0
+    assert _describe(*q8b, [16384] * 16, group_first=1)[0] == 0
+    assert _describe(*q8b, [16384] * 16, no_resident=1)[0] == 0
+    assert _describe(*q8b, [16384] * 16, assume=0)[0] in (0, 2)              # the current device, if there is one
+    # a smaller device: more launches, never more workgroups than it holds
+    path, tile, tiles, groups, _, launches = _describe(*q8b, [16384] * 16, assume=64)
+    assert path == 2 and groups == 1 and launches * 64 >= 16 * tiles
+    import ctypes as C
+    assert _lib.load().tri_describe_plan(None, None, None, None, 0, None) == _lib.TRI_ERR_INVALID_ARGUMENT

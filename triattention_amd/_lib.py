@@ -13,7 +13,7 @@ import os
 # TRIATTN_HIP_LIBRARY points at another build of the same ABI (e.g. an instrumented one).
 LIB_PATH = Path(os.environ.get("TRIATTN_HIP_LIBRARY") or Path(__file__).resolve().parent / "libtriattention_hip.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 STATIC_WORKSPACE_BYTES = 64 << 20
 TRI_OK = 0
 TRI_ERR_INVALID_ARGUMENT = -1
@@ -33,7 +33,7 @@ EXPORTS = (
     "tri_abi_version", "tri_last_error", "tri_source_digest", "tri_set_tuning", "tri_get_tuning", "tri_resident_gate_enter",
     "tri_resident_gate_leave", "tri_fold_stats", "tri_workspace_bytes", "tri_workspace_status_offset",
     "tri_score_paged",
-    "tri_select", "tri_select_paged", "tri_select_path", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
+    "tri_select", "tri_select_paged", "tri_select_path", "tri_describe_plan", "tri_topk_rows", "tri_compact_paged", "tri_compact_full_staging_bytes",
     "tri_compact_paged_full", "tri_compress_step", "tri_compress_step_static", "tri_qstats_workspace_bytes", "tri_qstats",
 )
 
@@ -54,6 +54,14 @@ class Batch(C.Structure):
         ("block_table_pitch", C.c_int32),
         ("block_table", C.c_void_p), ("seq_lens", C.c_void_p), ("round_start", C.c_void_p),
         ("prefill_lens", C.c_void_p), ("budgets", C.c_void_p), ("seq_lens_host", C.c_void_p),
+    ]
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [
+        ("path", C.c_int32), ("tile_tokens", C.c_int32), ("tiles_per_seq", C.c_int32), ("layer_groups", C.c_int32),
+        ("layers_per_group", C.c_int32), ("launches", C.c_int32), ("waves_per_workgroup", C.c_int32),
+        ("resident_workgroups", C.c_int32), ("workspace_bytes", C.c_int64),
     ]
 
 
@@ -113,6 +121,8 @@ def load() -> C.CDLL:
                                      C.POINTER(SelectParams), P, P, P, U64, P]
     lib.tri_select_path.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
                                     C.POINTER(SelectParams)]
+    lib.tri_describe_plan.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), C.POINTER(ScoreParams),
+                                      C.POINTER(SelectParams), I32, C.POINTER(PlanInfo)]
     lib.tri_topk_rows.argtypes = [P, I64, I32, P, P, I32, I32, P, I32, P]
     lib.tri_compact_paged.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch), P, I32, I32, P]
     lib.tri_compact_full_staging_bytes.argtypes = [C.POINTER(KvLayout), C.POINTER(Batch)]

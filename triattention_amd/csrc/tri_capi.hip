@@ -96,7 +96,7 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
   return TRI_OK;
 }
 
-tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp) {
+tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp, int assume_resident = 0) {
   // Resident kernels: two-byte and fp8 keys go to the matrix-core kernel where the shape has one,
   // and only launches that fill most of the chip take them.  TRI_TUNE_RESIDENT_KERNEL overrides
   // the choice: 1 / 2 take the matrix-core / vector-unit kernel whenever the shape has it (however
@@ -111,7 +111,8 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
                          kv->stride_token > 0 && kv->stride_token < (1 << 25);
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;
-  const int resident = f_off ? 0 : tri::fused_resident_workgroups();
+  // assume_resident > 0: a dry run for a device of that size (tri_describe_plan); no device is asked.
+  const int resident = f_off ? 0 : (assume_resident > 0 ? assume_resident : tri::fused_resident_workgroups());
   tri::FusedPlan fused{};
   // Small batches are cut by layers as well (TRI_TUNE_LAYER_SPLIT = 0 switches that off, 1 switches
   // it on where the kernel was forced, which otherwise keeps whole-model workgroups).
@@ -526,6 +527,37 @@ int tri_select_path(const tri_kv_layout* kv, const tri_batch* batch, const tri_s
   if (check_layout(kv, false) || check_batch(batch, false) || check_score(kv, sp) || check_select(sel)) return -1;
   const tri::Workspace w = plan(kv, batch, sp);
   return takes_resident(w, kv, sel) ? w.fused.eligible : 0;
+}
+
+int tri_describe_plan(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_params* sp,
+                      const tri_select_params* sel, int32_t assume_resident_workgroups, tri_plan_info* out) {
+  if (!out) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_describe_plan: out is NULL");
+  if (assume_resident_workgroups < 0)
+    return fail(TRI_ERR_INVALID_ARGUMENT, "assume_resident_workgroups %d", assume_resident_workgroups);
+  int rc = check_layout(kv, false);
+  if (!rc) rc = check_batch(batch, false);
+  if (!rc) rc = check_score(kv, sp);
+  if (!rc) rc = check_select(sel);
+  if (rc) return rc;
+  const tri::Workspace w = plan(kv, batch, sp, assume_resident_workgroups);
+  *out = tri_plan_info{};
+  out->workspace_bytes = w.total;
+  out->layer_groups = 1;
+  out->layers_per_group = kv->num_layers;
+  if (!takes_resident(w, kv, sel)) return TRI_OK;
+  const tri::FusedPlan& f = w.fused;
+  out->path = f.eligible;
+  out->tile_tokens = f.tile_tokens;
+  out->tiles_per_seq = f.tiles_per_seq;
+  out->resident_workgroups = (f.eligible == 2 && f.waves == 4) ? f.resident / 2 : f.resident;
+  out->waves_per_workgroup = f.eligible == 2 ? f.waves : 8;
+  if (f.eligible == 2 && f.layer_groups > 1) {
+    out->layer_groups = f.layer_groups;
+    out->layers_per_group = f.layers_per_group;
+  }
+  if (batch->num_seqs <= f.seqs_per_launch) out->launches = 1;
+  else out->launches = f.launches;      // > 0: the planner replayed the packing of the host's lengths
+  return TRI_OK;
 }
 
 int tri_topk_rows(const float* scores, int64_t row_pitch, int32_t num_rows, const int32_t* row_lens,

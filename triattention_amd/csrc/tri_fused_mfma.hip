@@ -1116,8 +1116,9 @@ FusedPlan plan_fused_mfma(int B, int Hkv, int D, int G, int block_size, bool pag
   if (host_lens && (int64_t)B * tiles * HC > resident) {
     // Several launches, and the lengths are known: a launch takes as long as its tiles are
     // long, however many of its workgroups have work, so the tile size that packs the
-    // sequences into the fewest tile-lengths wins (64 sequences of 2k-32k tokens: 1120 tiles of
-    // 1024 tokens are 4.4 launches' worth and take five; tiles of 896 fill five launches).
+    // sequences into the fewest tile-lengths wins (64 sequences of 2k-32k tokens, 1.12 M in all:
+    // 1124 tiles of 1024 tokens are 4.4 launches' worth and take five, 5 x 1024 tile-lengths;
+    // 1777 tiles of 640 fill seven launches to 98 %, 7 x 640).
     const int granule = (kv_dtype == TRI_KV_FP8_E4M3 || (D == 64 && G <= 4)) ? 128 : 64;
     int64_t best_cost = -1;
     for (int cand = tw; cand >= tw / 2 && cand >= 128; cand -= granule) {

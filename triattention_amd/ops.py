@@ -497,6 +497,19 @@ def select_path(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfi
     return {2: "resident_mfma", 1: "resident_valu"}.get(rc, "two_pass")
 
 
+def describe_plan(kv: PagedKV, batch: StepBatch, sc: ScoreConfig, sel: SelectConfig,
+                  assume_resident_workgroups: int = 0) -> dict:
+    """How select_paged / compress_step would cut these arguments into workgroups (``tri_describe_plan``):
+    path, tile length, tiles of the longest sequence, layer groups, launches, workspace bytes --
+    for the current device, or for one that holds ``assume_resident_workgroups`` at once."""
+    sp, ss, info = sc.struct(), sel.struct(), _lib.PlanInfo()
+    _lib.check(_lib.load().tri_describe_plan(C.byref(kv.struct), C.byref(batch.struct), C.byref(sp), C.byref(ss),
+                                             int(assume_resident_workgroups), C.byref(info)))
+    out = {name: int(getattr(info, name)) for name, _ in _lib.PlanInfo._fields_}
+    out["path"] = {2: "resident_mfma", 1: "resident_valu"}.get(out["path"], "two_pass")
+    return out
+
+
 def topk_rows(scores: torch.Tensor, k: int | Sequence[int], lens: Sequence[int] | None = None) -> torch.Tensor:
     """Ascending int32 indices of the k largest entries of every row of a 2-D fp32 tensor."""
     lib = _lib.load()
