@@ -350,6 +350,9 @@ class StepRun:
         self.fin_buf = torch.empty(rows, self.batch.max_seq_len, dtype=torch.float32, device=dev)
         self.path = "two_pass" if force_two_pass else ops.select_path(self.kv, self.batch, sc, sel)
         self.two_pass = self.path == "two_pass"
+        # How the library cuts this step into workgroups (tile length, layer groups, launches).
+        self.plan = None if force_two_pass else {k: v for k, v in ops.describe_plan(self.kv, self.batch, sc, sel).items()
+                                                 if k != "path"}
         self.raw_buf = None
         if self.two_pass:
             self.raw_buf = torch.empty(w.num_seqs, w.num_layers, self.batch.max_seq_len, w.num_q_heads,
@@ -481,7 +484,7 @@ def measure(run: "StepRun", warmup: int, steps: int) -> dict:
     gbs = algo["total"] / (ms * 1e-3) / 1e9
     return {
         "steps": steps, "ms_per_step": ms, "value": sum(w.seq_lens) / (ms * 1e-3), "achieved_gbs": gbs,
-        "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "path": run.path,
+        "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "path": run.path, "plan": run.plan,
         "stage_ms": {"score": mean(score_ms), "select" if run.two_pass else "topk": mean(select_ms),
                      "compact": mean(compact_ms)},
         "staged_ms_per_step": mean([e[0].elapsed_time(e[3]) for e in sev]),
@@ -724,6 +727,7 @@ def main() -> int:
         "timed_region_wall_s": m["timed_region_wall_s"],
         "setup_s": setup_s,
         "path": path,
+        "plan": m["plan"],
         "roofline": {"kernel": {"two_pass": two_pass_kernel, "resident_valu": "fused_select_kernel",
                                 "resident_mfma": "fused_mfma_kernel"}[path], "bound": "hbm",
                      "achieved": score_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": score_gbs / HBM_PEAK_GBS,
