@@ -688,14 +688,16 @@ def test_header_is_plain_c_and_a_c_program_links_the_library(tmp_path):
 #include <string.h>
 #include "triattention_hip.h"
 int main(void) {
-  tri_kv_layout kv; tri_batch b; tri_score_params sp; tri_select_params sel;
+  tri_kv_layout kv; tri_batch b; tri_score_params sp; tri_select_params sel; tri_plan_info info;
   memset(&kv, 0, sizeof kv); memset(&b, 0, sizeof b); memset(&sp, 0, sizeof sp); memset(&sel, 0, sizeof sel);
   printf("abi %d %d\n", tri_abi_version(), TRI_ABI_VERSION);
-  printf("sizes %zu %zu %zu %zu\n", sizeof kv, sizeof b, sizeof sp, sizeof sel);
+  printf("sizes %zu %zu %zu %zu %zu\n", sizeof kv, sizeof b, sizeof sp, sizeof sel, sizeof info);
   printf("bytes %llu\n", (unsigned long long)tri_workspace_bytes(&kv, &b, &sp));
   int rc = tri_compress_step(&kv, &b, &sp, &sel, NULL, NULL, 0, NULL);
   printf("rc %d msg %s\n", rc, tri_last_error());
   rc = tri_compress_step_static(NULL, &b, &sp, &sel, NULL, NULL, NULL);
+  printf("rc %d msg %s\n", rc, tri_last_error());
+  rc = tri_describe_plan(&kv, &b, &sp, &sel, 256, &info);
   printf("rc %d msg %s\n", rc, tri_last_error());
   return 0;
 }
@@ -712,10 +714,12 @@ int main(void) {
     lines = out.stdout.splitlines()
     assert lines[0] == f"abi {_lib.ABI_VERSION} {_lib.ABI_VERSION}"
     sizes = [int(x) for x in lines[1].split()[1:]]
-    assert sizes == [C.sizeof(_lib.KvLayout), C.sizeof(_lib.Batch), C.sizeof(_lib.ScoreParams), C.sizeof(_lib.SelectParams)]
+    assert sizes == [C.sizeof(_lib.KvLayout), C.sizeof(_lib.Batch), C.sizeof(_lib.ScoreParams), C.sizeof(_lib.SelectParams),
+                     C.sizeof(_lib.PlanInfo)]
     assert lines[2] == "bytes 0"
     assert lines[3].startswith("rc -") and "bad layer/head count" in lines[3]
     assert lines[4].startswith("rc -") and "kv layout is NULL" in lines[4]
+    assert lines[5].startswith("rc -") and "bad layer/head count" in lines[5]
 
 
 def test_product_raises_when_the_library_is_missing(tmp_path, monkeypatch):
