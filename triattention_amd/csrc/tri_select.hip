@@ -190,8 +190,9 @@ __device__ __forceinline__ float zscore(float x, float mean, float sd) {
 }
 
 // One thread per (token, output row).  Grid: (token tiles, layers or 1, B).
-// VEC4: groups of four query heads, raw scores head-contiguous and 16-byte aligned.
-template <bool VEC4>
+// NV > 0: groups of 4 * NV query heads (4 or 8), raw scores head-contiguous and 16-byte aligned, read as
+// NV 16-byte loads per layer; NV = 0: any layout, one score at a time.
+template <int NV>
 __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
   extern __shared__ float tile[];  // [rows_per_seq][tokens_per_wg]
   const int b = blockIdx.z;
@@ -212,67 +213,74 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     const int h_begin = a.shared ? 0 : r;
     const int h_end = a.shared ? a.Hkv : r + 1;
     float acc = 0.f;
-    if (VEC4 && !a.shared) {
-      // Default shape: one KV head per thread, four query heads in one 16-byte load;
-      // four layers in flight per thread.
-      const float* raw0 = a.raw + (int64_t)b * a.L * a.raw_stride_layer + (int64_t)n * a.raw_stride_token + r * 4;
+    if (NV > 0 && !a.shared) {
+      // Default shapes: one KV head per thread, its query heads in NV 16-byte loads; several layers in
+      // flight per thread.
+      constexpr int NVV = NV > 0 ? NV : 1;
+      constexpr int GQ = 4 * NVV;                  // query heads per KV head
+      constexpr int U = NVV == 1 ? 4 : 2;          // layers in flight
+      const float* raw0 = a.raw + (int64_t)b * a.L * a.raw_stride_layer + (int64_t)n * a.raw_stride_token + r * GQ;
       // Reduce-first order (group_first): the statistics are those of the KV head's reduced score and
-      // sit in entry r of the layer's table; they arrive in m01.x / m01.y (m23 unused).
-      const float* ms0 = a.mustd + ((int64_t)b * a.L * a.A + (a.group_first ? r : r * 4)) * 2;
-      auto layer_value = [&](const float4& x, const float4& m01, const float4& m23) {
-        // mustd is [head][mean, std]: m01 = (mean0, std0, mean1, std1), m23 likewise.
+      // sit in entry r of the layer's table; they arrive in m[0].x / m[0].y (the rest unused).
+      const float* ms0 = a.mustd + ((int64_t)b * a.L * a.A + (a.group_first ? r : r * GQ)) * 2;
+      struct LayerIn { float4 x[NVV]; float4 m[2 * NVV]; };
+      auto load_layer = [&](int l, LayerIn& in) {
+        const float* rl = raw0 + (int64_t)l * a.raw_stride_layer;
+        const float* ms = ms0 + (int64_t)l * a.A * 2;
+#pragma unroll
+        for (int i = 0; i < NVV; ++i) in.x[i] = *reinterpret_cast<const float4*>(rl + 4 * i);
+        if (a.group_first) {
+          const float2 m = *reinterpret_cast<const float2*>(ms);
+#pragma unroll
+          for (int i = 0; i < 2 * NVV; ++i) in.m[i] = float4{m.x, m.y, 0.f, 0.f};
+        } else {
+          // mustd is [head][mean, std]: m[2 i] = (mean, std) of query heads 4 i and 4 i + 1, m[2 i + 1] of the next two.
+#pragma unroll
+          for (int i = 0; i < 2 * NVV; ++i) in.m[i] = *reinterpret_cast<const float4*>(ms + 4 * i);
+        }
+      };
+      auto layer_value = [&](const LayerIn& in) {
+        float xs[GQ];
+#pragma unroll
+        for (int i = 0; i < NVV; ++i) { xs[4 * i] = in.x[i].x; xs[4 * i + 1] = in.x[i].y; xs[4 * i + 2] = in.x[i].z; xs[4 * i + 3] = in.x[i].w; }
         float v;
         if (a.group_first) {
-          const float m = (a.group_reduce == TRI_REDUCE_MAX)
-                              ? fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))
-                              : __fdiv_rn(__fadd_rn(__fadd_rn(__fadd_rn(x.x, x.y), x.z), x.w), 4.f);
-          v = zscore(m, m01.x, m01.y);
-        } else if (a.group_reduce == TRI_REDUCE_MAX) {
-          v = fmaxf(fmaxf(zscore(x.x, m01.x, m01.y), zscore(x.y, m01.z, m01.w)),
-                    fmaxf(zscore(x.z, m23.x, m23.y), zscore(x.w, m23.z, m23.w)));
+          // (the order of the scalar path below: query heads one after the other)
+          float m = xs[0];
+#pragma unroll
+          for (int q = 1; q < GQ; ++q) m = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(m, xs[q]) : __fadd_rn(m, xs[q]);
+          if (a.group_reduce != TRI_REDUCE_MAX) m = __fdiv_rn(m, (float)GQ);
+          v = zscore(m, in.m[0].x, in.m[0].y);
         } else {
-          v = __fadd_rn(__fadd_rn(__fadd_rn(zscore(x.x, m01.x, m01.y), zscore(x.y, m01.z, m01.w)),
-                                  zscore(x.z, m23.x, m23.y)), zscore(x.w, m23.z, m23.w));
-          v = __fdiv_rn(v, 4.f);
+          float z[GQ];
+#pragma unroll
+          for (int i = 0; i < 2 * NVV; ++i) {
+            z[2 * i] = zscore(xs[2 * i], in.m[i].x, in.m[i].y);
+            z[2 * i + 1] = zscore(xs[2 * i + 1], in.m[i].z, in.m[i].w);
+          }
+          v = z[0];
+#pragma unroll
+          for (int q = 1; q < GQ; ++q) v = (a.group_reduce == TRI_REDUCE_MAX) ? fmaxf(v, z[q]) : __fadd_rn(v, z[q]);
+          if (a.group_reduce != TRI_REDUCE_MAX) v = __fdiv_rn(v, (float)GQ);
         }
         return guard ? INFINITY : v;
       };
       int l = l_begin;
-      for (; l + 4 <= l_end; l += 4) {
-        float4 x[4], m01[4], m23[4];
+      for (; l + U <= l_end; l += U) {
+        LayerIn in[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          x[u] = *reinterpret_cast<const float4*>(raw0 + (int64_t)(l + u) * a.raw_stride_layer);
-          const float* ms = ms0 + (int64_t)(l + u) * a.A * 2;
-          if (a.group_first) {
-            const float2 m = *reinterpret_cast<const float2*>(ms);
-            m01[u] = float4{m.x, m.y, 0.f, 0.f};
-            m23[u] = m01[u];
-          } else {
-            m01[u] = *reinterpret_cast<const float4*>(ms);
-            m23[u] = *reinterpret_cast<const float4*>(ms + 4);
-          }
-        }
+        for (int u = 0; u < U; ++u) load_layer(l + u, in[u]);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const float v = layer_value(x[u], m01[u], m23[u]);
+        for (int u = 0; u < U; ++u) {
+          const float v = layer_value(in[u]);
           if (l + u == l_begin) acc = v;
           else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
         }
       }
       for (; l < l_end; ++l) {
-        const float4 x = *reinterpret_cast<const float4*>(raw0 + (int64_t)l * a.raw_stride_layer);
-        const float* ms = ms0 + (int64_t)l * a.A * 2;
-        float4 m01, m23;
-        if (a.group_first) {
-          const float2 m = *reinterpret_cast<const float2*>(ms);
-          m01 = float4{m.x, m.y, 0.f, 0.f};
-          m23 = m01;
-        } else {
-          m01 = *reinterpret_cast<const float4*>(ms);
-          m23 = *reinterpret_cast<const float4*>(ms + 4);
-        }
-        const float v = layer_value(x, m01, m23);
+        LayerIn in;
+        load_layer(l, in);
+        const float v = layer_value(in);
         if (l == l_begin) acc = v;
         else acc = (a.layer_reduce == TRI_REDUCE_MAX) ? fmaxf(acc, v) : __fadd_rn(acc, v);
       }
@@ -683,13 +691,15 @@ hipError_t launch_select(const SelectLaunch& a, hipStream_t s) {
   const bool per_layer = a.layer_reduce < 0;
   dim3 grid(ceil_div(a.Tmax, c.tokens_per_wg), per_layer ? a.L : 1, a.B);
   const size_t smem = (size_t)c.rows_per_seq * c.tokens_per_wg * sizeof(float);
-  const bool vec4 = a.G == 4 && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
-                    a.raw_stride_layer % 4 == 0 && (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 &&
-                    (reinterpret_cast<uintptr_t>(a.mustd) % 16) == 0;
-  if (vec4)
-    hipLaunchKernelGGL(combine_kernel<true>, grid, dim3(256), smem, s, c);
+  const bool vec = (a.G == 4 || a.G == 8) && a.raw_stride_head == 1 && a.raw_stride_token % 4 == 0 &&
+                   a.raw_stride_layer % 4 == 0 && (reinterpret_cast<uintptr_t>(a.raw) % 16) == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.mustd) % 16) == 0;
+  if (vec && a.G == 4)
+    hipLaunchKernelGGL(combine_kernel<1>, grid, dim3(256), smem, s, c);
+  else if (vec)
+    hipLaunchKernelGGL(combine_kernel<2>, grid, dim3(256), smem, s, c);
   else
-    hipLaunchKernelGGL(combine_kernel<false>, grid, dim3(256), smem, s, c);
+    hipLaunchKernelGGL(combine_kernel<0>, grid, dim3(256), smem, s, c);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
 
