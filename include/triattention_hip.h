@@ -219,9 +219,10 @@ int tri_select(const tri_kv_layout* kv, const tri_batch* batch, const tri_score_
  * the caller: the device side of _select_keep_indices_for_group_per_head's paged branch
  * (runtime/selector_hf.py:813-1033) and of the per-layer selector (:473-677).  When the
  * shape allows (head_dim 128, or 64 / 256 with two-byte keys; at most eight query heads
- * per KV head; mean aggregation over offsets; power-of-two block size; layer_reduce >= 0;
- * not shared; a batch that fills most of the GPU and whose sequences fit its LDS in
- * tiles) one resident kernel keeps each layer's raw scores in LDS
+ * per KV head; mean aggregation over offsets; power-of-two block size; layer_reduce >= 0,
+ * or a single layer, where a keep set per layer is the same thing; not shared; workgroups
+ * that run one layer each, or a batch that fills most of the GPU; sequences that fit its
+ * LDS in tiles) one resident kernel keeps each layer's raw scores in LDS
  * and they never reach memory; otherwise the two calls above run back to back on the
  * workspace.  Outputs as tri_select; keep may be NULL when only final_scores is wanted
  * (tri_topk_rows then turns them into keep rows). */
