@@ -102,7 +102,7 @@ typedef struct tri_score_params {
 typedef struct tri_select_params {
   int32_t normalize;            /* 0: raw scores; 1: sparse_normalize_scores (streaming unbiased std, std < 1e-8 -> 1,
                                    runtime/selector_hf.py:902-909); 2: the research path's z-score (population std
-                                   clamped at 1e-6, methods/triattention.py:255-258; two-pass kernels only) */
+                                   clamped at 1e-6, methods/triattention.py:255-258) */
   int32_t window_size;          /* recent tokens forced to +inf (runtime/selector_hf.py:121-130) */
   int32_t protect_prefill;      /* tokens < prefill_len forced to +inf */
   int32_t group_reduce;         /* tri_reduce over the query heads of a KV head (runtime/selector_hf.py:277-297) */
@@ -113,7 +113,7 @@ typedef struct tri_select_params {
                                    (layer, KV head) with torch mean / unbiased std (SGLang backend,
                                    sglang/scheduler_hooks.py:655-690, core/utils.py:466-480) */
   int32_t no_resident;          /* 1: never take a resident kernel for this call, whatever the shape and the
-                                   TRIATTN_RESIDENT_KERNEL override say (a caller repeating a step whose resident
+                                   TRI_TUNE_RESIDENT_KERNEL setting say (a caller repeating a step whose resident
                                    launch raised the status word).  No counterpart in the reference. */
 } tri_select_params;
 
