@@ -186,7 +186,7 @@ uint64_t tri_workspace_bytes(const tri_kv_layout* kv, const tri_batch* batch,
  * (no magnitude of 2^-9 among those looked at) that the pieces would be subnormals (2)
  * (results are then invalid; the compaction
  * inside tri_compress_step sees the word and moves nothing, so the cache is intact and
- * the caller can repeat the step with TRIATTN_RESIDENT_KERNEL=off).  The caller may read
+ * the caller can repeat the step with tri_select_params.no_resident = 1).  The caller may read
  * it after synchronising the stream.  Host-only; no counterpart in the reference. */
 uint64_t tri_workspace_status_offset(const tri_kv_layout* kv, const tri_batch* batch,
                                      const tri_score_params* sp);
