@@ -297,9 +297,10 @@ int tri_compress_step(const tri_kv_layout* kv, const tri_batch* batch, const tri
  * TRI_STATIC_WORKSPACE_BYTES per GPU from the moment the library is loaded until the process
  * ends; the call allocates nothing, frees nothing, creates no stream or event, and always takes
  * the score-then-select kernels (never a resident kernel; for fp8 caches the scales follow the
- * rows on `stream`).  A step whose scratch (tri_workspace_bytes) exceeds the array is rejected
- * with TRI_ERR_WORKSPACE: Qwen3-8B shapes (36 layers) fit up to 4 sequences of budget + 128 = 2176
- * tokens, or one sequence of 11400.  Every call on a GPU uses that GPU's one array, which keeps the
+ * rows on `stream`).  A step whose scratch for those kernels exceeds the array is rejected
+ * with TRI_ERR_WORKSPACE (tri_workspace_bytes is an upper bound of it: on a device with resident
+ * kernels it also covers their regions, which this call does not use): Qwen3-8B shapes (36 layers)
+ * fit up to 4 sequences of budget + 128 = 2176 tokens, or one sequence of 11400.  Every call on a GPU uses that GPU's one array, which keeps the
  * previous call's contents (nothing in it needs to start at zero except the status word, which
  * the call clears): calls that overlap in time on one GPU, from any streams or threads, race.
  * Results are those of tri_compress_step with no_resident = 1.  status_out (may be NULL)

@@ -7,7 +7,7 @@ import ctypes as C
 import pytest
 import torch
 
-from helpers import build_inputs, device_objects
+from helpers import build_inputs, device_objects, tune
 from triattention_amd import _lib, ops, synth
 
 pytestmark = pytest.mark.gpu
@@ -86,6 +86,30 @@ def test_static_scratch_rejects_steps_beyond_its_array():
     rc = lib.tri_compress_step_static(C.byref(kv.struct), C.byref(huge.struct), C.byref(sp), C.byref(ss),
                                       keep.data_ptr(), None, None)
     assert rc == _lib.TRI_ERR_WORKSPACE and b"static array" in lib.tri_last_error()
+
+
+def test_static_scratch_limits_are_the_documented_ones():
+    """Qwen3-8B shapes: four requests of 2176 tokens or one of 11400 fit the array, five or 11500 do not
+    (the scratch is sized for the score-then-select kernels the call runs, not for a resident plan).
+    The refusals come from the host-side check; the accepted shapes are not launched here (the
+    steady-state test above runs one)."""
+    w = synth.Workload("static_limits", 36, 32, 8, 128, (16,), 8, index=36)
+    inp = build_inputs(w)
+    caches, kv, batch, sc = device_objects(w, inp, DEV)
+    sp, ss = sc.struct(), ops.SelectConfig(window_size=128).struct()
+    lib = _lib.load()
+    keep = torch.empty(5 * w.num_kv_heads, 2048, dtype=torch.int32, device=DEV)
+    for lens, fits in (((2176,) * 5, False), ((11500,), False)):
+        claim = ops.StepBatch(DEV, list(lens), budgets=2048, block_tables=[list(range(800))] * len(lens))
+        rc = lib.tri_compress_step_static(C.byref(kv.struct), C.byref(claim.struct), C.byref(sp), C.byref(ss),
+                                          keep.data_ptr(), None, None)
+        assert rc == _lib.TRI_ERR_WORKSPACE and b"static array" in lib.tri_last_error(), lens
+    # the accepted side of the limit, through the planner's own answer for a device without resident kernels
+    tune(resident_kernel="off")
+    for lens in ((2176,) * 4, (11400,)):
+        claim = ops.StepBatch(DEV, list(lens), budgets=2048, block_tables=[list(range(800))] * len(lens))
+        need = int(lib.tri_workspace_bytes(C.byref(kv.struct), C.byref(claim.struct), C.byref(sp)))
+        assert 0 < need <= _lib.STATIC_WORKSPACE_BYTES, (lens, need)
 
 
 def _free_device_bytes() -> int:

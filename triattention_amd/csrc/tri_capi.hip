@@ -96,7 +96,8 @@ int check_score(const tri_kv_layout* kv, const tri_score_params* sp) {
   return TRI_OK;
 }
 
-tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp, int assume_resident = 0) {
+tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score_params* sp, int assume_resident = 0,
+                    bool allow_resident = true) {
   // Resident kernels: two-byte and fp8 keys go to the matrix-core kernel where the shape has one,
   // and only launches that fill most of the chip take them.  TRI_TUNE_RESIDENT_KERNEL overrides
   // the choice: 1 / 2 take the matrix-core / vector-unit kernel whenever the shape has it (however
@@ -112,7 +113,8 @@ tri::Workspace plan(const tri_kv_layout* kv, const tri_batch* b, const tri_score
   const int G = sp->num_score_heads / kv->num_kv_heads;
   const bool paged = b->block_table != nullptr;
   // assume_resident > 0: a dry run for a device of that size (tri_describe_plan); no device is asked.
-  const int resident = f_off ? 0 : (assume_resident > 0 ? assume_resident : tri::fused_resident_workgroups());
+  const int resident = (f_off || !allow_resident) ? 0
+                       : (assume_resident > 0 ? assume_resident : tri::fused_resident_workgroups());
   tri::FusedPlan fused{};
   // Small batches are cut by layers as well (TRI_TUNE_LAYER_SPLIT = 0 switches that off, 1 switches
   // it on where the kernel was forced, which otherwise keeps whole-model workgroups).
@@ -644,7 +646,9 @@ int tri_compress_step_static(const tri_kv_layout* kv, const tri_batch* batch, co
   if (!batch->round_start) return fail(TRI_ERR_INVALID_ARGUMENT, "round_start is NULL");
   if (!batch->block_table) return fail(TRI_ERR_INVALID_ARGUMENT, "tri_compress_step_static needs a block table");
   if (!keep) return fail(TRI_ERR_INVALID_ARGUMENT, "keep is NULL");
-  const tri::Workspace w = plan(kv, batch, sp);
+  // Always the score-then-select kernels, so the scratch is sized for them alone (a resident plan
+  // would add its coefficient slabs and exchange words; the status word sits at the same offset).
+  const tri::Workspace w = plan(kv, batch, sp, 0, false);
   if ((uint64_t)w.total > (uint64_t)TRI_STATIC_WORKSPACE_BYTES)
     return fail(TRI_ERR_WORKSPACE, "this step needs %lld bytes of scratch, the library's static array holds %llu; "
                 "use tri_compress_step with a workspace of the caller's", (long long)w.total,
